@@ -1,0 +1,77 @@
+// extern "C" boundary of libgmc_hip.so (declarations and contracts: include/gmc_hip.h).
+// Validates shapes on the host before any launch, so that a kernel never sees operands its grid does not fit.
+#include "gmc_common.h"
+
+namespace gmc {
+int dense_forward(const void* mixture, const void* xes, void* out, const gmc_shape& s, hipStream_t stream);
+size_t dense_backward_workspace_bytes(const gmc_shape& s);
+int dense_backward(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                   void* workspace, const gmc_shape& s, bool need_gm, bool need_gx, hipStream_t stream);
+
+int check_shape(const gmc_shape* s) {
+    if (!s) return GMC_E_NULL;
+    if (s->D != 2 && s->D != 3) return GMC_E_DIMS;
+    if (s->dtype != GMC_F32 && s->dtype != GMC_F64) return GMC_E_DTYPE;
+    if (s->B < 0 || s->L < 0 || s->M < 0 || s->N < 0) return GMC_E_SHAPE;
+    if (s->Bx != 1 && s->Bx != s->B) return GMC_E_SHAPE;
+    if (s->Lx != 1 && s->Lx != s->L) return GMC_E_SHAPE;
+    // per-(b,l) index arithmetic inside the kernels is 32-bit
+    if (size_t(s->M) * 13 > 0x7fffffffull || size_t(s->N) * 3 > 0x7fffffffull) return GMC_E_SHAPE;
+    if (size_t(s->B) * s->L > 0x7fffffffull / 64) return GMC_E_SHAPE;
+    return GMC_OK;
+}
+}  // namespace gmc
+
+extern "C" {
+
+int gmc_abi_version(void) { return 1; }
+
+const char* gmc_error_string(int code) {
+    switch (code) {
+        case GMC_OK: return "ok";
+        case GMC_E_DIMS: return "mixture must have 7 or 13 elements in the last dimension (D must be 2 or 3)";
+        case GMC_E_DTYPE: return "unsupported dtype (float32 and float64 only)";
+        case GMC_E_SHAPE: return "invalid shape (negative size, xes batch/layer dimension not 1 or equal to the mixture's, or too large)";
+        case GMC_E_NULL: return "null pointer argument";
+        case GMC_E_WORKSPACE: return "workspace too small";
+        case GMC_E_LAUNCH: return "HIP launch failed";
+        case GMC_E_CONFIG: return "invalid BVH configuration";
+        default: return "unknown error";
+    }
+}
+
+int gmc_eval_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream) {
+    const int rc = gmc::check_shape(shape);
+    if (rc != GMC_OK) return rc;
+    const size_t n_out = size_t(shape->B) * shape->L * shape->N;
+    if (n_out == 0) return GMC_OK;
+    if (!out || !xes || (!mixture && shape->M > 0)) return GMC_E_NULL;
+    return gmc::dense_forward(mixture, xes, out, *shape, (hipStream_t)stream);
+}
+
+size_t gmc_eval_bwd_workspace_bytes(const gmc_shape* shape) {
+    if (gmc::check_shape(shape) != GMC_OK) return 0;
+    return gmc::dense_backward_workspace_bytes(*shape);
+}
+
+int gmc_eval_bwd(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                 void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
+                 int need_grad_xes, void* stream) {
+    const int rc = gmc::check_shape(shape);
+    if (rc != GMC_OK) return rc;
+    const bool gm = need_grad_mixture != 0, gx = need_grad_xes != 0;
+    if (!gm && !gx) return GMC_OK;
+    const size_t n_g = size_t(shape->B) * shape->L * shape->M;
+    const size_t n_x = size_t(shape->Bx) * shape->Lx * shape->N;
+    if (gm && n_g > 0 && !grad_mixture) return GMC_E_NULL;
+    if (gx && n_x > 0 && !grad_xes) return GMC_E_NULL;
+    if (n_g > 0 && n_x > 0 && (!grad_out || !mixture || !xes)) return GMC_E_NULL;
+    if (gm && n_g > 0 && n_x > 0) {
+        if (workspace_bytes < gmc::dense_backward_workspace_bytes(*shape)) return GMC_E_WORKSPACE;
+        if (!workspace) return GMC_E_NULL;
+    }
+    return gmc::dense_backward(grad_out, mixture, xes, grad_mixture, grad_xes, workspace, *shape, gm, gx,
+                               (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,221 @@
+// Shared device helpers of libgmc_hip (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gmc_hip.h"
+
+namespace gmc {
+
+constexpr int kBlock = 256;          // threads per workgroup of the dense kernels (4 wavefronts)
+constexpr int kWave = 64;
+
+template <int D> struct Kappa;       // (2 pi)^(-D/2)
+template <> struct Kappa<2> { static constexpr double v = 0.15915494309189535; };
+template <> struct Kappa<3> { static constexpr double v = 0.06349363593424097; };
+
+// 0.5 * log2(e): folded into the Cholesky factor so that the kernel's exponential is a bare exp2
+constexpr double kHalfLog2e = 0.72134752044448170368;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ double fast_exp2(double x) { return exp2(x); }
+__device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+// Per-Gaussian quantities derived once from the stored record (weight, position b, inverse covariance C):
+//   u     upper-triangular factor with u^T u = 0.5*log2(e) * sym(C)   (row-major packed: D=2: 00 01 11, D=3: 00 01 02 11 12 22)
+//   nd    -(u * b)
+//   bound max_i sum_j |u_ij b_j|: magnitude of the partial sums of (u x + nd) for every pair that matters
+//   norm  (2 pi)^(-D/2) * sqrt(det C),  det of C as stored
+// so that  exp(-1/2 (x-b)^T C (x-b)) = exp2(-|u x + nd|^2) = exp2(-|u (x - b)|^2).
+template <int D> struct Derived {
+    double u[D * (D + 1) / 2];
+    double nd[D];
+    double b[D];
+    double bound;
+    double norm;
+    double w;
+};
+
+template <typename T, int D>
+__device__ __forceinline__ Derived<D> derive(const T* __restrict__ g) {
+    Derived<D> r;
+    r.w = double(g[0]);
+    const T* c = g + 1 + D;
+    if constexpr (D == 2) {
+        const double c00 = c[0], c01 = c[1], c10 = c[2], c11 = c[3];
+        const double det = c00 * c11 - c01 * c10;
+        const double a00 = kHalfLog2e * c00, a01 = kHalfLog2e * 0.5 * (c01 + c10), a11 = kHalfLog2e * c11;
+        const double u00 = sqrt(a00);
+        const double u01 = a01 / u00;
+        const double u11 = sqrt(a11 - u01 * u01);
+        r.u[0] = u00; r.u[1] = u01; r.u[2] = u11;
+        const double b0 = double(g[1]), b1 = double(g[2]);
+        r.b[0] = b0; r.b[1] = b1;
+        r.nd[0] = -(u00 * b0 + u01 * b1);
+        r.nd[1] = -(u11 * b1);
+        r.bound = fmax(fabs(u00 * b0) + fabs(u01 * b1), fabs(u11 * b1));
+        r.norm = Kappa<2>::v * sqrt(det);
+    } else {
+        const double c00 = c[0], c01 = c[1], c02 = c[2], c10 = c[3], c11 = c[4], c12 = c[5], c20 = c[6], c21 = c[7],
+                     c22 = c[8];
+        const double det = c00 * (c11 * c22 - c12 * c21) - c01 * (c10 * c22 - c12 * c20) + c02 * (c10 * c21 - c11 * c20);
+        const double a00 = kHalfLog2e * c00, a11 = kHalfLog2e * c11, a22 = kHalfLog2e * c22;
+        const double a01 = kHalfLog2e * 0.5 * (c01 + c10), a02 = kHalfLog2e * 0.5 * (c02 + c20),
+                     a12 = kHalfLog2e * 0.5 * (c12 + c21);
+        const double u00 = sqrt(a00);
+        const double u01 = a01 / u00, u02 = a02 / u00;
+        const double u11 = sqrt(a11 - u01 * u01);
+        const double u12 = (a12 - u01 * u02) / u11;
+        const double u22 = sqrt(a22 - u02 * u02 - u12 * u12);
+        r.u[0] = u00; r.u[1] = u01; r.u[2] = u02; r.u[3] = u11; r.u[4] = u12; r.u[5] = u22;
+        const double b0 = double(g[1]), b1 = double(g[2]), b2 = double(g[3]);
+        r.b[0] = b0; r.b[1] = b1; r.b[2] = b2;
+        r.nd[0] = -(u00 * b0 + u01 * b1 + u02 * b2);
+        r.nd[1] = -(u11 * b1 + u12 * b2);
+        r.nd[2] = -(u22 * b2);
+        r.bound = fmax(fabs(u00 * b0) + fabs(u01 * b1) + fabs(u02 * b2), fmax(fabs(u11 * b1) + fabs(u12 * b2), fabs(u22 * b2)));
+        r.norm = Kappa<3>::v * sqrt(det);
+    }
+    return r;
+}
+
+// LDS record of one Gaussian for the pair loop: u, then nd ("shifted" form) or b ("centred" form), the
+// amplitude, and the Gaussian's index within its tile; padded to a multiple of 16 bytes.
+//
+// Two ways to get y = u (x - b):
+//   shifted:  y = u x + nd        D(D+1)/2 FMAs, but the partial sums are as large as |u b|, so the absolute
+//             rounding error of y grows with the distance of the Gaussian from the origin in units of its width;
+//   centred:  t = x - b, y = u t  D more instructions, error relative to |y| only.
+// A Gaussian takes the shifted form iff its `bound` is at most ShiftedBound<T>::v (absolute error of y about
+// 2 * unit roundoff * bound: 2e-6 in float, 6e-14 in double).
+template <typename T> struct ShiftedBound;
+template <> struct ShiftedBound<float> { static constexpr double v = 16.0; };
+template <> struct ShiftedBound<double> { static constexpr double v = 256.0; };
+
+template <typename T, int D> struct Rec {
+    static constexpr int kU = D * (D + 1) / 2;
+    static constexpr int kAmp = kU + D;
+    static constexpr int kIdx = kU + D + 1;
+    static constexpr int kUsed = kU + D + 1;                                     // 6 / 10 (without the index)
+    static constexpr int kStride = (D == 2) ? 8 : 12;
+};
+
+template <typename T, int D>
+__device__ __forceinline__ void store_record(T* rec, const Derived<D>& d, bool centred, double amplitude, int index) {
+    constexpr int kU = Rec<T, D>::kU;
+#pragma unroll
+    for (int i = 0; i < kU; ++i) rec[i] = T(d.u[i]);
+#pragma unroll
+    for (int i = 0; i < D; ++i) rec[kU + i] = T(centred ? d.b[i] : d.nd[i]);
+    rec[Rec<T, D>::kAmp] = T(amplitude);
+    reinterpret_cast<int*>(rec + Rec<T, D>::kIdx)[0] = index;
+}
+
+template <typename T, int D>
+__device__ __forceinline__ int record_index(const T* rec) {
+    return reinterpret_cast<const int*>(rec + Rec<T, D>::kIdx)[0];
+}
+
+// y = u (x - b) in the shifted (CENTRED == false) or centred form; returns q = |y|^2
+template <typename T, int D, bool CENTRED>
+__device__ __forceinline__ T quad_form(const T* __restrict__ r, const T* __restrict__ x, T* __restrict__ y) {
+    if constexpr (D == 2) {
+        if constexpr (CENTRED) {
+            const T t0 = x[0] - r[3], t1 = x[1] - r[4];
+            y[1] = r[2] * t1;
+            y[0] = fma_(r[0], t0, r[1] * t1);
+        } else {
+            y[1] = fma_(r[2], x[1], r[4]);
+            y[0] = fma_(r[0], x[0], fma_(r[1], x[1], r[3]));
+        }
+        return fma_(y[1], y[1], y[0] * y[0]);
+    } else {
+        if constexpr (CENTRED) {
+            const T t0 = x[0] - r[6], t1 = x[1] - r[7], t2 = x[2] - r[8];
+            y[2] = r[5] * t2;
+            y[1] = fma_(r[3], t1, r[4] * t2);
+            y[0] = fma_(r[0], t0, fma_(r[1], t1, r[2] * t2));
+        } else {
+            y[2] = fma_(r[5], x[2], r[8]);
+            y[1] = fma_(r[3], x[1], fma_(r[4], x[2], r[7]));
+            y[0] = fma_(r[0], x[0], fma_(r[1], x[1], fma_(r[2], x[2], r[6])));
+        }
+        return fma_(y[2], y[2], fma_(y[1], y[1], y[0] * y[0]));
+    }
+}
+
+// Stages up to 256 Gaussians (one per lane of a 256-lane workgroup) into LDS, shifted-form records first,
+// centred-form records after them (stable order within each group); counts[8] receives the number of shifted
+// records.  Contains two workgroup barriers: the first also orders the overwrite of the tile after every lane's
+// reads of the previous one, the second publishes the new tile, so the caller needs no barrier of its own.
+template <typename T, int D>
+__device__ __forceinline__ void stage_tile(const T* __restrict__ gaussians, int cnt, double amp_scale, T* lds,
+                                           int* counts /* LDS int[10] */) {
+    constexpr int S = Rec<T, D>::kStride;
+    constexpr int G = 1 + D + D * D;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const bool active = tid < cnt;
+    Derived<D> dv;
+    bool centred = false;
+    if (active) {
+        dv = derive<T, D>(gaussians + size_t(tid) * G);
+        centred = !(dv.bound <= ShiftedBound<T>::v);
+    }
+    const unsigned long long mc = __ballot(active && centred);
+    const unsigned long long ms = __ballot(active && !centred);
+    if (lane == 0) { counts[wave] = __popcll(ms); counts[4 + wave] = __popcll(mc); }
+    __syncthreads();
+    int shifted_before = 0, centred_before = 0, shifted_total = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const int cs = counts[w], cc = counts[4 + w];
+        if (w < wave) { shifted_before += cs; centred_before += cc; }
+        shifted_total += cs;
+    }
+    if (active) {
+        const unsigned long long below = (1ull << lane) - 1ull;
+        const int slot = centred ? shifted_total + centred_before + __popcll(mc & below)
+                                 : shifted_before + __popcll(ms & below);
+        store_record<T, D>(lds + slot * S, dv, centred, dv.w * dv.norm * amp_scale, tid);
+    }
+    if (tid == 0) counts[8] = shifted_total;
+    __syncthreads();
+}
+
+// ---- wavefront (64 lanes) sum; the total arrives in lane 63 -------------------------------------------
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+    v += dpp_mov<0x111>(v);          // row_shr:1
+    v += dpp_mov<0x112>(v);          // row_shr:2
+    v += dpp_mov<0x114>(v);          // row_shr:4
+    v += dpp_mov<0x118>(v);          // row_shr:8   -> lane 15 of every row holds the row sum
+    v += dpp_mov<0x142, 0xa>(v);     // row_bcast:15 into rows 1 and 3
+    v += dpp_mov<0x143, 0xc>(v);     // row_bcast:31 into rows 2 and 3 -> lane 63 holds the total
+    return v;
+}
+
+__device__ __forceinline__ double wave_sum_to_lane63(double v) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const double o = __shfl_up(v, off, 64);
+        if ((threadIdx.x & 63) >= off) v += o;
+    }
+    return v;
+}
+
+__device__ __forceinline__ void atomic_add(float* p, float v) { unsafeAtomicAdd(p, v); }
+__device__ __forceinline__ void atomic_add(double* p, double v) { unsafeAtomicAdd(p, v); }
+
+template <typename T>
+__global__ void fill_zero_kernel(T* p, size_t n) {
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = T(0);
+}
+
+}  // namespace gmc

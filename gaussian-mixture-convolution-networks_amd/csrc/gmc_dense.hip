@@ -1,0 +1,412 @@
+// Dense all-pairs Gaussian-mixture evaluation for gfx950: forward, backward and the per-Gaussian epilogue.
+//
+// Replaces the per-point serial loops of the reference
+// (src/gmc/cpp/extensions/evaluate_inversed/parallel_implementation.cu:23-55 forward, :133-173 backward,
+//  parallel_implementation_optimised_backward.cu:39-107) with a points x Gaussians tiling:
+//   * a workgroup of 256 lanes owns P points per lane of one (b,l) mixture and keeps them in registers;
+//   * Gaussians are staged tile by tile into LDS as pre-transformed records (Cholesky factor u of the scaled
+//     inverse covariance, -u b, amplitude), so a pair costs D(D+1)/2 FMAs for y = u x - u b, D for |y|^2, one
+//     exp2 and one FMA, with no per-pair subtraction, determinant or square root; Gaussians that sit too far
+//     from the origin for that form (in units of their width) keep an explicit x - b instead;
+//   * backward keeps dL/dx per point in registers and reduces the 1 + D + D(D+1)/2 per-Gaussian sums over the
+//     wavefront (DPP), over the workgroup (LDS) and over workgroups (one atomic per scalar and workgroup);
+//     a per-Gaussian epilogue turns the sums into (dw, db, dC).
+#include "gmc_common.h"
+
+namespace gmc {
+
+constexpr int kTile = 256;   // Gaussians staged per LDS tile (one per lane)
+
+template <typename T, int D, int P, bool CENTRED>
+__device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, int begin, int end, const T (&x)[P][D], T (&acc)[P]) {
+    constexpr int S = Rec<T, D>::kStride;
+#pragma unroll 2
+    for (int g = begin; g < end; ++g) {
+        T r[Rec<T, D>::kUsed];
+#pragma unroll
+        for (int i = 0; i < Rec<T, D>::kUsed; ++i) r[i] = lds[g * S + i];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            T y[D];
+            const T q = quad_form<T, D, CENTRED>(r, x[p], y);
+            acc[p] = fma_(r[Rec<T, D>::kAmp], fast_exp2(-q), acc[p]);
+        }
+    }
+}
+
+template <typename T, int D, int P>
+__global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ mixture, const T* __restrict__ xes,
+                                                          T* __restrict__ out, int L, int M, int N, int Bx, int Lx,
+                                                          int chunks) {
+    constexpr int G = 1 + D + D * D;
+    constexpr int S = Rec<T, D>::kStride;
+    __shared__ __attribute__((aligned(16))) T lds[kTile * S];
+    __shared__ int counts[10];
+
+    const int bl = blockIdx.x / chunks;
+    const int chunk = blockIdx.x - bl * chunks;
+    const int b = bl / L, l = bl - b * L;
+    const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
+    const T* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
+    const T* __restrict__ x_bl = xes + (size_t(xb) * Lx + xl) * N * D;
+
+    T x[P][D];
+    T acc[P];
+    const int n0 = chunk * (kBlock * P) + threadIdx.x;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        int n = n0 + p * kBlock;
+        n = n < N ? n : N - 1;
+#pragma unroll
+        for (int d = 0; d < D; ++d) x[p][d] = x_bl[size_t(n) * D + d];
+        acc[p] = T(0);
+    }
+
+    for (int g0 = 0; g0 < M; g0 += kTile) {
+        const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
+        stage_tile<T, D>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts);
+        const int n_shifted = counts[8];
+        fwd_pairs<T, D, P, false>(lds, 0, n_shifted, x, acc);
+        fwd_pairs<T, D, P, true>(lds, n_shifted, cnt, x, acc);
+    }
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int n = n0 + p * kBlock;
+        if (n < N) out[size_t(bl) * N + n] = acc[p];
+    }
+}
+
+// Per-Gaussian partial sums of the backward pass, in the transformed coordinates y = u (x - b):
+//   R0 = sum_n e g,  R1_i = sum_n e g y_i,  R2_ij = sum_n e g y_i y_j (i <= j)     with e = exp2(-|y|^2)
+template <int D> struct Sums { static constexpr int k = 1 + D + D * (D + 1) / 2; };   // 6 / 10
+
+template <typename T, int D, int P, bool NEED_GM, bool NEED_GX, bool CENTRED>
+__device__ __forceinline__ void bwd_pairs(const T* __restrict__ lds, T* __restrict__ block_sums, int begin, int end,
+                                          const T (&x)[P][D], const T (&go)[P], T (&gx)[P][D]) {
+    constexpr int S = Rec<T, D>::kStride;
+    constexpr int NR = Sums<D>::k;
+    for (int g = begin; g < end; ++g) {
+        T r[Rec<T, D>::kUsed];
+#pragma unroll
+        for (int i = 0; i < Rec<T, D>::kUsed; ++i) r[i] = lds[g * S + i];
+        T rs[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) rs[i] = T(0);
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            T y[D];
+            const T q = quad_form<T, D, CENTRED>(r, x[p], y);
+            const T e = fast_exp2(-q);
+            if (NEED_GX) {
+                const T s = r[Rec<T, D>::kAmp] * e;
+                if constexpr (D == 2) {
+                    const T sy0 = s * y[0], sy1 = s * y[1];
+                    gx[p][0] = fma_(r[0], sy0, gx[p][0]);
+                    gx[p][1] = fma_(r[1], sy0, fma_(r[2], sy1, gx[p][1]));
+                } else {
+                    const T sy0 = s * y[0], sy1 = s * y[1], sy2 = s * y[2];
+                    gx[p][0] = fma_(r[0], sy0, gx[p][0]);
+                    gx[p][1] = fma_(r[1], sy0, fma_(r[3], sy1, gx[p][1]));
+                    gx[p][2] = fma_(r[2], sy0, fma_(r[4], sy1, fma_(r[5], sy2, gx[p][2])));
+                }
+            }
+            if (NEED_GM) {
+                const T eg = e * go[p];
+                rs[0] += eg;
+                if constexpr (D == 2) {
+                    const T a0 = eg * y[0], a1 = eg * y[1];
+                    rs[1] += a0; rs[2] += a1;
+                    rs[3] = fma_(a0, y[0], rs[3]); rs[4] = fma_(a0, y[1], rs[4]); rs[5] = fma_(a1, y[1], rs[5]);
+                } else {
+                    const T a0 = eg * y[0], a1 = eg * y[1], a2 = eg * y[2];
+                    rs[1] += a0; rs[2] += a1; rs[3] += a2;
+                    rs[4] = fma_(a0, y[0], rs[4]); rs[5] = fma_(a0, y[1], rs[5]); rs[6] = fma_(a0, y[2], rs[6]);
+                    rs[7] = fma_(a1, y[1], rs[7]); rs[8] = fma_(a1, y[2], rs[8]); rs[9] = fma_(a2, y[2], rs[9]);
+                }
+            }
+        }
+        if (NEED_GM) {
+#pragma unroll
+            for (int i = 0; i < NR; ++i) rs[i] = wave_sum_to_lane63(rs[i]);
+            if ((threadIdx.x & 63) == 63) {
+                const int idx = record_index<T, D>(lds + g * S);
+#pragma unroll
+                for (int i = 0; i < NR; ++i) atomic_add(&block_sums[idx * NR + i], rs[i]);
+            }
+        }
+    }
+}
+
+template <typename T, int D, int P, bool NEED_GM, bool NEED_GX>
+__global__ __launch_bounds__(kBlock) void eval_bwd_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture,
+                                                          const T* __restrict__ xes, T* __restrict__ sums,
+                                                          T* __restrict__ grad_xes, int L, int M, int N, int Bx, int Lx,
+                                                          int chunks, int xes_shared) {
+    constexpr int G = 1 + D + D * D;
+    constexpr int S = Rec<T, D>::kStride;
+    constexpr int NR = Sums<D>::k;
+    __shared__ __attribute__((aligned(16))) T lds[kTile * S];
+    __shared__ T block_sums[NEED_GM ? kTile * NR : 1];
+    __shared__ int counts[10];
+
+    const int bl = blockIdx.x / chunks;
+    const int chunk = blockIdx.x - bl * chunks;
+    const int b = bl / L, l = bl - b * L;
+    const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
+    const T* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
+    const size_t x_off = (size_t(xb) * Lx + xl) * N;
+    const T* __restrict__ x_bl = xes + x_off * D;
+
+    T x[P][D];
+    T go[P];
+    T gx[P][D];
+    const int n0 = chunk * (kBlock * P) + threadIdx.x;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int n = n0 + p * kBlock;
+        const int nc = n < N ? n : N - 1;
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            x[p][d] = x_bl[size_t(nc) * D + d];
+            gx[p][d] = T(0);
+        }
+        go[p] = n < N ? grad_out[size_t(bl) * N + nc] : T(0);   // padding lanes contribute nothing
+    }
+    if (NEED_GM) {
+        for (int i = threadIdx.x; i < kTile * NR; i += kBlock) block_sums[i] = T(0);
+    }
+
+    for (int g0 = 0; g0 < M; g0 += kTile) {
+        const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
+        // amplitude for dL/dx: w * norm / (0.5 log2 e), because C t = u^T y / (0.5 log2 e)
+        stage_tile<T, D>(mix_bl + size_t(g0) * G, cnt, 1.0 / kHalfLog2e, lds, counts);
+        const int n_shifted = counts[8];
+        bwd_pairs<T, D, P, NEED_GM, NEED_GX, false>(lds, block_sums, 0, n_shifted, x, go, gx);
+        bwd_pairs<T, D, P, NEED_GM, NEED_GX, true>(lds, block_sums, n_shifted, cnt, x, go, gx);
+        if (NEED_GM) {
+            __syncthreads();
+            T* __restrict__ dst = sums + (size_t(bl) * M + g0) * NR;
+            for (int i = threadIdx.x; i < cnt * NR; i += kBlock) {
+                atomic_add(&dst[i], block_sums[i]);
+                block_sums[i] = T(0);
+            }
+        }
+    }
+    if (NEED_GX) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int n = n0 + p * kBlock;
+            if (n < N) {
+                T* dst = grad_xes + (x_off + n) * D;
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    const T v = -go[p] * gx[p][d];
+                    if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
+                }
+            }
+        }
+    }
+}
+
+// Epilogue, one lane per Gaussian: (R0, R1, R2) -> (dw, db, dC), written to grad_mixture in the reference's
+// layout.  With t = u^-1 y and f g = w norm e g (util/grad/gaussian.h:31-65):
+//   dw  = norm R0
+//   db  = w norm / (0.5 log2 e) * u^T R1
+//   dC  = -1/2 w norm * u^-1 R2 u^-T  +  cofactor(C) * w kappa R0 / (2 sqrt(det C))
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void eval_bwd_epilogue_kernel(const T* __restrict__ mixture,
+                                                                   const T* __restrict__ sums,
+                                                                   T* __restrict__ grad_mixture, size_t n_gaussians) {
+    constexpr int G = 1 + D + D * D;
+    constexpr int NR = Sums<D>::k;
+    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n_gaussians) return;
+    const T* g = mixture + i * G;
+    const T* rs = sums + i * NR;
+    T* o = grad_mixture + i * G;
+    const Derived<D> dv = derive<T, D>(g);
+    const double R0 = double(rs[0]);
+    const double wn = dv.w * dv.norm;
+    o[0] = T(dv.norm * R0);
+    const T* c = g + 1 + D;
+    if constexpr (D == 2) {
+        const double u00 = dv.u[0], u01 = dv.u[1], u11 = dv.u[2];
+        const double r1[2] = {double(rs[1]), double(rs[2])};
+        const double k = wn / kHalfLog2e;
+        o[1] = T(k * (u00 * r1[0]));
+        o[2] = T(k * (u01 * r1[0] + u11 * r1[1]));
+        // V = u^-1 (upper triangular)
+        const double v00 = 1.0 / u00, v11 = 1.0 / u11, v01 = -u01 * v00 * v11;
+        const double s00 = double(rs[3]), s01 = double(rs[4]), s11 = double(rs[5]);
+        // A = V S V^T
+        const double m00 = v00 * s00 + v01 * s01, m01 = v00 * s01 + v01 * s11, m11 = v11 * s11;
+        const double a00 = m00 * v00 + m01 * v01, a01 = m01 * v11, a11 = m11 * v11;
+        const double det = double(c[0]) * double(c[3]) - double(c[1]) * double(c[2]);
+        const double kd = dv.w * Kappa<2>::v * R0 / (2.0 * sqrt(det));
+        o[3] = T(-0.5 * wn * a00 + double(c[3]) * kd);
+        o[4] = T(-0.5 * wn * a01 - double(c[2]) * kd);
+        o[5] = T(-0.5 * wn * a01 - double(c[1]) * kd);
+        o[6] = T(-0.5 * wn * a11 + double(c[0]) * kd);
+    } else {
+        const double u00 = dv.u[0], u01 = dv.u[1], u02 = dv.u[2], u11 = dv.u[3], u12 = dv.u[4], u22 = dv.u[5];
+        const double r1[3] = {double(rs[1]), double(rs[2]), double(rs[3])};
+        const double k = wn / kHalfLog2e;
+        o[1] = T(k * (u00 * r1[0]));
+        o[2] = T(k * (u01 * r1[0] + u11 * r1[1]));
+        o[3] = T(k * (u02 * r1[0] + u12 * r1[1] + u22 * r1[2]));
+        const double v00 = 1.0 / u00, v11 = 1.0 / u11, v22 = 1.0 / u22;
+        const double v01 = -u01 * v00 * v11;
+        const double v12 = -u12 * v11 * v22;
+        const double v02 = -(u01 * v12 + u02 * v22) * v00;
+        const double s[3][3] = {{double(rs[4]), double(rs[5]), double(rs[6])},
+                                {double(rs[5]), double(rs[7]), double(rs[8])},
+                                {double(rs[6]), double(rs[8]), double(rs[9])}};
+        const double V[3][3] = {{v00, v01, v02}, {0.0, v11, v12}, {0.0, 0.0, v22}};
+        double m[3][3], a[3][3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int q = 0; q < 3; ++q) m[r][q] = V[r][0] * s[0][q] + V[r][1] * s[1][q] + V[r][2] * s[2][q];
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int q = 0; q < 3; ++q) a[r][q] = m[r][0] * V[q][0] + m[r][1] * V[q][1] + m[r][2] * V[q][2];
+        double cc[3][3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int q = 0; q < 3; ++q) cc[r][q] = double(c[r * 3 + q]);
+        const double det = cc[0][0] * (cc[1][1] * cc[2][2] - cc[1][2] * cc[2][1]) -
+                           cc[0][1] * (cc[1][0] * cc[2][2] - cc[1][2] * cc[2][0]) +
+                           cc[0][2] * (cc[1][0] * cc[2][1] - cc[1][1] * cc[2][0]);
+        const double kd = dv.w * Kappa<3>::v * R0 / (2.0 * sqrt(det));
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const int r1i = r == 0 ? 1 : 0, r2i = r == 2 ? 1 : 2;
+#pragma unroll
+            for (int q = 0; q < 3; ++q) {
+                const int q1 = q == 0 ? 1 : 0, q2 = q == 2 ? 1 : 2;
+                const double sign = ((r + q) & 1) ? -1.0 : 1.0;
+                const double cof = sign * (cc[r1i][q1] * cc[r2i][q2] - cc[r1i][q2] * cc[r2i][q1]);
+                o[4 + r * 3 + q] = T(-0.5 * wn * a[r][q] + cof * kd);
+            }
+        }
+    }
+}
+
+// ---- host-side launchers ------------------------------------------------------------------------------
+
+static int pick_points_per_lane(int N, int BL) {
+    // keep the padding of the last chunk small and leave enough workgroups for 256 CUs
+    const int cands[4] = {8, 4, 2, 1};
+    for (int c : cands) {
+        const int span = kBlock * c;
+        const int chunks = (N + span - 1) / span;
+        const double waste = double(chunks) * span / double(N > 0 ? N : 1);
+        if (waste <= 1.15 && (size_t(chunks) * BL >= 1024 || c == 1)) return c;
+    }
+    int best = 1;
+    double best_waste = 1e30;
+    for (int c : cands) {
+        const int span = kBlock * c;
+        const int chunks = (N + span - 1) / span;
+        const double waste = double(chunks) * span / double(N > 0 ? N : 1);
+        if (waste < best_waste - 1e-9) { best_waste = waste; best = c; }
+    }
+    return best;
+}
+
+template <typename T>
+static void zero_async(T* p, size_t n, hipStream_t stream) {
+    if (n == 0) return;
+    const size_t blocks = (n + 255) / 256;
+    fill_zero_kernel<T><<<dim3(unsigned(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream>>>(p, n);
+}
+
+template <typename T, int D>
+static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s, hipStream_t stream) {
+    const size_t BL = size_t(s.B) * s.L;
+    if (BL == 0 || s.N == 0) return GMC_OK;
+    if (s.M == 0) { zero_async(out, BL * s.N, stream); return GMC_OK; }
+    const int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
+    const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
+    const dim3 grid(unsigned(BL * chunks));
+#define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks)
+    switch (P) {
+        case 8: GMC_FWD(8); break;
+        case 4: GMC_FWD(4); break;
+        case 2: GMC_FWD(2); break;
+        default: GMC_FWD(1); break;
+    }
+#undef GMC_FWD
+    return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
+
+template <typename T, int D, bool GM, bool GX>
+static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T* sums, T* grad_xes, const gmc_shape& s,
+                            int xes_shared, hipStream_t stream) {
+    const size_t BL = size_t(s.B) * s.L;
+    int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
+    if (P > 4 && sizeof(T) == 8) P = 4;
+    const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
+    const dim3 grid(unsigned(BL * chunks));
+#define GMC_BWD(PP) eval_bwd_kernel<T, D, PP, GM, GX><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared)
+    switch (P) {
+        case 8: GMC_BWD(8); break;
+        case 4: GMC_BWD(4); break;
+        case 2: GMC_BWD(2); break;
+        default: GMC_BWD(1); break;
+    }
+#undef GMC_BWD
+}
+
+template <typename T, int D>
+static int launch_bwd(const T* grad_out, const T* mixture, const T* xes, T* grad_mixture, T* grad_xes, T* sums,
+                      const gmc_shape& s, bool need_gm, bool need_gx, hipStream_t stream) {
+    constexpr int G = 1 + D + D * D;
+    const size_t BL = size_t(s.B) * s.L;
+    const size_t n_gauss = BL * s.M;
+    const size_t n_x = size_t(s.Bx) * s.Lx * s.N * D;
+    const int xes_shared = (s.Bx != s.B || s.Lx != s.L) ? 1 : 0;
+    if (BL == 0) return GMC_OK;
+    if (s.N == 0 || s.M == 0) {
+        if (need_gm) zero_async(grad_mixture, n_gauss * G, stream);
+        if (need_gx) zero_async(grad_xes, n_x, stream);
+        return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+    }
+    if (need_gm) zero_async(sums, n_gauss * Sums<D>::k, stream);
+    if (need_gx && xes_shared) zero_async(grad_xes, n_x, stream);
+    if (need_gm && need_gx) launch_bwd_main<T, D, true, true>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, stream);
+    else if (need_gm) launch_bwd_main<T, D, true, false>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, stream);
+    else if (need_gx) launch_bwd_main<T, D, false, true>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, stream);
+    if (need_gm) {
+        const size_t blocks = (n_gauss + kBlock - 1) / kBlock;
+        eval_bwd_epilogue_kernel<T, D><<<dim3(unsigned(blocks)), dim3(kBlock), 0, stream>>>(mixture, sums, grad_mixture, n_gauss);
+    }
+    return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
+
+int dense_forward(const void* mixture, const void* xes, void* out, const gmc_shape& s, hipStream_t stream) {
+    if (s.dtype == GMC_F32) {
+        if (s.D == 2) return launch_fwd<float, 2>((const float*)mixture, (const float*)xes, (float*)out, s, stream);
+        return launch_fwd<float, 3>((const float*)mixture, (const float*)xes, (float*)out, s, stream);
+    }
+    if (s.D == 2) return launch_fwd<double, 2>((const double*)mixture, (const double*)xes, (double*)out, s, stream);
+    return launch_fwd<double, 3>((const double*)mixture, (const double*)xes, (double*)out, s, stream);
+}
+
+size_t dense_backward_workspace_bytes(const gmc_shape& s) {
+    const size_t elt = s.dtype == GMC_F32 ? 4 : 8;
+    const size_t nr = s.D == 2 ? Sums<2>::k : Sums<3>::k;
+    return size_t(s.B) * s.L * s.M * nr * elt;
+}
+
+int dense_backward(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                   void* workspace, const gmc_shape& s, bool need_gm, bool need_gx, hipStream_t stream) {
+#define GMC_CALL(T, DD) launch_bwd<T, DD>((const T*)grad_out, (const T*)mixture, (const T*)xes, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, s, need_gm, need_gx, stream)
+    if (s.dtype == GMC_F32) return s.D == 2 ? GMC_CALL(float, 2) : GMC_CALL(float, 3);
+    return s.D == 2 ? GMC_CALL(double, 2) : GMC_CALL(double, 3);
+#undef GMC_CALL
+}
+
+}  // namespace gmc

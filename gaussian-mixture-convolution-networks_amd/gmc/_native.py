@@ -1,0 +1,161 @@
+"""Loader and thin ctypes front end of libgmc_hip.so (the C ABI declared in include/gmc_hip.h).
+
+PyTorch is used for device memory and streams only: tensors are allocated with torch, raw device pointers and the
+current HIP stream are handed to the library.  There is no CPU or pure-torch fallback: if the library is
+missing, or a tensor does not live on a HIP device, the call raises.
+"""
+import ctypes
+import os
+import subprocess
+
+import torch
+
+_PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC_DIR = os.path.join(_PKG_DIR, "csrc")
+LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
+
+GMC_F32, GMC_F64 = 0, 1
+GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
+ABI_VERSION = 1
+
+
+class Shape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int) for n in ("B", "L", "M", "N", "D", "Bx", "Lx", "dtype")]
+
+
+class BvhConfigC(ctypes.Structure):
+    _fields_ = [("aabb_mode", ctypes.c_int), ("aabb_threshold", ctypes.c_float)]
+
+
+def build(verbose: bool = False) -> str:
+    """Compiles every HIP source of the library for gfx950 (hipcc cross-compiles without a GPU)."""
+    out = None if verbose else subprocess.DEVNULL
+    subprocess.run(["make", "-B", "-j8", "-C", CSRC_DIR, "libgmc_hip.so"], check=True, stdout=out, stderr=out)
+    global _lib
+    _lib = None
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is missing: build it first (python -c 'import __graft_entry__ as g; g.build()' "
+                           f"or make -C {CSRC_DIR}); there is no fallback implementation")
+    l = ctypes.CDLL(LIB_PATH)
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    shp = ctypes.POINTER(Shape)
+    cfg = ctypes.POINTER(BvhConfigC)
+    l.gmc_error_string.restype = ctypes.c_char_p
+    l.gmc_error_string.argtypes = [ci]
+    l.gmc_abi_version.restype = ci
+    l.gmc_eval_fwd.argtypes = [vp, vp, vp, shp, vp]
+    l.gmc_eval_bwd_workspace_bytes.restype = sz
+    l.gmc_eval_bwd_workspace_bytes.argtypes = [shp]
+    l.gmc_eval_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
+    if hasattr(l, "gmc_bvh_bytes"):
+        l.gmc_bvh_bytes.restype = sz
+        l.gmc_bvh_bytes.argtypes = [shp]
+        l.gmc_bvh_build.argtypes = [vp, vp, vp, sz, shp, cfg, vp]
+        l.gmc_bvh_export_boxes.argtypes = [vp, vp, vp, shp, vp]
+        l.gmc_bvh_export_nodes.argtypes = [vp, vp, vp, shp, vp]
+        l.gmc_eval_bvh_fwd.argtypes = [vp, vp, vp, vp, shp, vp]
+        l.gmc_eval_bvh_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
+    if l.gmc_abi_version() != ABI_VERSION:
+        raise RuntimeError("libgmc_hip.so was built from a different include/gmc_hip.h; rebuild it")
+    _lib = l
+    return l
+
+
+def check(code: int) -> None:
+    if code != 0:
+        raise RuntimeError("gmc_hip: " + lib().gmc_error_string(code).decode())
+
+
+def n_dimensions(mixture: torch.Tensor) -> int:
+    last = mixture.shape[-1]
+    if last == 7:
+        return 2
+    if last == 13:
+        return 3
+    raise RuntimeError("mixture must have 7 or 13 elements in the last dimension")
+
+
+def check_input(mixture: torch.Tensor, xes: torch.Tensor) -> Shape:
+    """Same rules and messages as gpe::check_input_and_get_ns (src/gmc/cpp/extensions/util/mixture.h:107-127)
+    plus the dtype dispatch of parallel_implementation.cu:78 (floating types only)."""
+    if mixture.dim() != 4:
+        raise RuntimeError("mixture must have 4 dimensions")
+    d = n_dimensions(mixture)
+    if not mixture.is_contiguous():
+        raise RuntimeError("mixture must be contiguous")
+    if not xes.is_contiguous():
+        raise RuntimeError("xes must be contiguous")
+    if xes.dim() != 4:
+        raise RuntimeError("xes must have 4 dimensions")
+    if xes.dtype != mixture.dtype:
+        raise RuntimeError("mixture and xes must have the same dtype")
+    if xes.device != mixture.device:
+        raise RuntimeError("mixture and xes must have the same device")
+    if mixture.dtype not in (torch.float32, torch.float64):
+        raise RuntimeError("unsupported datatype: evaluate_inversed is implemented for float32 and float64")
+    B, L, M, _ = mixture.shape
+    Bx, Lx, N, Dx = xes.shape
+    if Bx not in (1, B):
+        raise RuntimeError("xes must have a batch dimension equal to one or the mixture")
+    if Lx not in (1, L):
+        raise RuntimeError("xes must have a layer dimension equal to one or the mixture")
+    if Dx != d:
+        raise RuntimeError("xes must have the last dimension equal to the number of dimensions of the mixture")
+    if not mixture.is_cuda:
+        raise RuntimeError("gmc_hip evaluates on an AMD GPU only: mixture and xes must be HIP ('cuda') tensors; "
+                           "this build has no CPU implementation")
+    return Shape(B, L, M, N, d, Bx, Lx, GMC_F32 if mixture.dtype == torch.float32 else GMC_F64)
+
+
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else ctypes.c_void_p(0)
+
+
+def eval_fwd(mixture: torch.Tensor, xes: torch.Tensor) -> torch.Tensor:
+    shape = check_input(mixture, xes)
+    out = torch.empty((shape.B, shape.L, shape.N), dtype=mixture.dtype, device=mixture.device)
+    with torch.cuda.device(mixture.device):
+        check(lib().gmc_eval_fwd(_p(mixture), _p(xes), _p(out), ctypes.byref(shape), _stream(mixture.device)))
+    return out
+
+
+def eval_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool):
+    shape = check_input(mixture, xes)
+    if grad_output.dim() != 3:
+        raise RuntimeError("grad_output has wrong number of dimensions")
+    if grad_output.shape[0] != shape.B:
+        raise RuntimeError("grad_output has wrong batch dimension")
+    if grad_output.shape[1] != shape.L:
+        raise RuntimeError("grad_output has wrong layer dimension")
+    if grad_output.shape[2] != shape.N:
+        raise RuntimeError("grad_output has wrong xes dimension")
+    if grad_output.dtype != mixture.dtype:
+        raise RuntimeError("grad_output dtype does not match with mixture dtype")
+    if not grad_output.is_contiguous():
+        raise RuntimeError("grad_output must be contiguous")
+    dev = mixture.device
+    # both gradients are always returned, all-zero when not required (parallel_implementation.cu:120-121,175)
+    grad_mixture = torch.empty_like(mixture) if need_mixture else torch.zeros_like(mixture)
+    grad_xes = torch.empty_like(xes) if need_xes else torch.zeros_like(xes)
+    if not (need_mixture or need_xes):
+        return grad_mixture, grad_xes
+    with torch.cuda.device(dev):
+        ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
+        ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
+        check(lib().gmc_eval_bwd(_p(grad_output), _p(mixture), _p(xes), _p(grad_mixture), _p(grad_xes), _p(ws),
+                                 ws_bytes, ctypes.byref(shape), int(need_mixture), int(need_xes), _stream(dev)))
+    return grad_mixture, grad_xes

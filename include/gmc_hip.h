@@ -1,0 +1,101 @@
+/* C ABI of libgmc_hip.so: Gaussian-mixture evaluation (`evaluate_inversed`) on AMD MI355X (gfx950).
+ *
+ * Plain pointers and sizes only; every pointer is DEVICE memory owned by the caller, `stream` is a
+ * hipStream_t (NULL = the default stream).  All calls only enqueue work on `stream`; none synchronises the
+ * device or allocates memory.  Return value: 0 on success, a negative GMC_E_* code otherwise (nothing is
+ * enqueued then); gmc_error_string() names it.
+ *
+ * Tensor layout (identical to the reference, src/gmc/mixture.py:37-67):
+ *   mixture  [B][L][M][1+D+D*D]  weight, position (D), INVERSE covariance (DxD row-major), contiguous
+ *   xes      [Bx][Lx][N][D]      query points, Bx in {1,B}, Lx in {1,L} (size-1 dims broadcast)
+ *   out      [B][L][N]
+ *   D in {2,3}; dtype GMC_F32 or GMC_F64 for all tensors of a call.
+ */
+#ifndef GMC_HIP_H
+#define GMC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { GMC_F32 = 0, GMC_F64 = 1 };
+
+enum {
+    GMC_OK = 0,
+    GMC_E_DIMS = -1,       /* D not in {2,3} */
+    GMC_E_DTYPE = -2,      /* dtype not GMC_F32 / GMC_F64 */
+    GMC_E_SHAPE = -3,      /* negative size, Bx not in {1,B}, Lx not in {1,L}, size beyond 2^31-1 elements per (b,l) */
+    GMC_E_NULL = -4,       /* a required pointer is NULL */
+    GMC_E_WORKSPACE = -5,  /* workspace smaller than the matching *_workspace_bytes() */
+    GMC_E_LAUNCH = -6,     /* the HIP runtime refused a launch (hipGetLastError) */
+    GMC_E_CONFIG = -7      /* unknown aabb mode / invalid threshold */
+};
+
+/* shape of one call; replaces gpe::MixtureAndXesNs (src/gmc/cpp/extensions/util/mixture.h:9-17) */
+typedef struct gmc_shape {
+    int B, L, M, N, D, Bx, Lx, dtype;
+} gmc_shape;
+
+const char* gmc_error_string(int code);
+/* ABI version of this header; bumps when a signature changes */
+int gmc_abi_version(void);
+
+/* ---- dense all-pairs evaluation --------------------------------------------------------------------
+ * gmc_eval_fwd replaces evaluate_inversed::parallel_forward
+ *   (src/gmc/cpp/extensions/evaluate_inversed/evaluate_inversed.cpp:11-20, parallel_implementation.cu:61-100,
+ *    parallel_implementation_optimised_forward.cu:59-98):
+ *   out[b,l,n] = sum_m w * (2 pi)^(-D/2) * sqrt(det C) * exp(-1/2 (x-b)^T C (x-b)).  `out` is fully written.
+ * The quadratic form uses the symmetric part of C (identical for any C), and C must be positive definite.
+ */
+int gmc_eval_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream);
+
+/* gmc_eval_bwd replaces evaluate_inversed::parallel_backward
+ *   (evaluate_inversed.cpp:22-34, parallel_implementation.cu:102-176, parallel_implementation_optimised_backward.cu:111-169).
+ *   grad_mixture [B][L][M][1+D+D*D] and grad_xes [Bx][Lx][N][D] (summed over broadcast dims) are fully
+ *   written; with need_grad_* == 0 the respective output is not touched and may be NULL.
+ *   `workspace`: gmc_eval_bwd_workspace_bytes(shape) bytes of device scratch (per-Gaussian partial sums).
+ */
+size_t gmc_eval_bwd_workspace_bytes(const gmc_shape* shape);
+int gmc_eval_bwd(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                 void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
+                 int need_grad_xes, void* stream);
+
+/* ---- LBVH-culled evaluation ------------------------------------------------------------------------
+ * Replaces lbvh::Bvh<D,T> (src/gmc/cpp/extensions/lbvh/bvh.h:97-148, bvh.cu:24-144: per-Gaussian boxes from
+ * the contribution cutoff, Morton codes, sort, Karras node build, bottom-up box merge) and the point query
+ * lbvh::query_device_with_fun (lbvh/query.h:13-66) composed with the evaluation, i.e. the (absent)
+ * cuda_bvh_forward / cuda_bvh_backward named at evaluate_inversed/test_evaluate_inversed.cpp:22-23:
+ *   out[b,l,n] = sum over Gaussians m whose own box contains x_n (closed interval, lbvh/aabb.h:39-47).
+ */
+enum { GMC_AABB_REFERENCE = 0, GMC_AABB_TIGHT = 1 };
+
+typedef struct gmc_bvh_config {
+    int aabb_mode;          /* GMC_AABB_REFERENCE: the rule of lbvh/bvh.cu:190-223; GMC_AABB_TIGHT: exact box */
+    float aabb_threshold;   /* lbvh/Config.h:9, default 0.001f */
+} gmc_bvh_config;
+
+/* Bytes of the opaque BVH object for `shape` (nodes, boxes, sorted orders, build scratch). */
+size_t gmc_bvh_bytes(const gmc_shape* shape);
+/* Builds one LBVH per (b,l) mixture into `bvh` (gmc_bvh_bytes bytes) and, when `xes` is not NULL, a
+ * Morton order of the query points of every (bx,lx) so that wavefronts traverse coherent point tiles. */
+int gmc_bvh_build(const void* mixture, const void* xes, void* bvh, size_t bvh_bytes, const gmc_shape* shape,
+                  const gmc_bvh_config* config, void* stream);
+/* Copies the per-Gaussian boxes out of a built BVH: lower [B][L][M][D], upper [B][L][M][D] (component order). */
+int gmc_bvh_export_boxes(const void* bvh, void* lower, void* upper, const gmc_shape* shape, void* stream);
+/* Tree invariants for tests: nodes [B][L][2M-1][4] int32 = (parent, left, right, component or -1), internal
+ * nodes first, and node boxes [B][L][2M-1][2*D] (lower, upper). */
+int gmc_bvh_export_nodes(const void* bvh, int32_t* nodes, void* node_boxes, const gmc_shape* shape, void* stream);
+
+int gmc_eval_bvh_fwd(const void* mixture, const void* xes, const void* bvh, void* out, const gmc_shape* shape,
+                     void* stream);
+int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh,
+                     void* grad_mixture, void* grad_xes, void* workspace, size_t workspace_bytes,
+                     const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GMC_HIP_H */

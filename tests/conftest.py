@@ -1,3 +1,4 @@
+import math
 import os
 import sys
 
@@ -14,11 +15,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
-def rel_l2(a, b) -> float:
-    """relative L2 error ||a - b|| / ||b|| (b is the reference); 0 if both vanish"""
+def rel_l2(a, b, floor: float = 0.0) -> float:
+    """relative L2 error ||a - b|| / ||b|| (b is the reference); 0 if both vanish.  `floor` is an absolute
+    per-element magnitude below which the reference counts as zero: results that underflow in float32
+    (a Gaussian evaluated 15 sigma away is 1e-50 in float64 and 0 in float32) are not relative errors."""
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)
-    nb = np.linalg.norm(b)
+    nb = max(np.linalg.norm(b), floor * math.sqrt(max(b.size, 1)))
     na = np.linalg.norm(a - b)
     if nb == 0.0:
         return 0.0 if na == 0.0 else float("inf")

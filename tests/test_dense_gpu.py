@@ -1,0 +1,238 @@
+"""Parity of the dense HIP path (through the C ABI, via the gmc.mixture API) against the CPU oracle.
+Tolerances: relative L2 <= 1e-5 (float32) and <= 1e-12 (float64) per output tensor."""
+import itertools
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import cpu_ref
+import gm_oracle as o
+from conftest import rel_l2
+from gmc import mixture as gm
+from gmc import synthetic
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.float64: 1e-12}
+# magnitudes below these count as zero (float32 flushes them, the float64 oracle does not)
+FLOOR = {torch.float32: 1e-30, torch.float64: 1e-290}
+DEV = "cuda:0"
+
+
+def _run(mix_np, xes_np, gout_np, dtype, need_m=True, need_x=True):
+    mix = torch.tensor(mix_np, dtype=dtype, device=DEV, requires_grad=need_m)
+    xes = torch.tensor(xes_np, dtype=dtype, device=DEV, requires_grad=need_x)
+    out = gm.evaluate_inversed(mix, xes)
+    out.backward(torch.tensor(gout_np, dtype=dtype, device=DEV))
+    torch.cuda.synchronize()
+    gmix = mix.grad.cpu().numpy() if need_m else None
+    gxes = xes.grad.cpu().numpy() if need_x else None
+    return out.detach().cpu().numpy(), gmix, gxes
+
+
+def _case(B, L, M, N, D, seed, broadcast):
+    g = torch.Generator().manual_seed(seed)
+    mix = synthetic.random_inversed_mixture(B, L, M, D, g, dtype=torch.float64).numpy()
+    shape = (1, 1, N, D) if broadcast else (B, L, N, D)
+    xes = (torch.rand(shape, generator=g, dtype=torch.float64) * 20 - 10).numpy()
+    gout = torch.randn((B, L, N), generator=g, dtype=torch.float64).numpy()
+    return mix, xes, gout
+
+
+def _check(mix, xes, gout, dtype, tag=""):
+    # the oracle sees exactly the values the device sees (rounded to dtype first)
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    mix, xes, gout = mix.astype(npdt), xes.astype(npdt), gout.astype(npdt)
+    out, gmix, gxes = _run(mix, xes, gout, dtype)
+    ref = o.evaluate_inversed(mix, xes)
+    rgm, rgx = o.evaluate_inversed_backward(gout, mix, xes)
+    tol, fl = TOL[dtype], FLOOR[dtype]
+    D = xes.shape[-1]
+    assert out.shape == ref.shape and gmix.shape == rgm.shape and gxes.shape == rgx.shape
+    assert rel_l2(out, ref, fl) <= tol, f"forward {tag}"
+    assert rel_l2(gmix[..., 0], rgm[..., 0], fl) <= tol, f"grad weights {tag}"
+    assert rel_l2(gmix[..., 1:1 + D], rgm[..., 1:1 + D], fl) <= tol, f"grad positions {tag}"
+    assert rel_l2(gmix[..., 1 + D:], rgm[..., 1 + D:], fl) <= tol, f"grad inverse covariances {tag}"
+    assert rel_l2(gxes, rgx, fl) <= tol, f"grad xes {tag}"
+
+
+def test_known_answer(golden_dir):
+    data = json.load(open(os.path.join(golden_dir, "support_collections.json")))["known_answer"]
+    for dtype, tol in ((torch.float32, 1e-7), (torch.float64, 1e-15)):
+        mix = torch.tensor(data["mixture"], dtype=dtype, device=DEV).view(1, 1, 1, 7)
+        x = torch.tensor(data["x"], dtype=dtype, device=DEV).view(1, 1, 1, 2)
+        assert abs(gm.evaluate_inversed(mix, x).item() - data["value"]) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_sweep_like_reference_tests(dtype, D):
+    """shape sweep of src/gmc/test_cpp_eval.py:29-44,66-95 (forward and backward, full and broadcast xes)"""
+    seed = 100
+    for B, L, M, N in itertools.product((1, 5), (1, 4), (1, 6, 17, 50), (1, 8, 23, 50)):
+        for broadcast in (False, True):
+            seed += 1
+            mix, xes, gout = _case(B, L, M, N, D, seed, broadcast)
+            _check(mix, xes, gout, dtype, tag=f"B{B} L{L} M{M} N{N} D{D} bc{broadcast}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_tile_and_chunk_boundaries(dtype, D):
+    """component counts around the 256-wide LDS tile, point counts around the 256*P chunk sizes"""
+    seed = 500
+    for M, N in ((255, 257), (256, 2048), (257, 2049), (513, 300), (700, 4100)):
+        seed += 1
+        mix, xes, gout = _case(2, 1, M, N, D, seed, False)
+        _check(mix, xes, gout, dtype, tag=f"M{M} N{N} D{D}")
+    mix, xes, gout = _case(3, 2, 300, 1000, D, seed + 1, True)
+    _check(mix, xes, gout, dtype, tag="broadcast large")
+
+
+@pytest.mark.parametrize("D", [2, 3])
+def test_reference_literal_collections(golden_dir, D):
+    """the literal Gaussians / points of unittests/support.h:68-183 (weights 0, identity and skewed matrices)"""
+    data = json.load(open(os.path.join(golden_dir, "support_collections.json")))
+    covs = [data["cov_identity"], data["cov_2I_minus_half"]] + data["cov_sym6_xx_xy_xz_yy_yz_zz"]
+    rows = []
+    for w, p, c in itertools.product(data["gaussian_weights"] + data["gaussian_weights2"], data["gaussian_positions"], covs):
+        xx, xy, xz, yy, yz, zz = c
+        m = np.array([[xx, xy, xz], [xy, yy, yz], [xz, yz, zz]])[:D, :D]
+        rows.append(np.concatenate([[w], np.array(p[:D]), m.reshape(-1)]))
+    mix = np.stack(rows).reshape(1, 1, len(rows), -1)
+    xes = np.array(data["vec_collection"], dtype=np.float64)[:, :D].reshape(1, 1, -1, D)
+    for s in data["scalar_collection"][:5]:
+        gout = np.full((1, 1, xes.shape[2]), s)
+        for dtype in (torch.float32, torch.float64):
+            _check(mix, xes, gout, dtype, tag=f"literal D{D} g{s}")
+
+
+def test_need_flags_and_zero_grads():
+    mix, xes, gout = _case(2, 2, 9, 40, 3, 900, False)
+    out, gmix, gxes = _run(mix, xes, gout, torch.float64, need_m=True, need_x=False)
+    rgm, rgx = o.evaluate_inversed_backward(gout, mix, xes)
+    assert gxes is None and rel_l2(gmix, rgm) < 1e-12
+    out, gmix, gxes = _run(mix, xes, gout, torch.float64, need_m=False, need_x=True)
+    assert gmix is None and rel_l2(gxes, rgx) < 1e-12
+    # the raw binding returns both tensors, zero-filled when not required (parallel_implementation.cu:120-121)
+    from gmc.cpp.extensions.evaluate_inversed import evaluate_inversed as ei
+    m = torch.tensor(mix, device=DEV)
+    x = torch.tensor(xes, device=DEV)
+    g = torch.tensor(gout, device=DEV)
+    gm_, gx_ = ei.bindings.parallel_backward(g, m, x, (), False, True)
+    assert gm_.shape == m.shape and not gm_.any().item() and rel_l2(gx_.cpu().numpy(), rgx) < 1e-12
+    gm_, gx_ = ei.bindings.parallel_backward(g, m, x, (), True, False)
+    assert gx_.shape == x.shape and not gx_.any().item() and rel_l2(gm_.cpu().numpy(), rgm) < 1e-12
+
+
+def test_empty_inputs():
+    for M, N in ((0, 5), (4, 0), (0, 0)):
+        mix = torch.zeros(2, 3, M, 13, device=DEV, requires_grad=True)
+        xes = torch.zeros(2, 3, N, 3, device=DEV, requires_grad=True)
+        out = gm.evaluate_inversed(mix, xes)
+        assert out.shape == (2, 3, N) and not out.any().item()
+        out.sum().backward()
+        assert mix.grad.shape == mix.shape and not mix.grad.any().item()
+        assert xes.grad.shape == xes.shape and not xes.grad.any().item()
+
+
+@pytest.mark.parametrize("D", [2, 3])
+def test_gradcheck_fp64(D):
+    """src/gmc/test_cpp_eval.py:97-132: B=3, L=5, M=7, N=11, eps 1e-6, atol 1e-3, nondet_tol 1e-6"""
+    g = torch.Generator().manual_seed(7)
+    cov = synthetic.random_inversed_mixture(3, 5, 7, D, g, cov_radius=40.0, dtype=torch.float64)
+    xes = (torch.rand((3, 5, 11, D), generator=g, dtype=torch.float64) * 20 - 10)
+    mix = cov.to(DEV).requires_grad_(True)
+    x = xes.to(DEV).requires_grad_(True)
+    assert torch.autograd.gradcheck(gm.evaluate_inversed, (mix, x), eps=1e-6, atol=1e-3, nondet_tol=1e-6)
+
+
+def test_evaluate_covariance_form(golden_dir):
+    """src/gmc/test_mixture.py:31-56 through gm.evaluate (inversion + repack + evaluation), 5 places"""
+    data = json.load(open(os.path.join(golden_dir, "support_collections.json")))
+    rng = np.random.default_rng(5)
+    for D in (2, 3):
+        covs = np.stack([np.array(data["triangle_A"])[:D, :D], np.array(data["triangle_B"])[:D, :D]])
+        w = rng.random(2) * 2 - 1
+        pos = rng.random((2, D)) * 10 - 5
+        mix = gm.pack_mixture(torch.tensor(w, dtype=torch.float32).view(1, 1, 2),
+                              torch.tensor(pos, dtype=torch.float32).view(1, 1, 2, D),
+                              torch.tensor(covs, dtype=torch.float32).view(1, 1, 2, D, D)).to(DEV)
+        x = rng.random((50, D))
+        got = gm.evaluate(mix, torch.tensor(x, dtype=torch.float32, device=DEV).view(1, 1, 50, D)).cpu().numpy().reshape(-1)
+        ref = o.evaluate(mix.cpu().numpy().astype(np.float64), x.astype(np.float32).reshape(1, 1, 50, D)).reshape(-1)
+        assert np.abs(got - ref).max() < 1e-5 * 0.5
+        assert rel_l2(got, ref) < 1e-5
+
+
+def _workload_check(name, **kw):
+    wl, mix, xes, gout = synthetic.make_workload(name, **kw)
+    out, gmix, gxes = _run(mix.numpy(), xes.numpy(), gout.numpy(), wl.dtype)
+    # checker: the C restatement of the reference CPU path in float64 on the same (already rounded) inputs
+    m64, x64, g64 = (t.numpy().astype(np.float64) for t in (mix, xes, gout))
+    ref = cpu_ref.forward(m64, x64, n_threads=16)
+    rgm, rgx = cpu_ref.backward(g64, m64, x64, n_threads=16)
+    tol = TOL[wl.dtype]
+    D = wl.dims
+    errs = dict(out=rel_l2(out, ref), gw=rel_l2(gmix[..., 0], rgm[..., 0]), gb=rel_l2(gmix[..., 1:1 + D], rgm[..., 1:1 + D]),
+                gc=rel_l2(gmix[..., 1 + D:], rgm[..., 1 + D:]), gx=rel_l2(gxes, rgx))
+    print(name, kw, errs, flush=True)
+    assert all(v <= tol for v in errs.values()), errs
+
+
+def test_workload_c1():
+    _workload_check("C1")
+
+
+def test_workload_c2():
+    _workload_check("C2", B=20)
+
+
+def test_workload_c3():
+    _workload_check("C3", B=4)
+
+
+def test_workload_c4_slice():
+    _workload_check("C4", B=1, L=4)
+
+
+def test_workload_c5_dense_slice():
+    _workload_check("C5", M=2048, N=4096)
+
+
+def test_c4_full_size_properties():
+    """size-independent checks at the full headline size: exact scaling with the weights, additivity over a
+    split of the components, and gradient linearity in the upstream gradient"""
+    wl, mix, xes, gout = synthetic.make_workload("C4")
+    mix, xes, gout = mix.to(DEV), xes.to(DEV), gout.to(DEV)
+    out = gm.evaluate_inversed(mix, xes)
+    m2 = mix.clone()
+    m2[..., 0] *= 2.0
+    assert torch.equal(gm.evaluate_inversed(m2, xes), out * 2.0)
+    half = wl.M // 2
+    parts = gm.evaluate_inversed(mix[:, :, :half].contiguous(), xes) + gm.evaluate_inversed(mix[:, :, half:].contiguous(), xes)
+    assert ((parts - out).norm() / out.norm()).item() < 1e-6
+    # spot check against the checker on two mixtures of the full tensor
+    for b, l in ((0, 0), (31, 63)):
+        ref = cpu_ref.forward(mix[b:b + 1, l:l + 1].cpu().numpy().astype(np.float64),
+                              xes[b:b + 1, l:l + 1].cpu().numpy().astype(np.float64), n_threads=16)
+        assert rel_l2(out[b:b + 1, l:l + 1].cpu().numpy(), ref) < 1e-5
+    mg = mix.clone().requires_grad_(True)
+    xg = xes.clone().requires_grad_(True)
+    gm.evaluate_inversed(mg, xg).backward(gout)
+    g1m, g1x = mg.grad.clone(), xg.grad.clone()
+    mg.grad = None
+    xg.grad = None
+    gm.evaluate_inversed(mg, xg).backward(gout * 2.0)
+    assert ((mg.grad - 2.0 * g1m).norm() / g1m.norm()).item() < 1e-6
+    assert torch.equal(xg.grad, 2.0 * g1x)
+    for b, l in ((3, 5),):
+        rgm, rgx = cpu_ref.backward(gout[b:b + 1, l:l + 1].cpu().numpy().astype(np.float64),
+                                    mix[b:b + 1, l:l + 1].cpu().numpy().astype(np.float64),
+                                    xes[b:b + 1, l:l + 1].cpu().numpy().astype(np.float64), n_threads=16)
+        assert rel_l2(g1m[b:b + 1, l:l + 1].cpu().numpy(), rgm) < 1e-5
+        assert rel_l2(g1x[b:b + 1, l:l + 1].cpu().numpy(), rgx) < 1e-5

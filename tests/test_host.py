@@ -1,0 +1,102 @@
+"""Host-side checks that need no GPU: the C ABI library loads and exports every declared symbol, and the Python
+boundary rejects bad inputs with RuntimeError before anything is launched (rules of
+src/gmc/cpp/extensions/util/mixture.h:37-45,107-127 and parallel_implementation.cu:113-117)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from conftest import ROOT
+from gmc import _native
+from gmc import mixture as gm
+from gmc.cpp.extensions.evaluate_inversed import evaluate_inversed as ei
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "gmc_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    names = sorted(set(re.findall(r"\b(gmc_[a-z0-9_]+)\s*\(", header)))
+    assert "gmc_eval_fwd" in names and "gmc_eval_bwd" in names and len(names) >= 5
+    lib = ctypes.CDLL(_native.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/gmc_hip.h but not exported"
+    assert _native.lib().gmc_abi_version() == _native.ABI_VERSION
+    assert _native.lib().gmc_error_string(0) == b"ok"
+    assert b"7 or 13" in _native.lib().gmc_error_string(-1)
+
+
+def test_c_abi_rejects_bad_shapes_without_launching():
+    lib = _native.lib()
+    S = _native.Shape
+    ok = S(2, 3, 4, 5, 3, 2, 3, 0)
+    assert lib.gmc_eval_bwd_workspace_bytes(ctypes.byref(ok)) == 2 * 3 * 4 * 10 * 4
+    assert lib.gmc_eval_bwd_workspace_bytes(ctypes.byref(S(2, 3, 4, 5, 2, 2, 3, 1))) == 2 * 3 * 4 * 6 * 8
+    null = ctypes.c_void_p(0)
+    assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(2, 3, 4, 5, 4, 2, 3, 0)), null) == -1
+    assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(2, 3, 4, 5, 3, 2, 3, 7)), null) == -2
+    assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(2, 3, 4, 5, 3, 3, 3, 0)), null) == -3
+    assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(2, 3, 4, -5, 3, 2, 3, 0)), null) == -3
+    assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(ok), null) == -4
+    assert lib.gmc_eval_fwd(null, null, null, None, null) == -4
+    assert lib.gmc_eval_bwd(null, null, null, null, null, null, 0, ctypes.byref(ok), 1, 1, null) == -4
+
+
+def test_python_boundary_errors():
+    m = torch.zeros(2, 3, 4, 13)
+    x = torch.zeros(2, 3, 5, 3)
+    with pytest.raises(RuntimeError, match="7 or 13"):
+        gm.evaluate_inversed(torch.zeros(2, 3, 4, 12), x)
+    with pytest.raises(RuntimeError, match="mixture must have 4 dimensions"):
+        gm.evaluate_inversed(torch.zeros(3, 4, 13), x)
+    with pytest.raises(RuntimeError, match="xes must have 4 dimensions"):
+        gm.evaluate_inversed(m, torch.zeros(3, 5, 3))
+    with pytest.raises(RuntimeError, match="same dtype"):
+        gm.evaluate_inversed(m, x.double())
+    with pytest.raises(RuntimeError, match="batch dimension"):
+        gm.evaluate_inversed(m, torch.zeros(3, 3, 5, 3))
+    with pytest.raises(RuntimeError, match="layer dimension"):
+        gm.evaluate_inversed(m, torch.zeros(2, 2, 5, 3))
+    with pytest.raises(RuntimeError, match="last dimension"):
+        gm.evaluate_inversed(m, torch.zeros(2, 3, 5, 2))
+    with pytest.raises(RuntimeError, match="float32 and float64"):
+        gm.evaluate_inversed(m.half(), x.half())
+    # there is no CPU implementation behind this boundary: host tensors are refused, never silently evaluated
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        gm.evaluate_inversed(m, x)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ei.bindings.parallel_forward(m, x.transpose(0, 1).contiguous().transpose(0, 1))
+
+
+def test_layout_helpers_roundtrip():
+    g = torch.Generator().manual_seed(1)
+    w = torch.rand(2, 3, 4, generator=g)
+    p = torch.rand(2, 3, 4, 3, generator=g)
+    c = torch.rand(2, 3, 4, 3, 3, generator=g)
+    m = gm.pack_mixture(w, p, c)
+    assert m.shape == (2, 3, 4, 13) and gm.n_dimensions(m) == 3
+    assert gm.n_batch(m) == 2 and gm.n_layers(m) == 3 and gm.n_components(m) == 4
+    assert torch.equal(gm.weights(m), w) and torch.equal(gm.positions(m), p) and torch.equal(gm.covariances(m), c)
+    assert torch.equal(gm.integrate(m), w.sum(-1))
+    amp = gm.convert_priors_to_amplitudes(gm.pack_mixture(w, p, c @ c.transpose(-1, -2) + torch.eye(3)))
+    back = gm.convert_amplitudes_to_priors(amp)
+    assert torch.allclose(gm.weights(back), w, atol=1e-6)
+
+
+def test_small_matrix_inverse_and_its_gradient():
+    from gmc import mat_tools
+    g = torch.Generator().manual_seed(2)
+    for d in (2, 3):
+        a = torch.rand(5, 4, d, d, generator=g, dtype=torch.float64)
+        a = a @ a.transpose(-1, -2) + torch.eye(d, dtype=torch.float64)
+        a.requires_grad_(True)
+        inv = mat_tools.inverse(a)
+        assert torch.allclose(inv, torch.linalg.inv(a.detach()), atol=1e-12)
+        # symmetric upstream gradient: -A^-1 g A^-1 is then the exact gradient
+        up = torch.rand(5, 4, d, d, generator=g, dtype=torch.float64)
+        up = up + up.transpose(-1, -2)
+        inv.backward(up)
+        a2 = a.detach().clone().requires_grad_(True)
+        torch.linalg.inv(a2).backward(up)
+        assert torch.allclose(a.grad, a2.grad, atol=1e-10)
