@@ -1,0 +1,142 @@
+#!/usr/bin/env python3
+"""Benchmark of the Gaussian-mixture evaluation path on one MI355X.
+
+A step is one forward plus one backward (both gradients) of `evaluate_inversed` over one synthetic batch of the
+named workload (default C4: 3-D, float32, B=32, L=64, M=512 Gaussians, N=8192 points per mixture, 8.59e9
+Gaussian-point pairs).  Inputs are resident in HBM before the timed region.  Prints ONE JSON line:
+  value            whole-step throughput, Gaussian-point pairs per second (forward + backward)
+  fwd / fwd_bwd    pairs per second and fraction of the FP32 vector peak at the contract flop counts
+                   (D=3: 20 flop per forward pair, 52 per backward pair; D=2: 12 / 30)
+  roofline         dominant kernel (the backward pair kernel), HIP-event time on the launch stream
+  cpu_baseline     the C/OpenMP restatement of the reference's CPU path on a bounded slice of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "gaussian-mixture-convolution-networks_amd"))
+
+FLOP_FWD = {2: 12, 3: 20}
+FLOP_BWD = {2: 30, 3: 52}
+PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}     # MI355X vector peaks
+
+
+def cpu_baseline(name: str, seconds_budget: float = 20.0):
+    """Times oracle/libcpu_ref.so (checker code, used here only as the reported CPU baseline)."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import cpu_ref
+    from gmc import synthetic
+    base = synthetic.WORKLOADS[name]
+    # bounded sample of the same distributions: one batch entry, a few layers
+    kw = dict(B=1) if name != "C5" else dict(N=2000)
+    wl, mix, xes, gout = synthetic.make_workload(name, **kw)
+    m, x, g = mix.numpy(), xes.numpy(), gout.numpy()
+    threads = 128                                    # the reference's own choice (parallel_start.h:94-99)
+    cores = len(os.sched_getaffinity(0))
+    cpu_ref.forward(m[:, :1], x[:, :1], n_threads=threads)       # warm-up (thread pool, page faults)
+    t0 = time.perf_counter()
+    cpu_ref.forward(m, x, n_threads=threads)
+    t_fwd = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    cpu_ref.backward(g, m, x, n_threads=threads)
+    t_bwd = time.perf_counter() - t0
+    return {
+        "value": wl.pairs / (t_fwd + t_bwd), "unit": "pairs/s (fwd+bwd)", "cores": cores, "threads": threads,
+        "kind": "port", "fwd_pairs_per_s": wl.pairs / t_fwd, "bwd_pairs_per_s": wl.pairs / t_bwd,
+        "sample": f"{name} slice B={wl.B} L={wl.L} M={wl.M} N={wl.N} ({wl.pairs:.3g} pairs), "
+                  f"fwd {t_fwd:.2f} s + bwd {t_bwd:.2f} s, C/OpenMP restatement of the reference CPU path",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (known HBM traffic) so that a counter run of "
+                         "this command holds the calibration kernel next to the evaluation kernels")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path runs on ONE GPU; --gpus N with N > 1 is not supported (nothing here uses a "
+              "second GPU; mixtures would shard over batch x layers without communication)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from gmc import _native, synthetic
+
+    wl, mix, xes, gout = synthetic.make_workload(args.workload)
+    dev = torch.device("cuda:0")
+    mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)
+    torch.cuda.synchronize()
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        out = _native.eval_fwd(mix, xes)
+        if ev:
+            ev[1].record()
+        gm_, gx_ = _native.eval_bwd(gout, mix, xes, True, True)
+        if ev:
+            ev[2].record()
+        return out, gm_, gx_
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(events[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    ms_step = wall * 1e3 / args.steps
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    D = wl.dims
+    dt = "f32" if wl.dtype == torch.float32 else "f64"
+    peak = PEAK_TFLOPS[dt]
+    fwd_tf = FLOP_FWD[D] * wl.pairs / (fwd_ms * 1e-3) / 1e12
+    bwd_tf = FLOP_BWD[D] * wl.pairs / (bwd_ms * 1e-3) / 1e12
+    step_tf = (FLOP_FWD[D] + FLOP_BWD[D]) * wl.pairs / (ms_step * 1e-3) / 1e12
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(f"eval_bwd_kernel:{args.workload}")
+
+    line = {
+        "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
+        "value": wl.pairs / (ms_step * 1e-3), "unit": "Gaussian-point pairs/s (forward + backward step)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
+        "config": {"workload": f"{wl.name}: D={D} {dt} B={wl.B} L={wl.L} M={wl.M} N={wl.N}, dense all-pairs, "
+                               f"{wl.pairs:.4g} pairs per step, forward + backward (grad mixture and grad xes)"},
+        "fwd": {"ms": fwd_ms, "pairs_per_s": wl.pairs / (fwd_ms * 1e-3), "tflops": fwd_tf, "frac_of_peak": fwd_tf / peak},
+        "fwd_bwd": {"ms": ms_step, "pairs_per_s": wl.pairs / (ms_step * 1e-3), "tflops": step_tf,
+                    "frac_of_peak": step_tf / peak},
+        "roofline": {"kernel": "eval_bwd_kernel (backward pair kernel; its zero-fill and epilogue launches, <1% of "
+                               "the time, are inside the event pair)",
+                     "bound": "valu", "achieved": bwd_tf, "peak": peak, "unit": "TFLOP/s", "frac": bwd_tf / peak,
+                     "traffic": traffic, "launch_ms": bwd_ms, "flop_per_pair": FLOP_BWD[D]},
+        "roofline_fwd": {"kernel": "eval_fwd_kernel", "bound": "valu", "achieved": fwd_tf, "peak": peak,
+                         "unit": "TFLOP/s", "frac": fwd_tf / peak, "launch_ms": fwd_ms, "flop_per_pair": FLOP_FWD[D]},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
