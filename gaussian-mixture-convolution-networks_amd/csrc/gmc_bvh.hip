@@ -1,0 +1,983 @@
+// LBVH-culled Gaussian-mixture evaluation for gfx950.
+//
+// Semantics (what the reference's parts define; the composed evaluator is not in the reference snapshot):
+//   every Gaussian gets an axis-aligned box from the contribution cutoff (src/gmc/cpp/extensions/lbvh/bvh.cu:164-231);
+//   a point receives the contributions of exactly those Gaussians whose own box contains it (closed interval,
+//   lbvh/aabb.h:39-47; traversal lbvh/query.h:13-66).  Internal boxes are exact unions of their children
+//   (lbvh/bvh.cu:460-510), so the result does not depend on tree shape, Morton resolution or sort order.
+//
+// Build, one tree per (b,l) mixture, all on device and without host synchronisation:
+//   boxes + centre bounds -> 30-bit Morton codes of the centres (lbvh/morton_code.h:77-85,145-168) -> segmented LSD
+//   radix sort (8 bits per pass, stable, keys uint32 + index payload) -> leaves in Morton order with their
+//   evaluation records -> Karras radix tree over the unique keys (morton << 32 | rank), as lbvh/building.h:11-103
+//   -> bottom-up union of boxes with one visit counter per internal node.
+// Query points are Morton-sorted the same way so that a wavefront owns 64 neighbouring points.
+//
+// Traversal: one wavefront per 64 sorted points, ONE stack per wavefront (LDS).  A node is entered when any
+// lane's point lies in its box (ballot); node data is wave-uniform; at a leaf every lane evaluates the Gaussian
+// and lanes outside the leaf's own box add zero, which reproduces the per-point rule exactly.  Backward reduces
+// the per-Gaussian sums over the wavefront and issues one atomic per scalar, leaf visit and wavefront.
+#include "gmc_common.h"
+
+namespace gmc {
+
+int check_shape(const gmc_shape* s);
+
+constexpr int kStackDepth = 80;         // the radix tree over 64-bit unique keys is at most 64 levels deep
+constexpr double kSqFloor = 5.991464547107982;   // -2 ln 0.05 (lbvh/bvh.cu:194)
+
+// ---------------------------------------------------------------------------------------------------------------
+// layout of the opaque BVH object
+// ---------------------------------------------------------------------------------------------------------------
+struct BvhLayout {
+    size_t box_lo, box_hi;      // T [BL][M][D]            per-Gaussian boxes, component order
+    size_t node_box;            // T [BL][2M-1][2D]        lower, upper; internal nodes first, then leaves (Morton order)
+    size_t leaf_rec;            // T [BL][M][RS]           evaluation records in leaf order
+    size_t children;            // int2 [BL][M-1]          left, right: >= 0 internal node, < 0 leaf ~index
+    size_t parent;              // int [BL][2M-1]
+    size_t leaf_comp;           // int [BL][M]             component id of each leaf
+    size_t visit;               // int [BL][M-1]           arrival counters of the bottom-up pass
+    size_t g_bounds;            // T [BL][2D]              bounds of the centres
+    size_t p_bounds;            // T [BxLx][2D]            bounds of the query points
+    size_t keys_a, keys_b, vals_a, vals_b;   // uint32 [max(BL*M, BxLx*N)] radix ping-pong
+    size_t hist;                // uint32 [segments][256][blocks]
+    size_t p_order;             // int [BxLx][N]           Morton order of the query points
+    size_t g_keys;              // uint32 [BL][M]          sorted Morton codes of the leaves
+    size_t total;
+};
+
+constexpr int kSortItems = 8;                       // items per lane and radix block
+constexpr int kSortChunk = kBlock * kSortItems;     // 2048
+
+template <int D> struct LeafRec { static constexpr int kStride = (D == 2) ? 8 : 12; };
+// D=3: b0 b1 b2 c00 c01 c02 c11 c12 c22 amp comp -   D=2: b0 b1 c00 c01 c11 amp comp -
+
+static size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
+
+static BvhLayout bvh_layout(const gmc_shape& s) {
+    const size_t e = s.dtype == GMC_F32 ? 4 : 8;
+    const size_t BL = size_t(s.B) * s.L, XL = size_t(s.Bx) * s.Lx;
+    const size_t M = s.M, N = s.N, D = s.D;
+    const size_t nodes = M > 0 ? 2 * M - 1 : 0;
+    const size_t rs = s.D == 2 ? LeafRec<2>::kStride : LeafRec<3>::kStride;
+    BvhLayout l;
+    size_t o = 0;
+    auto take = [&](size_t bytes) { const size_t at = o; o = align_up(o + bytes); return at; };
+    l.box_lo = take(BL * M * D * e);
+    l.box_hi = take(BL * M * D * e);
+    l.node_box = take(BL * nodes * 2 * D * e);
+    l.leaf_rec = take(BL * M * rs * e);
+    l.children = take(BL * (M > 0 ? M - 1 : 0) * 8);
+    l.parent = take(BL * nodes * 4);
+    l.leaf_comp = take(BL * M * 4);
+    l.visit = take(BL * (M > 0 ? M - 1 : 0) * 4);
+    l.g_bounds = take(BL * 2 * D * e);
+    l.p_bounds = take(XL * 2 * D * e);
+    const size_t items = BL * M > XL * N ? BL * M : XL * N;
+    l.keys_a = take(items * 4);
+    l.keys_b = take(items * 4);
+    l.vals_a = take(items * 4);
+    l.vals_b = take(items * 4);
+    const size_t bg = BL * ((M + kSortChunk - 1) / kSortChunk), bp = XL * ((N + kSortChunk - 1) / kSortChunk);
+    l.hist = take((bg > bp ? bg : bp) * 256 * 4);
+    l.p_order = take(XL * N * 4);
+    l.g_keys = take(BL * M * 4);
+    l.total = o;
+    return l;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// per-Gaussian boxes
+// ---------------------------------------------------------------------------------------------------------------
+
+// Symmetric eigen-decomposition as the reference's device functions define it (math/symeig_detail.h:17-72 for
+// 2x2, :75-138 for 3x3), restated here because the "reference" box rule is a function of ITS outputs, quirks
+// included (absolute 1e-7 test for "diagonal", identity vectors when the off-diagonal is exactly zero).
+// lam[j]: values in the reference's output order; v[i][j]: j-th component of the i-th vector.
+__device__ inline void ref_symeig2(const double a[2][2], double lam[2], double v[2][2]) {
+    const double tr = a[0][0] + a[1][1];
+    const double det = a[0][0] * a[1][1] - a[0][1] * a[1][0];
+    const double aa = a[0][0], bb = a[0][1], dd = a[1][1];
+    const double f1 = tr / 2.0, f2 = sqrt(fabs(tr * tr / 4.0 - det));
+    lam[0] = f1 - f2;
+    lam[1] = f1 + f2;
+    if (bb == 0.0) {
+        v[0][0] = 1.0; v[0][1] = 0.0; v[1][0] = 0.0; v[1][1] = 1.0;
+        return;
+    }
+    double e0[2], e1[2];
+    if (aa < dd) { e0[0] = bb; e0[1] = lam[0] - aa; e1[0] = bb; e1[1] = lam[1] - aa; }
+    else         { e0[0] = lam[0] - dd; e0[1] = bb; e1[0] = lam[1] - dd; e1[1] = bb; }
+    const double n0 = sqrt(e0[0] * e0[0] + e0[1] * e0[1]), n1 = sqrt(e1[0] * e1[0] + e1[1] * e1[1]);
+    v[0][0] = e0[0] / n0; v[0][1] = e0[1] / n0;
+    v[1][0] = e1[0] / n1; v[1][1] = e1[1] / n1;
+}
+
+// longest column of the symmetric matrix p, normalised; false if every column vanishes
+__device__ inline bool longest_column(const double p[3][3], double out[3]) {
+    double best = 0.0;
+    int idx = -1;
+    for (int j = 0; j < 3; ++j) {
+        const double len = p[0][j] * p[0][j] + p[1][j] * p[1][j] + p[2][j] * p[2][j];
+        if (len > best) { best = len; idx = j; }
+    }
+    if (idx < 0) return false;
+    const double inv = 1.0 / sqrt(best);
+    for (int i = 0; i < 3; ++i) out[i] = p[i][idx] * inv;
+    return true;
+}
+
+__device__ inline void shifted_product(const double a[3][3], double s1, double s2, double p[3][3]) {
+    double x[3][3], y[3][3];
+    for (int i = 0; i < 3; ++i)
+        for (int j = 0; j < 3; ++j) {
+            x[i][j] = a[i][j] - (i == j ? s1 : 0.0);
+            y[i][j] = a[i][j] - (i == j ? s2 : 0.0);
+        }
+    for (int i = 0; i < 3; ++i)
+        for (int j = 0; j < 3; ++j) p[i][j] = x[i][0] * y[0][j] + x[i][1] * y[1][j] + x[i][2] * y[2][j];
+}
+
+__device__ inline bool ref_symeig3(const double a[3][3], double lam[3], double v[3][3]) {
+    const double kPi = 3.14159265358979323846;
+    double eig0, eig1, eig2;
+    const double p1 = a[0][1] * a[0][1] + a[0][2] * a[0][2] + a[1][2] * a[1][2];
+    if (p1 <= 0.0000001) {
+        eig0 = a[0][0]; eig1 = a[1][1]; eig2 = a[2][2];
+    } else {
+        const double q = (a[0][0] + a[1][1] + a[2][2]) / 3.0;
+        const double p2 = (a[0][0] - q) * (a[0][0] - q) + (a[1][1] - q) * (a[1][1] - q) + (a[2][2] - q) * (a[2][2] - q) + 2.0 * p1;
+        const double p = sqrt(p2 / 6.0);
+        double b[3][3];
+        for (int i = 0; i < 3; ++i)
+            for (int j = 0; j < 3; ++j) b[i][j] = (a[i][j] - (i == j ? q : 0.0)) / p;
+        const double detb = b[0][0] * (b[1][1] * b[2][2] - b[1][2] * b[2][1]) - b[0][1] * (b[1][0] * b[2][2] - b[1][2] * b[2][0]) +
+                            b[0][2] * (b[1][0] * b[2][1] - b[1][1] * b[2][0]);
+        const double r = detb / 2.0;
+        double phi;
+        if (r <= -1.0) phi = kPi / 3.0;
+        else if (r >= 1.0) phi = 0.0;
+        else phi = acos(r) / 3.0;
+        eig0 = q + 2.0 * p * cos(phi);
+        eig2 = q + 2.0 * p * cos(phi + 2.0 * kPi / 3.0);
+        eig1 = 3.0 * q - eig0 - eig2;
+    }
+    double pm[3][3], v0[3], v1[3];
+    shifted_product(a, eig1, eig2, pm);
+    if (!longest_column(pm, v0)) return false;
+    shifted_product(a, eig0, eig2, pm);
+    if (!longest_column(pm, v1)) return false;
+    lam[0] = eig2; lam[1] = eig1; lam[2] = eig0;
+    v[0][0] = v0[1] * v1[2] - v0[2] * v1[1];
+    v[0][1] = v0[2] * v1[0] - v0[0] * v1[2];
+    v[0][2] = v0[0] * v1[1] - v0[1] * v1[0];
+    for (int j = 0; j < 3; ++j) { v[1][j] = v1[j]; v[2][j] = v0[j]; }
+    return true;
+}
+
+// half extents of the cutoff box of one Gaussian (record g: weight, position, inverse covariance)
+template <typename T, int D>
+__device__ inline void box_half_extent(const T* __restrict__ g, double threshold, int mode, double* delta) {
+    const double w = fabs(double(g[0]));
+    double s2 = -2.0 * log(threshold / w);
+    s2 = fmax(s2, kSqFloor);
+    const double s = sqrt(s2);
+    const T* c = g + 1 + D;
+    double sigma[D][D];
+    // the reference inverts the stored matrix read column-major, i.e. C^T (util/glm.h:108-128)
+    if constexpr (D == 2) {
+        const double m00 = c[0], m01 = c[2], m10 = c[1], m11 = c[3];
+        const double det = m00 * m11 - m01 * m10;
+        sigma[0][0] = m11 / det; sigma[0][1] = -m01 / det; sigma[1][0] = -m10 / det; sigma[1][1] = m00 / det;
+    } else {
+        double m[3][3];
+        for (int i = 0; i < 3; ++i)
+            for (int j = 0; j < 3; ++j) m[i][j] = double(c[j * 3 + i]);
+        const double c00 = m[1][1] * m[2][2] - m[1][2] * m[2][1];
+        const double c01 = m[1][2] * m[2][0] - m[1][0] * m[2][2];
+        const double c02 = m[1][0] * m[2][1] - m[1][1] * m[2][0];
+        const double det = m[0][0] * c00 + m[0][1] * c01 + m[0][2] * c02;
+        sigma[0][0] = c00 / det;
+        sigma[1][0] = c01 / det;
+        sigma[2][0] = c02 / det;
+        sigma[0][1] = (m[0][2] * m[2][1] - m[0][1] * m[2][2]) / det;
+        sigma[1][1] = (m[0][0] * m[2][2] - m[0][2] * m[2][0]) / det;
+        sigma[2][1] = (m[0][1] * m[2][0] - m[0][0] * m[2][1]) / det;
+        sigma[0][2] = (m[0][1] * m[1][2] - m[0][2] * m[1][1]) / det;
+        sigma[1][2] = (m[0][2] * m[1][0] - m[0][0] * m[1][2]) / det;
+        sigma[2][2] = (m[0][0] * m[1][1] - m[0][1] * m[1][0]) / det;
+    }
+    double tight[D];
+    for (int k = 0; k < D; ++k) tight[k] = sqrt(fmax(sigma[k][k], 0.0));
+    bool literal = (mode == GMC_AABB_REFERENCE);
+    double lit[D];
+    if (literal) {
+        double lam[D], v[D][D];
+        if constexpr (D == 2) ref_symeig2(sigma, lam, v);
+        else literal = ref_symeig3(sigma, lam, v);
+        if (literal) {
+            for (int k = 0; k < D; ++k) {
+                double acc = 0.0;
+                for (int j = 0; j < D; ++j) acc += lam[j] * v[k][j] * v[k][j];
+                lit[k] = sqrt(acc);
+                if (!(lit[k] == lit[k]) || isinf(lit[k])) literal = false;   // undefined rule -> tight box
+            }
+        }
+    }
+    for (int k = 0; k < D; ++k) delta[k] = s * (literal ? lit[k] : tight[k]);
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
+                                                          T* __restrict__ box_hi, size_t n, double threshold, int mode) {
+    constexpr int G = 1 + D + D * D;
+    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const T* g = mixture + i * G;
+    double delta[D];
+    box_half_extent<T, D>(g, threshold, mode, delta);
+    for (int k = 0; k < D; ++k) {
+        box_lo[i * D + k] = T(double(g[1 + k]) - delta[k]);
+        box_hi[i * D + k] = T(double(g[1 + k]) + delta[k]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// bounds of a point set, Morton keys
+// ---------------------------------------------------------------------------------------------------------------
+
+// one workgroup per segment: bounds[seg] = (min_0..min_D-1, max_0..max_D-1) over `count` points of stride `stride`
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bounds_kernel(const T* __restrict__ pts, int stride, int offset, int count,
+                                                       T* __restrict__ bounds) {
+    __shared__ T red[2 * D][kBlock];
+    const size_t seg = blockIdx.x;
+    const T* p = pts + seg * size_t(count) * stride + offset;
+    T lo[D], hi[D];
+    for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
+    for (int i = threadIdx.x; i < count; i += kBlock)
+        for (int d = 0; d < D; ++d) {
+            const T v = p[size_t(i) * stride + d];
+            lo[d] = v < lo[d] ? v : lo[d];
+            hi[d] = v > hi[d] ? v : hi[d];
+        }
+    for (int d = 0; d < D; ++d) { red[d][threadIdx.x] = lo[d]; red[D + d][threadIdx.x] = hi[d]; }
+    __syncthreads();
+    for (int s = kBlock / 2; s > 0; s >>= 1) {
+        if (int(threadIdx.x) < s)
+            for (int d = 0; d < D; ++d) {
+                const T a = red[d][threadIdx.x + s], b = red[D + d][threadIdx.x + s];
+                if (a < red[d][threadIdx.x]) red[d][threadIdx.x] = a;
+                if (b > red[D + d][threadIdx.x]) red[D + d][threadIdx.x] = b;
+            }
+        __syncthreads();
+    }
+    if (threadIdx.x < 2 * D) bounds[seg * 2 * D + threadIdx.x] = red[threadIdx.x][0];
+}
+
+__device__ __forceinline__ uint32_t expand_bits3(uint32_t v) {
+    v = (v * 0x00010001u) & 0xFF0000FFu;
+    v = (v * 0x00000101u) & 0x0F00F00Fu;
+    v = (v * 0x00000011u) & 0xC30C30C3u;
+    v = (v * 0x00000005u) & 0x49249249u;
+    return v;
+}
+
+// 10 bits per axis of the position normalised by `bounds`; an axis of zero extent maps to cell 0
+template <typename T, int D>
+__device__ __forceinline__ uint32_t morton30(const T* __restrict__ p, const T* __restrict__ bounds) {
+    uint32_t code = 0;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        const double lo = double(bounds[d]), ext = double(bounds[D + d]) - lo;
+        double q = ext > 0.0 ? (double(p[d]) - lo) / ext * 1024.0 : 0.0;
+        q = q < 0.0 ? 0.0 : (q > 1023.0 ? 1023.0 : q);
+        q = (q == q) ? q : 0.0;
+        code |= expand_bits3(uint32_t(q)) << (2 - d);
+    }
+    return code;
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void morton_kernel(const T* __restrict__ pts, int stride, int offset, int count,
+                                                       const T* __restrict__ bounds, uint32_t* __restrict__ keys,
+                                                       uint32_t* __restrict__ vals, size_t total) {
+    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const size_t seg = i / count;
+    keys[i] = morton30<T, D>(pts + i * stride + offset, bounds + seg * 2 * D);
+    vals[i] = uint32_t(i - seg * count);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// segmented LSD radix sort, 8 bits per pass, stable; segments of equal length `count`
+// ---------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void radix_hist_kernel(const uint32_t* __restrict__ keys, int count, int blocks_per_seg,
+                                                           int shift, uint32_t* __restrict__ hist) {
+    __shared__ uint32_t h[256];
+    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    h[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t* k = keys + size_t(seg) * count;
+    const int begin = blk * kSortChunk;
+    const int end = begin + kSortChunk < count ? begin + kSortChunk : count;
+    for (int i = begin + threadIdx.x; i < end; i += kBlock) atomicAdd(&h[(k[i] >> shift) & 255u], 1u);
+    __syncthreads();
+    // digit-major layout so that one exclusive scan over (digit, block) yields the scatter offsets
+    hist[(size_t(seg) * 256 + threadIdx.x) * blocks_per_seg + blk] = h[threadIdx.x];
+}
+
+__global__ __launch_bounds__(kBlock) void radix_scan_kernel(uint32_t* __restrict__ hist, int blocks_per_seg) {
+    __shared__ uint32_t totals[256];
+    uint32_t* h = hist + (size_t(blockIdx.x) * 256 + threadIdx.x) * blocks_per_seg;
+    uint32_t run = 0;
+    for (int b = 0; b < blocks_per_seg; ++b) { const uint32_t c = h[b]; h[b] = run; run += c; }
+    totals[threadIdx.x] = run;
+    __syncthreads();
+    // exclusive scan of the 256 digit totals (Hillis-Steele on LDS)
+    uint32_t mine = run;
+    for (int off = 1; off < 256; off <<= 1) {
+        const uint32_t add = int(threadIdx.x) >= off ? totals[threadIdx.x - off] : 0u;
+        __syncthreads();
+        totals[threadIdx.x] += add;
+        __syncthreads();
+    }
+    const uint32_t base = totals[threadIdx.x] - mine;
+    for (int b = 0; b < blocks_per_seg; ++b) h[b] += base;
+}
+
+__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const uint32_t* __restrict__ keys_in,
+                                                              const uint32_t* __restrict__ vals_in,
+                                                              uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
+                                                              int count, int blocks_per_seg, int shift,
+                                                              const uint32_t* __restrict__ hist) {
+    __shared__ uint32_t running[256];        // next output slot of every digit for this block
+    __shared__ uint32_t wave_count[4][256];
+    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    running[threadIdx.x] = hist[(size_t(seg) * 256 + threadIdx.x) * blocks_per_seg + blk];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) wave_count[w][threadIdx.x] = 0;
+    __syncthreads();
+    const size_t seg_off = size_t(seg) * count;
+    const int begin = blk * kSortChunk;
+    for (int round = 0; round < kSortItems; ++round) {
+        const int i = begin + round * kBlock + threadIdx.x;
+        const bool valid = i < count && i < begin + kSortChunk;
+        uint32_t key = 0, val = 0, digit = 0;
+        if (valid) { key = keys_in[seg_off + i]; val = vals_in[seg_off + i]; digit = (key >> shift) & 255u; }
+        // lanes of this wavefront holding the same digit
+        unsigned long long same = __ballot(valid);
+#pragma unroll
+        for (int bit = 0; bit < 8; ++bit) {
+            const unsigned long long b = __ballot((digit >> bit) & 1u);
+            same &= ((digit >> bit) & 1u) ? b : ~b;
+        }
+        const int rank = __popcll(same & ((1ull << lane) - 1ull));
+        if (valid && rank == 0) wave_count[wave][digit] = uint32_t(__popcll(same));
+        __syncthreads();
+        if (valid) {
+            uint32_t slot = running[digit] + rank;
+            for (int w = 0; w < wave; ++w) slot += wave_count[w][digit];
+            if (slot < uint32_t(count)) {          // always true for a consistent histogram; keeps a bug from writing out of bounds
+                keys_out[seg_off + slot] = key;
+                vals_out[seg_off + slot] = val;
+            }
+        }
+        __syncthreads();
+        {
+            uint32_t add = 0;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) { add += wave_count[w][threadIdx.x]; wave_count[w][threadIdx.x] = 0; }
+            running[threadIdx.x] += add;
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// leaves, radix tree, bottom-up boxes
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, const T* __restrict__ box_lo,
+                                                           const T* __restrict__ box_hi, const uint32_t* __restrict__ order,
+                                                           T* __restrict__ node_box, T* __restrict__ leaf_rec,
+                                                           int* __restrict__ leaf_comp, int* __restrict__ visit,
+                                                           int* __restrict__ parent, int M, size_t total) {
+    constexpr int G = 1 + D + D * D;
+    constexpr int RS = LeafRec<D>::kStride;
+    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const size_t bl = i / M;
+    const int leaf = int(i - bl * M);
+    int comp = int(order[i]);
+    comp = (comp >= 0 && comp < M) ? comp : 0;      // a permutation by construction; never index out of bounds
+    const size_t gi = bl * M + comp;
+    const size_t node = bl * (2 * size_t(M) - 1) + (M - 1) + leaf;
+    for (int d = 0; d < D; ++d) {
+        node_box[node * 2 * D + d] = box_lo[gi * D + d];
+        node_box[node * 2 * D + D + d] = box_hi[gi * D + d];
+    }
+    leaf_comp[i] = comp;
+    if (leaf < M - 1) visit[bl * (M - 1) + leaf] = 0;
+    if (M == 1) parent[node] = -1;                  // a single leaf is its own root
+    const T* g = mixture + gi * G;
+    T* r = leaf_rec + i * RS;
+    const T* c = g + 1 + D;
+    for (int d = 0; d < D; ++d) r[d] = g[1 + d];
+    if constexpr (D == 2) {
+        const double det = double(c[0]) * double(c[3]) - double(c[1]) * double(c[2]);
+        r[2] = c[0]; r[3] = T(0.5 * (double(c[1]) + double(c[2]))); r[4] = c[3];
+        r[5] = T(double(g[0]) * Kappa<2>::v * sqrt(det));
+        reinterpret_cast<int*>(r + 6)[0] = comp;
+    } else {
+        const double c00 = c[0], c01 = c[1], c02 = c[2], c10 = c[3], c11 = c[4], c12 = c[5], c20 = c[6], c21 = c[7], c22 = c[8];
+        const double det = c00 * (c11 * c22 - c12 * c21) - c01 * (c10 * c22 - c12 * c20) + c02 * (c10 * c21 - c11 * c20);
+        r[3] = T(c00); r[4] = T(0.5 * (c01 + c10)); r[5] = T(0.5 * (c02 + c20));
+        r[6] = T(c11); r[7] = T(0.5 * (c12 + c21)); r[8] = T(c22);
+        r[9] = T(double(g[0]) * Kappa<3>::v * sqrt(det));
+        reinterpret_cast<int*>(r + 10)[0] = comp;
+    }
+}
+
+// number of leading bits shared by the unique keys (morton[i] << 32 | i) and (morton[j] << 32 | j); -1 outside
+__device__ __forceinline__ int common_prefix(const uint32_t* __restrict__ keys, int n, int i, int j) {
+    if (j < 0 || j >= n) return -1;
+    const uint32_t a = keys[i], b = keys[j];
+    if (a != b) return __clz(a ^ b);
+    return 32 + __clz(uint32_t(i) ^ uint32_t(j));
+}
+
+__global__ __launch_bounds__(kBlock) void bvh_tree_kernel(const uint32_t* __restrict__ keys, int2* __restrict__ children,
+                                                         int* __restrict__ parent, int M, size_t total) {
+    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= total) return;
+    const int n_int = M - 1;
+    const size_t bl = t / n_int;
+    const int i = int(t - bl * n_int);
+    const uint32_t* k = keys + bl * M;
+    // range of keys covered by internal node i
+    int first, last;
+    if (i == 0) { first = 0; last = M - 1; }
+    else {
+        const int dl = common_prefix(k, M, i, i - 1), dr = common_prefix(k, M, i, i + 1);
+        const int dir = dr > dl ? 1 : -1;
+        const int dmin = dr > dl ? dl : dr;
+        int lmax = 2;
+        while (common_prefix(k, M, i, i + lmax * dir) > dmin) lmax <<= 1;
+        int len = 0;
+        for (int step = lmax >> 1; step > 0; step >>= 1)
+            if (common_prefix(k, M, i, i + (len + step) * dir) > dmin) len += step;
+        const int j = i + len * dir;
+        first = i < j ? i : j;
+        last = i < j ? j : i;
+    }
+    // split: the highest key that shares more than the node's prefix with the first key
+    const int dnode = common_prefix(k, M, first, last);
+    int split = first, stride = last - first;
+    do {
+        stride = (stride + 1) >> 1;
+        const int mid = split + stride;
+        if (mid < last && common_prefix(k, M, first, mid) > dnode) split = mid;
+    } while (stride > 1);
+    const int left = (split == first) ? ~split : split;               // leaf `split` or internal node `split`
+    const int right = (split + 1 == last) ? ~(split + 1) : split + 1;
+    children[t] = make_int2(left, right);
+    int* par = parent + bl * (2 * size_t(M) - 1);
+    par[left >= 0 ? left : (M - 1) + ~left] = i;
+    par[right >= 0 ? right : (M - 1) + ~right] = i;
+    if (i == 0) par[0] = -1;
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int2* __restrict__ children, const int* __restrict__ parent,
+                                                          T* node_box, int* visit, int M, size_t total) {
+    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= total) return;
+    const size_t bl = t / M;
+    const int leaf = int(t - bl * M);
+    const size_t nbase = bl * (2 * size_t(M) - 1);
+    T* boxes = node_box + nbase * 2 * D;
+    int node = parent[nbase + (M - 1) + leaf];
+    // a leaf is at most M - 1 levels below the root; the bound also ends the walk on a malformed parent chain
+    for (int level = 0; node >= 0 && node < M - 1 && level < M; ++level) {
+        __threadfence();                                   // publish this lane's box before announcing arrival
+        if (atomicAdd(&visit[bl * (M - 1) + node], 1) == 0) return;   // first arrival: the sibling will finish
+        __threadfence();
+        const int2 ch = children[bl * (M - 1) + node];
+        const int l = ch.x >= 0 ? ch.x : (M - 1) + ~ch.x, r = ch.y >= 0 ? ch.y : (M - 1) + ~ch.y;
+        // child boxes were written by other lanes; the fence pair around the counter orders them before these loads
+        for (int d = 0; d < D; ++d) {
+            const T a = boxes[size_t(l) * 2 * D + d];
+            const T b = boxes[size_t(r) * 2 * D + d];
+            const T c = boxes[size_t(l) * 2 * D + D + d];
+            const T e = boxes[size_t(r) * 2 * D + D + d];
+            boxes[size_t(node) * 2 * D + d] = a < b ? a : b;
+            boxes[size_t(node) * 2 * D + D + d] = c > e ? c : e;
+        }
+        node = parent[nbase + node];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// traversal
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T, int D>
+__device__ __forceinline__ bool inside_box(const T (&x)[D], const T* __restrict__ box) {
+    bool in = true;
+#pragma unroll
+    for (int d = 0; d < D; ++d) in = in && !(x[d] < box[d]) && !(x[d] > box[D + d]) && (x[d] == x[d]);
+    return in;
+}
+
+__device__ __forceinline__ float exp_neg_half(float q) { return __builtin_amdgcn_exp2f(q * -0.72134752044448170368f); }
+__device__ __forceinline__ double exp_neg_half(double q) { return exp(-0.5 * q); }
+
+// e = exp(-1/2 t^T C t), u = C t for the leaf record r
+template <typename T, int D>
+__device__ __forceinline__ T leaf_terms(const T* __restrict__ r, const T (&x)[D], T (&t)[D], T (&u)[D]) {
+    if constexpr (D == 2) {
+        t[0] = x[0] - r[0]; t[1] = x[1] - r[1];
+        u[0] = fma_(r[2], t[0], r[3] * t[1]);
+        u[1] = fma_(r[3], t[0], r[4] * t[1]);
+        return exp_neg_half(fma_(t[0], u[0], t[1] * u[1]));
+    } else {
+        t[0] = x[0] - r[0]; t[1] = x[1] - r[1]; t[2] = x[2] - r[2];
+        u[0] = fma_(r[3], t[0], fma_(r[4], t[1], r[5] * t[2]));
+        u[1] = fma_(r[4], t[0], fma_(r[6], t[1], r[7] * t[2]));
+        u[2] = fma_(r[5], t[0], fma_(r[7], t[1], r[8] * t[2]));
+        return exp_neg_half(fma_(t[0], u[0], fma_(t[1], u[1], t[2] * u[2])));
+    }
+}
+
+template <int D> struct BvhSums { static constexpr int k = 1 + D + D * (D + 1) / 2; };
+
+// MODE 0: forward.  MODE 1: backward (grad_out given; accumulates per-Gaussian sums and dL/dx).
+template <typename T, int D, int MODE, bool NEED_GM, bool NEED_GX>
+__global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
+        const T* __restrict__ xes, const int* __restrict__ p_order, const T* __restrict__ node_box,
+        const int2* __restrict__ children, const T* __restrict__ leaf_rec, T* __restrict__ out,
+        const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes,
+        int L, int M, int N, int Bx, int Lx, int chunks, int xes_shared) {
+    constexpr int RS = LeafRec<D>::kStride;
+    constexpr int NR = BvhSums<D>::k;
+    __shared__ int stack_mem[kBlock / kWave][kStackDepth];
+    const int bl = blockIdx.x / chunks;
+    const int chunk = blockIdx.x - bl * chunks;
+    const int b = bl / L, l = bl - b * L;
+    const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
+    const size_t xseg = size_t(xb) * Lx + xl;
+    const int wave = threadIdx.x >> 6;
+    int* stack = stack_mem[wave];
+
+    const int j = chunk * kBlock + threadIdx.x;
+    const bool valid = j < N;
+    const int pid = valid ? p_order[xseg * N + j] : 0;
+    T x[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) x[d] = xes[(xseg * N + pid) * D + d];
+    T g = T(0);
+    if (MODE == 1) g = valid ? grad_out[size_t(bl) * N + pid] : T(0);
+
+    const T* boxes = node_box + size_t(bl) * (2 * size_t(M) - 1) * 2 * D;
+    const int2* kids = children + size_t(bl) * (M - 1);
+    const T* recs = leaf_rec + size_t(bl) * M * RS;
+    T acc = T(0);
+    T gx[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) gx[d] = T(0);
+
+    auto visit_leaf = [&](int leaf, bool in) {
+        const T* r = recs + size_t(leaf) * RS;
+        T t[D], u[D];
+        const T e = leaf_terms<T, D>(r, x, t, u);
+        const T amp = r[D + D * (D + 1) / 2];
+        if (MODE == 0) {
+            acc += in ? amp * e : T(0);
+        } else {
+            const T eg = in ? e * g : T(0);
+            if (NEED_GX) {
+                const T s = in ? amp * e : T(0);
+#pragma unroll
+                for (int d = 0; d < D; ++d) gx[d] = fma_(s, u[d], gx[d]);
+            }
+            if (NEED_GM) {
+                T rs[NR];
+                rs[0] = eg;
+#pragma unroll
+                for (int d = 0; d < D; ++d) rs[1 + d] = eg * t[d];
+                int k = 1 + D;
+#pragma unroll
+                for (int a = 0; a < D; ++a)
+#pragma unroll
+                    for (int c = a; c < D; ++c) rs[k++] = rs[1 + a] * t[c];
+#pragma unroll
+                for (int i = 0; i < NR; ++i) rs[i] = wave_sum_to_lane63(rs[i]);
+                if ((threadIdx.x & 63) == 63) {
+                    const int comp = reinterpret_cast<const int*>(r + D + D * (D + 1) / 2 + 1)[0];
+                    T* dst = sums + (size_t(bl) * M + comp) * NR;
+#pragma unroll
+                    for (int i = 0; i < NR; ++i) atomic_add(&dst[i], rs[i]);
+                }
+            }
+        }
+    };
+
+    if (M == 1) {
+        const bool in = valid && inside_box<T, D>(x, boxes);
+        if (__ballot(in) != 0ull) visit_leaf(0, in);
+    } else {
+        int sp = 0;
+        stack[sp++] = 0;
+        // every iteration pops one node; a binary tree with M-1 internal nodes bounds the loop
+        for (int iter = 0; sp > 0 && iter < M; ++iter) {
+            const int node = __builtin_amdgcn_readfirstlane(stack[--sp]);
+            const int2 ch = kids[node];
+            const int c0 = __builtin_amdgcn_readfirstlane(ch.x), c1 = __builtin_amdgcn_readfirstlane(ch.y);
+#pragma unroll
+            for (int side = 0; side < 2; ++side) {
+                const int c = side == 0 ? c0 : c1;
+                if (c >= M - 1 || ~c >= M) continue;                 // not a node of this tree
+                const int cnode = c >= 0 ? c : (M - 1) + ~c;
+                const bool in = valid && inside_box<T, D>(x, boxes + size_t(cnode) * 2 * D);
+                if (__ballot(in) != 0ull) {
+                    if (c < 0) visit_leaf(~c, in);
+                    else if (sp < kStackDepth) stack[sp++] = c;
+                }
+            }
+        }
+    }
+
+    if (MODE == 0) {
+        if (valid) out[size_t(bl) * N + pid] = acc;
+    } else if (NEED_GX) {
+        if (valid) {
+            T* dst = grad_xes + (xseg * N + pid) * D;
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                const T v = -g * gx[d];
+                if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
+            }
+        }
+    }
+}
+
+// (R0, sum r t, sum r t t^T) -> (dw, db, dC); see the dense epilogue for the formulas (here y = t, u = identity)
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __restrict__ mixture, const T* __restrict__ sums,
+                                                                 T* __restrict__ grad_mixture, size_t n) {
+    constexpr int G = 1 + D + D * D;
+    constexpr int NR = BvhSums<D>::k;
+    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const T* g = mixture + i * G;
+    const T* rs = sums + i * NR;
+    T* o = grad_mixture + i * G;
+    const double w = double(g[0]);
+    double c[D][D];
+    for (int r = 0; r < D; ++r)
+        for (int q = 0; q < D; ++q) c[r][q] = double(g[1 + D + r * D + q]);
+    double det;
+    if constexpr (D == 2) det = c[0][0] * c[1][1] - c[0][1] * c[1][0];
+    else det = c[0][0] * (c[1][1] * c[2][2] - c[1][2] * c[2][1]) - c[0][1] * (c[1][0] * c[2][2] - c[1][2] * c[2][0]) +
+               c[0][2] * (c[1][0] * c[2][1] - c[1][1] * c[2][0]);
+    const double root = sqrt(det);
+    const double norm = Kappa<D>::v * root;
+    const double R0 = double(rs[0]);
+    o[0] = T(norm * R0);
+    double r1[D];
+    for (int d = 0; d < D; ++d) r1[d] = double(rs[1 + d]);
+    for (int r = 0; r < D; ++r) {
+        double acc = 0.0;
+        for (int q = 0; q < D; ++q) acc += 0.5 * (c[r][q] + c[q][r]) * r1[q];
+        o[1 + r] = T(w * norm * acc);
+    }
+    double s2[D][D];
+    int k = 1 + D;
+    for (int a = 0; a < D; ++a)
+        for (int q = a; q < D; ++q) { s2[a][q] = double(rs[k]); s2[q][a] = double(rs[k]); ++k; }
+    const double kd = w * Kappa<D>::v * R0 / (2.0 * root);
+    for (int r = 0; r < D; ++r)
+        for (int q = 0; q < D; ++q) {
+            double cof;
+            if constexpr (D == 2) {
+                cof = (r == q) ? c[1 - r][1 - q] : -c[q][r];
+            } else {
+                const int r1i = r == 0 ? 1 : 0, r2i = r == 2 ? 1 : 2, q1 = q == 0 ? 1 : 0, q2 = q == 2 ? 1 : 2;
+                cof = (((r + q) & 1) ? -1.0 : 1.0) * (c[r1i][q1] * c[r2i][q2] - c[r1i][q2] * c[r2i][q1]);
+            }
+            o[1 + D + r * D + q] = T(-0.5 * w * norm * s2[r][q] + cof * kd);
+        }
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void export_nodes_kernel(const int2* __restrict__ children, const int* __restrict__ parent,
+                                                             const int* __restrict__ leaf_comp, int32_t* __restrict__ nodes,
+                                                             int M, size_t total) {
+    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= total) return;
+    const size_t n_nodes = 2 * size_t(M) - 1;
+    const size_t bl = t / n_nodes;
+    const int node = int(t - bl * n_nodes);
+    int32_t* o = nodes + t * 4;
+    o[0] = parent[t];
+    if (node < M - 1) {
+        const int2 ch = children[bl * (M - 1) + node];
+        o[1] = ch.x >= 0 ? ch.x : (M - 1) + ~ch.x;
+        o[2] = ch.y >= 0 ? ch.y : (M - 1) + ~ch.y;
+        o[3] = -1;
+    } else {
+        o[1] = -1; o[2] = -1;
+        o[3] = leaf_comp[bl * M + (node - (M - 1))];
+    }
+}
+
+template <typename T>
+__global__ void copy_kernel(const T* __restrict__ src, T* __restrict__ dst, size_t n) {
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+
+__global__ void iota_segments_kernel(int* __restrict__ dst, int count, size_t total) {
+    const size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < total) dst[i] = int(i % count);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------------------------
+static unsigned grid_for(size_t n) { return unsigned((n + kBlock - 1) / kBlock); }
+
+// sorts `segments` segments of `count` (key, value) pairs held in (ka, va) on bits [0, 8*passes); returns 0 if the
+// result is in the a buffers, 1 if in the b buffers
+static int radix_sort(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* hist, int segments, int count,
+                      int passes, hipStream_t st) {
+    const int bps = (count + kSortChunk - 1) / kSortChunk;
+    const dim3 grid(unsigned(size_t(segments) * bps));
+    int cur = 0;
+    for (int p = 0; p < passes; ++p) {
+        uint32_t* kin = cur ? kb : ka; uint32_t* vin = cur ? vb : va;
+        uint32_t* kout = cur ? ka : kb; uint32_t* vout = cur ? va : vb;
+        radix_hist_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, count, bps, 8 * p, hist);
+        radix_scan_kernel<<<dim3(unsigned(segments)), dim3(kBlock), 0, st>>>(hist, bps);
+        radix_scatter_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, vin, kout, vout, count, bps, 8 * p, hist);
+        cur ^= 1;
+    }
+    return cur;
+}
+
+template <typename T, int D>
+static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shape& s, const gmc_bvh_config& cfg,
+                       hipStream_t st) {
+    constexpr int G = 1 + D + D * D;
+    const BvhLayout lay = bvh_layout(s);
+    const size_t BL = size_t(s.B) * s.L, XL = size_t(s.Bx) * s.Lx;
+    const int M = s.M, N = s.N;
+    T* box_lo = (T*)(bvh + lay.box_lo); T* box_hi = (T*)(bvh + lay.box_hi);
+    T* node_box = (T*)(bvh + lay.node_box); T* leaf_rec = (T*)(bvh + lay.leaf_rec);
+    int2* children = (int2*)(bvh + lay.children); int* parent = (int*)(bvh + lay.parent);
+    int* leaf_comp = (int*)(bvh + lay.leaf_comp); int* visit = (int*)(bvh + lay.visit);
+    uint32_t* ka = (uint32_t*)(bvh + lay.keys_a); uint32_t* kb = (uint32_t*)(bvh + lay.keys_b);
+    uint32_t* va = (uint32_t*)(bvh + lay.vals_a); uint32_t* vb = (uint32_t*)(bvh + lay.vals_b);
+    uint32_t* hist = (uint32_t*)(bvh + lay.hist);
+    if (BL > 0 && M > 0) {
+        const size_t n = BL * M;
+        bvh_boxes_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, n,
+                                                                          double(cfg.aabb_threshold), cfg.aabb_mode);
+        T* gb = (T*)(bvh + lay.g_bounds);
+        bounds_kernel<T, D><<<dim3(unsigned(BL)), dim3(kBlock), 0, st>>>(mixture, G, 1, M, gb);
+        morton_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, G, 1, M, gb, ka, va, n);
+        const int where = radix_sort(ka, va, kb, vb, hist, int(BL), M, 4, st);
+        uint32_t* g_keys = (uint32_t*)(bvh + lay.g_keys);
+        copy_kernel<uint32_t><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(where ? kb : ka, g_keys, n);
+        bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, where ? vb : va, node_box,
+                                                                           leaf_rec, leaf_comp, visit, parent, M, n);
+        if (M > 1) {
+            const size_t ni = BL * (M - 1);
+            bvh_tree_kernel<<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(g_keys, children, parent, M, ni);
+            bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(children, parent, node_box, visit, M, n);
+        }
+    }
+    if (XL > 0 && N > 0) {
+        int* p_order = (int*)(bvh + lay.p_order);
+        const size_t n = XL * N;
+        if (xes) {
+            T* pb = (T*)(bvh + lay.p_bounds);
+            bounds_kernel<T, D><<<dim3(unsigned(XL)), dim3(kBlock), 0, st>>>(xes, D, 0, N, pb);
+            morton_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(xes, D, 0, N, pb, ka, va, n);
+            const int where = radix_sort(ka, va, kb, vb, hist, int(XL), N, 4, st);
+            copy_kernel<uint32_t><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(
+                where ? vb : va, (uint32_t*)p_order, n);
+        } else {
+            iota_segments_kernel<<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(p_order, N, n);
+        }
+    }
+    return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
+
+template <typename T, int D>
+static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, hipStream_t st) {
+    const BvhLayout lay = bvh_layout(s);
+    const size_t BL = size_t(s.B) * s.L;
+    if (BL == 0 || s.N == 0) return GMC_OK;
+    if (s.M == 0) {
+        const size_t n = BL * s.N;
+        fill_zero_kernel<T><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(out, n);
+        return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+    }
+    const int chunks = (s.N + kBlock - 1) / kBlock;
+    bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kBlock), 0, st>>>(
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const int2*)(bvh + lay.children),
+        (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N, s.Bx, s.Lx, chunks, 0);
+    return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
+
+template <typename T, int D>
+static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, const char* bvh, T* grad_mixture, T* grad_xes,
+                     T* sums, const gmc_shape& s, bool gm, bool gx, hipStream_t st) {
+    constexpr int G = 1 + D + D * D;
+    constexpr int NR = BvhSums<D>::k;
+    const BvhLayout lay = bvh_layout(s);
+    const size_t BL = size_t(s.B) * s.L;
+    const size_t n_g = BL * s.M, n_x = size_t(s.Bx) * s.Lx * s.N * D;
+    const int xes_shared = (s.Bx != s.B || s.Lx != s.L) ? 1 : 0;
+    auto zero = [&](T* p, size_t n) {
+        if (n) fill_zero_kernel<T><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(p, n);
+    };
+    if (BL == 0) return GMC_OK;
+    if (s.N == 0 || s.M == 0) {
+        if (gm) zero(grad_mixture, n_g * G);
+        if (gx) zero(grad_xes, n_x);
+        return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+    }
+    if (gm) zero(sums, n_g * NR);
+    if (gx && xes_shared) zero(grad_xes, n_x);
+    const int chunks = (s.N + kBlock - 1) / kBlock;
+    const dim3 grid(unsigned(BL * chunks));
+#define GMC_TRAV(GM, GX) bvh_traverse_kernel<T, D, 1, GM, GX><<<grid, dim3(kBlock), 0, st>>>( \
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const int2*)(bvh + lay.children), \
+        (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared)
+    if (gm && gx) GMC_TRAV(true, true);
+    else if (gm) GMC_TRAV(true, false);
+    else if (gx) GMC_TRAV(false, true);
+#undef GMC_TRAV
+    if (gm) bvh_bwd_epilogue_kernel<T, D><<<dim3(grid_for(n_g)), dim3(kBlock), 0, st>>>(mixture, sums, grad_mixture, n_g);
+    return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
+
+template <typename T, int D>
+static int bvh_export_t(const char* bvh, T* lower, T* upper, int32_t* nodes, T* node_boxes, const gmc_shape& s,
+                        hipStream_t st) {
+    const BvhLayout lay = bvh_layout(s);
+    const size_t BL = size_t(s.B) * s.L;
+    const size_t n = BL * s.M * D;
+    auto copy = [&](const T* src, T* dst, size_t cnt) {
+        if (cnt) copy_kernel<T><<<dim3(grid_for(cnt) < 4096 ? grid_for(cnt) : 4096), dim3(kBlock), 0, st>>>(src, dst, cnt);
+    };
+    if (lower) copy((const T*)(bvh + lay.box_lo), lower, n);
+    if (upper) copy((const T*)(bvh + lay.box_hi), upper, n);
+    if (s.M > 0) {
+        const size_t nn = BL * (2 * size_t(s.M) - 1);
+        if (nodes && nn)
+            export_nodes_kernel<T, D><<<dim3(grid_for(nn)), dim3(kBlock), 0, st>>>(
+                (const int2*)(bvh + lay.children), (const int*)(bvh + lay.parent), (const int*)(bvh + lay.leaf_comp), nodes,
+                s.M, nn);
+        if (node_boxes) copy((const T*)(bvh + lay.node_box), node_boxes, nn * 2 * D);
+    }
+    return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
+
+}  // namespace gmc
+
+extern "C" {
+
+size_t gmc_bvh_bytes(const gmc_shape* shape) {
+    if (gmc::check_shape(shape) != GMC_OK) return 0;
+    return gmc::bvh_layout(*shape).total;
+}
+
+static int check_bvh_shape(const gmc_shape* shape) {
+    const int rc = gmc::check_shape(shape);
+    if (rc != GMC_OK) return rc;
+    // leaf indices are stored bit-inverted in an int, traversal loop counters are ints
+    if (shape->M > (1 << 30) || shape->N > (1 << 30)) return GMC_E_SHAPE;
+    return GMC_OK;
+}
+
+int gmc_bvh_build(const void* mixture, const void* xes, void* bvh, size_t bvh_bytes, const gmc_shape* shape,
+                  const gmc_bvh_config* config, void* stream) {
+    const int rc = check_bvh_shape(shape);
+    if (rc != GMC_OK) return rc;
+    if (!config) return GMC_E_NULL;
+    if (config->aabb_mode != GMC_AABB_REFERENCE && config->aabb_mode != GMC_AABB_TIGHT) return GMC_E_CONFIG;
+    if (!(config->aabb_threshold > 0.0f)) return GMC_E_CONFIG;
+    const size_t need = gmc::bvh_layout(*shape).total;
+    if (need == 0) return GMC_OK;
+    if (!bvh) return GMC_E_NULL;
+    if (bvh_bytes < need) return GMC_E_WORKSPACE;
+    if (!mixture && size_t(shape->B) * shape->L * shape->M > 0) return GMC_E_NULL;
+#define ARGS(T) (const T*)mixture, (const T*)xes, (char*)bvh, *shape, *config, (hipStream_t)stream
+    if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_build_t<float, 2>(ARGS(float)) : gmc::bvh_build_t<float, 3>(ARGS(float));
+    return shape->D == 2 ? gmc::bvh_build_t<double, 2>(ARGS(double)) : gmc::bvh_build_t<double, 3>(ARGS(double));
+#undef ARGS
+}
+
+int gmc_bvh_export_boxes(const void* bvh, void* lower, void* upper, const gmc_shape* shape, void* stream) {
+    const int rc = check_bvh_shape(shape);
+    if (rc != GMC_OK) return rc;
+    if (size_t(shape->B) * shape->L * shape->M == 0) return GMC_OK;
+    if (!bvh || !lower || !upper) return GMC_E_NULL;
+#define ARGS(T) (const char*)bvh, (T*)lower, (T*)upper, (int32_t*)nullptr, (T*)nullptr, *shape, (hipStream_t)stream
+    if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_export_t<float, 2>(ARGS(float)) : gmc::bvh_export_t<float, 3>(ARGS(float));
+    return shape->D == 2 ? gmc::bvh_export_t<double, 2>(ARGS(double)) : gmc::bvh_export_t<double, 3>(ARGS(double));
+#undef ARGS
+}
+
+int gmc_bvh_export_nodes(const void* bvh, int32_t* nodes, void* node_boxes, const gmc_shape* shape, void* stream) {
+    const int rc = check_bvh_shape(shape);
+    if (rc != GMC_OK) return rc;
+    if (size_t(shape->B) * shape->L * shape->M == 0) return GMC_OK;
+    if (!bvh || !nodes || !node_boxes) return GMC_E_NULL;
+#define ARGS(T) (const char*)bvh, (T*)nullptr, (T*)nullptr, nodes, (T*)node_boxes, *shape, (hipStream_t)stream
+    if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_export_t<float, 2>(ARGS(float)) : gmc::bvh_export_t<float, 3>(ARGS(float));
+    return shape->D == 2 ? gmc::bvh_export_t<double, 2>(ARGS(double)) : gmc::bvh_export_t<double, 3>(ARGS(double));
+#undef ARGS
+}
+
+int gmc_eval_bvh_fwd(const void* mixture, const void* xes, const void* bvh, void* out, const gmc_shape* shape,
+                     void* stream) {
+    (void)mixture;   // the leaf records inside the BVH hold everything the forward pass needs
+    const int rc = check_bvh_shape(shape);
+    if (rc != GMC_OK) return rc;
+    if (size_t(shape->B) * shape->L * shape->N == 0) return GMC_OK;
+    if (!out || !xes || (!bvh && shape->M > 0)) return GMC_E_NULL;
+#define ARGS(T) (const T*)xes, (const char*)bvh, (T*)out, *shape, (hipStream_t)stream
+    if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_fwd_t<float, 2>(ARGS(float)) : gmc::bvh_fwd_t<float, 3>(ARGS(float));
+    return shape->D == 2 ? gmc::bvh_fwd_t<double, 2>(ARGS(double)) : gmc::bvh_fwd_t<double, 3>(ARGS(double));
+#undef ARGS
+}
+
+int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh, void* grad_mixture,
+                     void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
+                     int need_grad_mixture, int need_grad_xes, void* stream) {
+    const int rc = check_bvh_shape(shape);
+    if (rc != GMC_OK) return rc;
+    const bool gm = need_grad_mixture != 0, gx = need_grad_xes != 0;
+    if (!gm && !gx) return GMC_OK;
+    const size_t n_g = size_t(shape->B) * shape->L * shape->M;
+    const size_t n_x = size_t(shape->Bx) * shape->Lx * shape->N;
+    if (gm && n_g > 0 && !grad_mixture) return GMC_E_NULL;
+    if (gx && n_x > 0 && !grad_xes) return GMC_E_NULL;
+    if (n_g > 0 && n_x > 0 && (!grad_out || !mixture || !xes || !bvh)) return GMC_E_NULL;
+    if (gm && n_g > 0 && n_x > 0) {
+        const size_t need = n_g * (shape->D == 2 ? 6 : 10) * (shape->dtype == GMC_F32 ? 4 : 8);
+        if (workspace_bytes < need) return GMC_E_WORKSPACE;
+        if (!workspace) return GMC_E_NULL;
+    }
+#define ARGS(T) (const T*)grad_out, (const T*)mixture, (const T*)xes, (const char*)bvh, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, *shape, gm, gx, (hipStream_t)stream
+    if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_bwd_t<float, 2>(ARGS(float)) : gmc::bvh_bwd_t<float, 3>(ARGS(float));
+    return shape->D == 2 ? gmc::bvh_bwd_t<double, 2>(ARGS(double)) : gmc::bvh_bwd_t<double, 3>(ARGS(double));
+#undef ARGS
+}
+
+}  // extern "C"

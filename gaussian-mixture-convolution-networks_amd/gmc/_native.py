@@ -159,3 +159,84 @@ def eval_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool):
         check(lib().gmc_eval_bwd(_p(grad_output), _p(mixture), _p(xes), _p(grad_mixture), _p(grad_xes), _p(ws),
                                  ws_bytes, ctypes.byref(shape), int(need_mixture), int(need_xes), _stream(dev)))
     return grad_mixture, grad_xes
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# LBVH-culled variant
+# ---------------------------------------------------------------------------------------------------------------
+
+_AABB_MODES = {"reference": GMC_AABB_REFERENCE, "tight": GMC_AABB_TIGHT}
+
+
+def _bvh_config(aabb_threshold: float, aabb_mode: str) -> BvhConfigC:
+    if aabb_mode not in _AABB_MODES:
+        raise RuntimeError(f"unknown aabb_mode {aabb_mode!r}; expected 'reference' or 'tight'")
+    if not aabb_threshold > 0:
+        raise RuntimeError("aabb_threshold must be positive")
+    return BvhConfigC(_AABB_MODES[aabb_mode], float(aabb_threshold))
+
+
+class Bvh:
+    """One LBVH per (batch, layer) mixture plus the Morton order of the query points, as an opaque device blob."""
+
+    def __init__(self, mixture: torch.Tensor, xes: torch.Tensor, aabb_threshold: float = 0.001,
+                 aabb_mode: str = "reference"):
+        self.shape = check_input(mixture, xes)
+        cfg = _bvh_config(aabb_threshold, aabb_mode)
+        dev = mixture.device
+        with torch.cuda.device(dev):
+            nbytes = lib().gmc_bvh_bytes(ctypes.byref(self.shape))
+            self.blob = torch.empty((max(nbytes, 8),), dtype=torch.uint8, device=dev)
+            check(lib().gmc_bvh_build(_p(mixture), _p(xes), _p(self.blob), nbytes, ctypes.byref(self.shape),
+                                      ctypes.byref(cfg), _stream(dev)))
+        self.dtype, self.device = mixture.dtype, dev
+
+    def boxes(self):
+        """(lower, upper), each [B, L, M, D], in component order"""
+        s = self.shape
+        lo = torch.empty((s.B, s.L, s.M, s.D), dtype=self.dtype, device=self.device)
+        up = torch.empty_like(lo)
+        with torch.cuda.device(self.device):
+            check(lib().gmc_bvh_export_boxes(_p(self.blob), _p(lo), _p(up), ctypes.byref(s), _stream(self.device)))
+        return lo, up
+
+    def nodes(self):
+        """(nodes [B, L, 2M-1, 4] int32 = parent, left, right, component-or--1; node boxes [B, L, 2M-1, 2D])"""
+        s = self.shape
+        n = max(2 * s.M - 1, 0)
+        nodes = torch.empty((s.B, s.L, n, 4), dtype=torch.int32, device=self.device)
+        nb = torch.empty((s.B, s.L, n, 2 * s.D), dtype=self.dtype, device=self.device)
+        with torch.cuda.device(self.device):
+            check(lib().gmc_bvh_export_nodes(_p(self.blob), _p(nodes), _p(nb), ctypes.byref(s), _stream(self.device)))
+        return nodes, nb
+
+
+def eval_bvh_fwd(mixture, xes, bvh: Bvh) -> torch.Tensor:
+    shape = check_input(mixture, xes)
+    out = torch.empty((shape.B, shape.L, shape.N), dtype=mixture.dtype, device=mixture.device)
+    with torch.cuda.device(mixture.device):
+        check(lib().gmc_eval_bvh_fwd(_p(mixture), _p(xes), _p(bvh.blob), _p(out), ctypes.byref(shape),
+                                     _stream(mixture.device)))
+    return out
+
+
+def eval_bvh_bwd(grad_output, mixture, xes, bvh: Bvh, need_mixture: bool, need_xes: bool):
+    shape = check_input(mixture, xes)
+    if tuple(grad_output.shape) != (shape.B, shape.L, shape.N):
+        raise RuntimeError("grad_output has wrong shape")
+    if grad_output.dtype != mixture.dtype:
+        raise RuntimeError("grad_output dtype does not match with mixture dtype")
+    if not grad_output.is_contiguous():
+        raise RuntimeError("grad_output must be contiguous")
+    dev = mixture.device
+    grad_mixture = torch.empty_like(mixture) if need_mixture else torch.zeros_like(mixture)
+    grad_xes = torch.empty_like(xes) if need_xes else torch.zeros_like(xes)
+    if not (need_mixture or need_xes):
+        return grad_mixture, grad_xes
+    with torch.cuda.device(dev):
+        ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
+        ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
+        check(lib().gmc_eval_bvh_bwd(_p(grad_output), _p(mixture), _p(xes), _p(bvh.blob), _p(grad_mixture), _p(grad_xes),
+                                     _p(ws), ws_bytes, ctypes.byref(shape), int(need_mixture), int(need_xes),
+                                     _stream(dev)))
+    return grad_mixture, grad_xes
