@@ -114,7 +114,7 @@ def main():
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(f"eval_bwd_kernel:{args.workload}")
+        traffic = json.load(open(tpath)).get(f"eval_bwd_rc_kernel:{args.workload}")
 
     line = {
         "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
@@ -126,7 +126,7 @@ def main():
         "fwd": {"ms": fwd_ms, "pairs_per_s": wl.pairs / (fwd_ms * 1e-3), "tflops": fwd_tf, "frac_of_peak": fwd_tf / peak},
         "fwd_bwd": {"ms": ms_step, "pairs_per_s": wl.pairs / (ms_step * 1e-3), "tflops": step_tf,
                     "frac_of_peak": step_tf / peak},
-        "roofline": {"kernel": "eval_bwd_kernel (backward pair kernel; its zero-fill and epilogue launches, <1% of "
+        "roofline": {"kernel": "eval_bwd_rc_kernel (backward pair kernel; its zero-fill and epilogue launches, <1% of "
                                "the time, are inside the event pair)",
                      "bound": "valu", "achieved": bwd_tf, "peak": peak, "unit": "TFLOP/s", "frac": bwd_tf / peak,
                      "traffic": traffic, "launch_ms": bwd_ms, "flop_per_pair": FLOP_BWD[D]},

@@ -146,10 +146,13 @@ __device__ __forceinline__ T quad_form(const T* __restrict__ r, const T* __restr
 }
 
 // Stages up to 256 Gaussians (one per lane of a 256-lane workgroup) into LDS, shifted-form records first,
-// centred-form records after them (stable order within each group); counts[8] receives the number of shifted
-// records.  Contains two workgroup barriers: the first also orders the overwrite of the tile after every lane's
-// reads of the previous one, the second publishes the new tile, so the caller needs no barrier of its own.
-template <typename T, int D>
+// centred-form records after them (stable order within each group).  Each of the two groups is padded with null
+// records (zero factor and amplitude, index -1) to a multiple of GROUP, so that GROUP consecutive records always
+// share one form; the tile needs room for 256 + 2*(GROUP-1) records.  counts[8] receives the start of the
+// centred group, counts[9] the padded total.  Contains two workgroup barriers: the first also orders the
+// overwrite of the tile after every lane's reads of the previous one, the second publishes the new tile, so the
+// caller needs no barrier of its own.
+template <typename T, int D, int GROUP = 1>
 __device__ __forceinline__ void stage_tile(const T* __restrict__ gaussians, int cnt, double amp_scale, T* lds,
                                            int* counts /* LDS int[10] */) {
     constexpr int S = Rec<T, D>::kStride;
@@ -167,20 +170,36 @@ __device__ __forceinline__ void stage_tile(const T* __restrict__ gaussians, int 
     const unsigned long long ms = __ballot(active && !centred);
     if (lane == 0) { counts[wave] = __popcll(ms); counts[4 + wave] = __popcll(mc); }
     __syncthreads();
-    int shifted_before = 0, centred_before = 0, shifted_total = 0;
+    int shifted_before = 0, centred_before = 0, shifted_total = 0, centred_total = 0;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
         const int cs = counts[w], cc = counts[4 + w];
         if (w < wave) { shifted_before += cs; centred_before += cc; }
         shifted_total += cs;
+        centred_total += cc;
     }
+    const int centred_start = (shifted_total + GROUP - 1) / GROUP * GROUP;
+    const int centred_end = centred_start + centred_total;
+    const int padded_total = (centred_end + GROUP - 1) / GROUP * GROUP;
     if (active) {
         const unsigned long long below = (1ull << lane) - 1ull;
-        const int slot = centred ? shifted_total + centred_before + __popcll(mc & below)
+        const int slot = centred ? centred_start + centred_before + __popcll(mc & below)
                                  : shifted_before + __popcll(ms & below);
         store_record<T, D>(lds + slot * S, dv, centred, dv.w * dv.norm * amp_scale, tid);
     }
-    if (tid == 0) counts[8] = shifted_total;
+    if constexpr (GROUP > 1) {
+        // null records: y = 0, e = 1, amplitude 0 -> no contribution; index -1 -> their sums are dropped
+        int slot = -1;
+        if (tid < centred_start - shifted_total) slot = shifted_total + tid;
+        else if (tid >= GROUP && tid - GROUP < padded_total - centred_end) slot = centred_end + (tid - GROUP);
+        if (slot >= 0) {
+            T* rec = lds + slot * S;
+#pragma unroll
+            for (int i = 0; i < Rec<T, D>::kUsed; ++i) rec[i] = T(0);
+            reinterpret_cast<int*>(rec + Rec<T, D>::kIdx)[0] = -1;
+        }
+    }
+    if (tid == 0) { counts[8] = centred_start; counts[9] = padded_total; }
     __syncthreads();
 }
 
@@ -205,6 +224,24 @@ __device__ __forceinline__ double wave_sum_to_lane63(double v) {
     for (int off = 1; off < 64; off <<= 1) {
         const double o = __shfl_up(v, off, 64);
         if ((threadIdx.x & 63) >= off) v += o;
+    }
+    return v;
+}
+
+// ---- sum over the 16 lanes of a DPP row; the total arrives in lane 15 of the row ---------------------------
+__device__ __forceinline__ float row_sum_to_lane15(float v) {
+    v += dpp_mov<0x111>(v);
+    v += dpp_mov<0x112>(v);
+    v += dpp_mov<0x114>(v);
+    v += dpp_mov<0x118>(v);
+    return v;
+}
+
+__device__ __forceinline__ double row_sum_to_lane15(double v) {
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        const double o = __shfl_up(v, off, 16);
+        if ((threadIdx.x & 15) >= off) v += o;
     }
     return v;
 }

@@ -8,9 +8,10 @@
 //     inverse covariance, -u b, amplitude), so a pair costs D(D+1)/2 FMAs for y = u x - u b, D for |y|^2, one
 //     exp2 and one FMA, with no per-pair subtraction, determinant or square root; Gaussians that sit too far
 //     from the origin for that form (in units of their width) keep an explicit x - b instead;
-//   * backward keeps dL/dx per point in registers and reduces the 1 + D + D(D+1)/2 per-Gaussian sums over the
-//     wavefront (DPP), over the workgroup (LDS) and over workgroups (one atomic per scalar and workgroup);
-//     a per-Gaussian epilogue turns the sums into (dw, db, dC).
+//   * backward splits the wavefront into 4 rows of 16 lanes (rows = Gaussians, columns = points), keeps dL/dx per
+//     point in registers and reduces the 1 + D + D(D+1)/2 per-Gaussian sums over a DPP row, over the workgroup
+//     (LDS) and over workgroups (one atomic per scalar and workgroup); a per-Gaussian epilogue turns the sums
+//     into (dw, db, dC).
 #include "gmc_common.h"
 
 namespace gmc {
@@ -37,14 +38,18 @@ __device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, int begin, 
 template <typename T, int D, int P>
 __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ mixture, const T* __restrict__ xes,
                                                           T* __restrict__ out, int L, int M, int N, int Bx, int Lx,
-                                                          int chunks) {
+                                                          int chunks, int n_mixtures) {
     constexpr int G = 1 + D + D * D;
     constexpr int S = Rec<T, D>::kStride;
     __shared__ __attribute__((aligned(16))) T lds[kTile * S];
     __shared__ int counts[10];
 
-    const int bl = blockIdx.x / chunks;
-    const int chunk = blockIdx.x - bl * chunks;
+    // workgroups are dealt round-robin to the 8 XCDs; keep all point chunks of one mixture on one XCD so that
+    // its L2 serves the repeated reads of the Gaussians
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int bl = (slot / chunks) * 8 + xcd;
+    const int chunk = slot % chunks;
+    if (bl >= n_mixtures) return;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const T* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
@@ -80,12 +85,16 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
 //   R0 = sum_n e g,  R1_i = sum_n e g y_i,  R2_ij = sum_n e g y_i y_j (i <= j)     with e = exp2(-|y|^2)
 template <int D> struct Sums { static constexpr int k = 1 + D + D * (D + 1) / 2; };   // 6 / 10
 
+// Backward pair kernel, "4 x 16" wavefront layout.  The 64 lanes of a wavefront form 4 DPP rows of 16 lanes:
+// row r works on Gaussian 4k + r of the tile in step k, column c on the points {c, c + 16, ..., c + 16 (P-1)} of
+// the wavefront's 16 P points.  The per-Gaussian sums are then reduced over one DPP row only (4 shifts, no
+// cross-row traffic) once per step and Gaussian, and dL/dx is reduced over the 4 rows once per kernel.
 template <typename T, int D, int P, bool NEED_GM, bool NEED_GX, bool CENTRED>
-__device__ __forceinline__ void bwd_pairs(const T* __restrict__ lds, T* __restrict__ block_sums, int begin, int end,
-                                          const T (&x)[P][D], const T (&go)[P], T (&gx)[P][D]) {
+__device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __restrict__ block_sums, int begin, int end,
+                                             int row, const T (&x)[P][D], const T (&go)[P], T (&gx)[P][D]) {
     constexpr int S = Rec<T, D>::kStride;
     constexpr int NR = Sums<D>::k;
-    for (int g = begin; g < end; ++g) {
+    for (int g = begin + row; g < end; g += 4) {
         T r[Rec<T, D>::kUsed];
 #pragma unroll
         for (int i = 0; i < Rec<T, D>::kUsed; ++i) r[i] = lds[g * S + i];
@@ -127,43 +136,52 @@ __device__ __forceinline__ void bwd_pairs(const T* __restrict__ lds, T* __restri
         }
         if (NEED_GM) {
 #pragma unroll
-            for (int i = 0; i < NR; ++i) rs[i] = wave_sum_to_lane63(rs[i]);
-            if ((threadIdx.x & 63) == 63) {
+            for (int i = 0; i < NR; ++i) rs[i] = row_sum_to_lane15(rs[i]);
+            if ((threadIdx.x & 15) == 15) {
                 const int idx = record_index<T, D>(lds + g * S);
+                if (idx >= 0) {
 #pragma unroll
-                for (int i = 0; i < NR; ++i) atomic_add(&block_sums[idx * NR + i], rs[i]);
+                    for (int i = 0; i < NR; ++i) atomic_add(&block_sums[idx * NR + i], rs[i]);
+                }
             }
         }
     }
 }
 
 template <typename T, int D, int P, bool NEED_GM, bool NEED_GX>
-__global__ __launch_bounds__(kBlock) void eval_bwd_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture,
-                                                          const T* __restrict__ xes, T* __restrict__ sums,
-                                                          T* __restrict__ grad_xes, int L, int M, int N, int Bx, int Lx,
-                                                          int chunks, int xes_shared) {
+__global__ __launch_bounds__(kBlock) void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture,
+                                                             const T* __restrict__ xes, T* __restrict__ sums,
+                                                             T* __restrict__ grad_xes, int L, int M, int N, int Bx, int Lx,
+                                                             int chunks, int xes_shared, int n_mixtures) {
     constexpr int G = 1 + D + D * D;
     constexpr int S = Rec<T, D>::kStride;
     constexpr int NR = Sums<D>::k;
-    __shared__ __attribute__((aligned(16))) T lds[kTile * S];
+    constexpr int kWavePoints = 16 * P;
+    __shared__ __attribute__((aligned(16))) T lds[(kTile + 6) * S];
     __shared__ T block_sums[NEED_GM ? kTile * NR : 1];
     __shared__ int counts[10];
 
-    const int bl = blockIdx.x / chunks;
-    const int chunk = blockIdx.x - bl * chunks;
+    // workgroups are dealt round-robin to the 8 XCDs; keep all point chunks of one mixture on one XCD so that
+    // its L2 serves the repeated reads of the Gaussians
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int bl = (slot / chunks) * 8 + xcd;
+    const int chunk = slot % chunks;
+    if (bl >= n_mixtures) return;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const T* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
     const size_t x_off = (size_t(xb) * Lx + xl) * N;
     const T* __restrict__ x_bl = xes + x_off * D;
 
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = lane >> 4, col = lane & 15;
     T x[P][D];
     T go[P];
     T gx[P][D];
-    const int n0 = chunk * (kBlock * P) + threadIdx.x;
+    const int n0 = (chunk * 4 + wave) * kWavePoints + col;
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-        const int n = n0 + p * kBlock;
+        const int n = n0 + p * 16;
         const int nc = n < N ? n : N - 1;
 #pragma unroll
         for (int d = 0; d < D; ++d) {
@@ -178,11 +196,10 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_kernel(const T* __restrict__ 
 
     for (int g0 = 0; g0 < M; g0 += kTile) {
         const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
-        // amplitude for dL/dx: w * norm / (0.5 log2 e), because C t = u^T y / (0.5 log2 e)
-        stage_tile<T, D>(mix_bl + size_t(g0) * G, cnt, 1.0 / kHalfLog2e, lds, counts);
-        const int n_shifted = counts[8];
-        bwd_pairs<T, D, P, NEED_GM, NEED_GX, false>(lds, block_sums, 0, n_shifted, x, go, gx);
-        bwd_pairs<T, D, P, NEED_GM, NEED_GX, true>(lds, block_sums, n_shifted, cnt, x, go, gx);
+        stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0 / kHalfLog2e, lds, counts);
+        const int centred_start = counts[8], padded_total = counts[9];
+        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, false>(lds, block_sums, 0, centred_start, row, x, go, gx);
+        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, true>(lds, block_sums, centred_start, padded_total, row, x, go, gx);
         if (NEED_GM) {
             __syncthreads();
             T* __restrict__ dst = sums + (size_t(bl) * M + g0) * NR;
@@ -195,13 +212,25 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_kernel(const T* __restrict__ 
     if (NEED_GX) {
 #pragma unroll
         for (int p = 0; p < P; ++p) {
-            const int n = n0 + p * kBlock;
-            if (n < N) {
-                T* dst = grad_xes + (x_off + n) * D;
 #pragma unroll
-                for (int d = 0; d < D; ++d) {
-                    const T v = -go[p] * gx[p][d];
-                    if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
+            for (int d = 0; d < D; ++d) {
+                T v = gx[p][d];
+                v += __shfl_xor(v, 16, 64);
+                v += __shfl_xor(v, 32, 64);
+                gx[p][d] = v;
+            }
+        }
+        if (row == 0) {
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                const int n = n0 + p * 16;
+                if (n < N) {
+                    T* dst = grad_xes + (x_off + n) * D;
+#pragma unroll
+                    for (int d = 0; d < D; ++d) {
+                        const T v = -go[p] * gx[p][d];
+                        if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
+                    }
                 }
             }
         }
@@ -330,8 +359,8 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
     if (s.M == 0) { zero_async(out, BL * s.N, stream); return GMC_OK; }
     const int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
     const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
-    const dim3 grid(unsigned(BL * chunks));
-#define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks)
+    const dim3 grid(unsigned((BL + 7) / 8 * 8 * chunks));
+#define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks, int(BL))
     switch (P) {
         case 8: GMC_FWD(8); break;
         case 4: GMC_FWD(4); break;
@@ -346,16 +375,25 @@ template <typename T, int D, bool GM, bool GX>
 static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T* sums, T* grad_xes, const gmc_shape& s,
                             int xes_shared, hipStream_t stream) {
     const size_t BL = size_t(s.B) * s.L;
-    int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
-    if (P > 4 && sizeof(T) == 8) P = 4;
-    const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
-    const dim3 grid(unsigned(BL * chunks));
-#define GMC_BWD(PP) eval_bwd_kernel<T, D, PP, GM, GX><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared)
+    // a workgroup covers 4 wavefronts x 16 P points; pick the largest P that wastes little of the last chunk
+    int P = 16;
+    if (sizeof(T) == 8) P = 8;
+    while (P > 2) {
+        const int span = 64 * P;
+        const int chunks = (s.N + span - 1) / span;
+        if (double(chunks) * span <= 1.15 * double(s.N) && size_t(chunks) * BL >= 512) break;
+        P >>= 1;
+    }
+    const int span = 64 * P;
+    const int chunks = (s.N + span - 1) / span;
+    const size_t bl8 = (BL + 7) / 8 * 8;
+    const dim3 grid(unsigned(bl8 * chunks));
+#define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL))
     switch (P) {
+        case 16: GMC_BWD(16); break;
         case 8: GMC_BWD(8); break;
         case 4: GMC_BWD(4); break;
-        case 2: GMC_BWD(2); break;
-        default: GMC_BWD(1); break;
+        default: GMC_BWD(2); break;
     }
 #undef GMC_BWD
 }
