@@ -54,12 +54,99 @@ def cpu_baseline(name: str, seconds_budget: float = 20.0):
     }
 
 
+def bench_bvh(args):
+    """LBVH-culled path on C5 (3-D, float64, one mixture of 16384 Gaussians, 100000 points).  A step builds the
+    tree (the mixture changes every training step), evaluates forward and backward.  Throughput is reported in
+    dense-equivalent pairs (B L M N per step); the roofline entry is against HBM with the compulsory bytes of the
+    step (Gaussians, node boxes and links, points in, values and gradients out)."""
+    import torch
+    from gmc import _native, synthetic
+    wl, mix, xes, gout = synthetic.make_workload("C5")
+    dev = torch.device("cuda:0")
+    mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)
+    torch.cuda.synchronize()
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        bvh = _native.Bvh(mix, xes, 0.001, args.aabb_mode)
+        if ev:
+            ev[1].record()
+        out = _native.eval_bvh_fwd(mix, xes, bvh)
+        if ev:
+            ev[2].record()
+        g = _native.eval_bvh_bwd(gout, mix, xes, bvh, True, True)
+        if ev:
+            ev[3].record()
+        return out, g
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(events[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_step = wall * 1e3 / args.steps
+    build_ms, fwd_ms, bwd_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(3))
+    s, M, N, D = 8, wl.M, wl.N, 3
+    bytes_fwd = M * 13 * s + (2 * M - 1) * (2 * D * s + 8) + N * (D + 1) * s
+    bytes_bwd = bytes_fwd + N * s + M * 13 * s + N * D * s
+    line = {
+        "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
+        "value": wl.pairs / (ms_step * 1e-3), "unit": "dense-equivalent Gaussian-point pairs/s (LBVH build + forward + backward step)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": f"C5: D=3 f64 B=1 L=1 M={M} N={N}, LBVH-culled (aabb_mode={args.aabb_mode}, "
+                               f"threshold 0.001), {wl.pairs:.4g} dense-equivalent pairs per step"},
+        "build_ms": build_ms, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "roofline": {"kernel": "bvh_traverse_kernel (backward mode; event pair also holds its zero-fill and epilogue)",
+                     "bound": "hbm", "achieved": bytes_bwd / (bwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
+                     "frac": bytes_bwd / (bwd_ms * 1e-3) / 8e12, "traffic": None, "launch_ms": bwd_ms,
+                     "algorithmic_bytes": bytes_bwd},
+        "roofline_fwd": {"kernel": "bvh_traverse_kernel (forward mode)", "bound": "hbm",
+                         "achieved": bytes_fwd / (fwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
+                         "frac": bytes_fwd / (fwd_ms * 1e-3) / 8e12, "launch_ms": fwd_ms, "algorithmic_bytes": bytes_fwd},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_bvh(args.aabb_mode)
+    print(json.dumps(line))
+
+
+def cpu_baseline_bvh(mode: str):
+    """CPU comparison for the culled path: the C restatement of the reference CPU loops with the per-pair box
+    test in front of each evaluation (the reference has no CPU BVH evaluator to restate), on the first 2000
+    query points of C5 with the boxes of the oracle's rule."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import cpu_ref
+    import gm_oracle
+    from gmc import synthetic
+    wl, mix, xes, gout = synthetic.make_workload("C5", N=2000)
+    m, x, g = mix.numpy(), xes.numpy(), gout.numpy()
+    lo, up = gm_oracle.gaussian_aabbs(m, mode=mode)
+    threads, cores = 128, len(os.sched_getaffinity(0))
+    t0 = time.perf_counter()
+    cpu_ref.forward(m, x, lo, up, n_threads=threads)
+    t_fwd = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    cpu_ref.backward(g, m, x, lo, up, n_threads=threads)
+    t_bwd = time.perf_counter() - t0
+    return {"value": wl.pairs / (t_fwd + t_bwd), "unit": "dense-equivalent pairs/s (fwd+bwd)", "cores": cores,
+            "threads": threads, "kind": "port",
+            "sample": f"C5 slice N=2000 of 100000 points, M=16384 ({wl.pairs:.3g} dense-equivalent pairs), brute-force "
+                      f"box test per pair, fwd {t_fwd:.2f} s + bwd {t_bwd:.2f} s"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4"])
+    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5"],
+                    help="C1..C4: dense all-pairs path; C5: LBVH-culled path (build + forward + backward per step)")
+    ap.add_argument("--aabb-mode", default="reference", choices=["reference", "tight"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (known HBM traffic) so that a counter run of "
@@ -73,6 +160,8 @@ def main():
     import torch
     from gmc import _native, synthetic
 
+    if args.workload == "C5":
+        return bench_bvh(args)
     wl, mix, xes, gout = synthetic.make_workload(args.workload)
     dev = torch.device("cuda:0")
     mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)

@@ -32,6 +32,7 @@ constexpr double kSqFloor = 5.991464547107982;   // -2 ln 0.05 (lbvh/bvh.cu:194)
 struct BvhLayout {
     size_t box_lo, box_hi;      // T [BL][M][D]            per-Gaussian boxes, component order
     size_t node_box;            // T [BL][2M-1][2D]        lower, upper; internal nodes first, then leaves (Morton order)
+    size_t child_box;           // T [BL][M-1][2][2D]      boxes of the left and right child, stored with the parent
     size_t leaf_rec;            // T [BL][M][RS]           evaluation records in leaf order
     size_t children;            // int2 [BL][M-1]          left, right: >= 0 internal node, < 0 leaf ~index
     size_t parent;              // int [BL][2M-1]
@@ -39,8 +40,10 @@ struct BvhLayout {
     size_t visit;               // int [BL][M-1]           arrival counters of the bottom-up pass
     size_t g_bounds;            // T [BL][2D]              bounds of the centres
     size_t p_bounds;            // T [BxLx][2D]            bounds of the query points
+    size_t part_bounds;         // T [segments][blocks][2D] per-block partial bounds
     size_t keys_a, keys_b, vals_a, vals_b;   // uint32 [max(BL*M, BxLx*N)] radix ping-pong
-    size_t hist;                // uint32 [segments][256][blocks]
+    size_t hist;                // uint32 [segments][256][blocks] block histograms, then [segments][256] digit totals
+    size_t hist_totals;         // offset of the digit totals inside the histogram area
     size_t p_order;             // int [BxLx][N]           Morton order of the query points
     size_t g_keys;              // uint32 [BL][M]          sorted Morton codes of the leaves
     size_t total;
@@ -48,6 +51,7 @@ struct BvhLayout {
 
 constexpr int kSortItems = 8;                       // items per lane and radix block
 constexpr int kSortChunk = kBlock * kSortItems;     // 2048
+constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the first bounds pass
 
 template <int D> struct LeafRec { static constexpr int kStride = (D == 2) ? 8 : 12; };
 // D=3: b0 b1 b2 c00 c01 c02 c11 c12 c22 amp comp -   D=2: b0 b1 c00 c01 c11 amp comp -
@@ -66,6 +70,7 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.box_lo = take(BL * M * D * e);
     l.box_hi = take(BL * M * D * e);
     l.node_box = take(BL * nodes * 2 * D * e);
+    l.child_box = take(BL * (M > 0 ? M - 1 : 0) * 4 * D * e);
     l.leaf_rec = take(BL * M * rs * e);
     l.children = take(BL * (M > 0 ? M - 1 : 0) * 8);
     l.parent = take(BL * nodes * 4);
@@ -73,6 +78,10 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.visit = take(BL * (M > 0 ? M - 1 : 0) * 4);
     l.g_bounds = take(BL * 2 * D * e);
     l.p_bounds = take(XL * 2 * D * e);
+    {
+        const size_t pg = BL * ((M + kBoundsChunk - 1) / kBoundsChunk), pp = XL * ((N + kBoundsChunk - 1) / kBoundsChunk);
+        l.part_bounds = take((pg > pp ? pg : pp) * 2 * D * e);
+    }
     const size_t items = BL * M > XL * N ? BL * M : XL * N;
     l.keys_a = take(items * 4);
     l.keys_b = take(items * 4);
@@ -80,6 +89,7 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.vals_b = take(items * 4);
     const size_t bg = BL * ((M + kSortChunk - 1) / kSortChunk), bp = XL * ((N + kSortChunk - 1) / kSortChunk);
     l.hist = take((bg > bp ? bg : bp) * 256 * 4);
+    l.hist_totals = take((BL > XL ? BL : XL) * 256 * 4);
     l.p_order = take(XL * N * 4);
     l.g_keys = take(BL * M * 4);
     l.total = o;
@@ -246,20 +256,24 @@ __global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__
 // bounds of a point set, Morton keys
 // ---------------------------------------------------------------------------------------------------------------
 
-// one workgroup per segment: bounds[seg] = (min_0..min_D-1, max_0..max_D-1) over `count` points of stride `stride`
+// Bounds of `count` points per segment in two passes.  Pass 1: workgroup (blk, seg) reduces kBoundsChunk points
+// to parts[seg][blk] = (min_0..min_D-1, max_0..max_D-1); pass 2 runs the same kernel over the partial results
+// (`hi_off` = D: maxima are taken from the second half of every partial record).
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bounds_kernel(const T* __restrict__ pts, int stride, int offset, int count,
-                                                       T* __restrict__ bounds) {
+__global__ __launch_bounds__(kBlock) void bounds_kernel(const T* __restrict__ pts, int stride, int offset, int hi_off,
+                                                       int count, int chunk, int blocks_per_seg, T* __restrict__ out) {
     __shared__ T red[2 * D][kBlock];
-    const size_t seg = blockIdx.x;
-    const T* p = pts + seg * size_t(count) * stride + offset;
+    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    const T* p = pts + size_t(seg) * count * stride + offset;
+    const int begin = blk * chunk;
+    const int end = begin + chunk < count ? begin + chunk : count;
     T lo[D], hi[D];
     for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
-    for (int i = threadIdx.x; i < count; i += kBlock)
+    for (int i = begin + threadIdx.x; i < end; i += kBlock)
         for (int d = 0; d < D; ++d) {
-            const T v = p[size_t(i) * stride + d];
-            lo[d] = v < lo[d] ? v : lo[d];
-            hi[d] = v > hi[d] ? v : hi[d];
+            const T a = p[size_t(i) * stride + d], b = p[size_t(i) * stride + hi_off + d];
+            lo[d] = a < lo[d] ? a : lo[d];
+            hi[d] = b > hi[d] ? b : hi[d];
         }
     for (int d = 0; d < D; ++d) { red[d][threadIdx.x] = lo[d]; red[D + d][threadIdx.x] = hi[d]; }
     __syncthreads();
@@ -272,7 +286,7 @@ __global__ __launch_bounds__(kBlock) void bounds_kernel(const T* __restrict__ pt
             }
         __syncthreads();
     }
-    if (threadIdx.x < 2 * D) bounds[seg * 2 * D + threadIdx.x] = red[threadIdx.x][0];
+    if (threadIdx.x < 2 * D) out[size_t(blockIdx.x) * 2 * D + threadIdx.x] = red[threadIdx.x][0];
 }
 
 __device__ __forceinline__ uint32_t expand_bits3(uint32_t v) {
@@ -327,37 +341,50 @@ __global__ __launch_bounds__(kBlock) void radix_hist_kernel(const uint32_t* __re
     hist[(size_t(seg) * 256 + threadIdx.x) * blocks_per_seg + blk] = h[threadIdx.x];
 }
 
-__global__ __launch_bounds__(kBlock) void radix_scan_kernel(uint32_t* __restrict__ hist, int blocks_per_seg) {
-    __shared__ uint32_t totals[256];
-    uint32_t* h = hist + (size_t(blockIdx.x) * 256 + threadIdx.x) * blocks_per_seg;
-    uint32_t run = 0;
-    for (int b = 0; b < blocks_per_seg; ++b) { const uint32_t c = h[b]; h[b] = run; run += c; }
-    totals[threadIdx.x] = run;
-    __syncthreads();
-    // exclusive scan of the 256 digit totals (Hillis-Steele on LDS)
-    uint32_t mine = run;
-    for (int off = 1; off < 256; off <<= 1) {
-        const uint32_t add = int(threadIdx.x) >= off ? totals[threadIdx.x - off] : 0u;
-        __syncthreads();
-        totals[threadIdx.x] += add;
-        __syncthreads();
+// one wavefront per (segment, digit): exclusive scan of that digit's block counts, digit total to `totals`
+__global__ __launch_bounds__(kWave) void radix_scan_kernel(uint32_t* __restrict__ hist, uint32_t* __restrict__ totals,
+                                                          int blocks_per_seg) {
+    uint32_t* h = hist + size_t(blockIdx.x) * blocks_per_seg;
+    const int lane = threadIdx.x;
+    uint32_t carry = 0;
+    for (int base = 0; base < blocks_per_seg; base += kWave) {
+        const int b = base + lane;
+        const uint32_t c = b < blocks_per_seg ? h[b] : 0u;
+        uint32_t incl = c;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const uint32_t o = __shfl_up(incl, off, kWave);
+            if (lane >= off) incl += o;
+        }
+        if (b < blocks_per_seg) h[b] = carry + incl - c;
+        carry += __shfl(incl, kWave - 1, kWave);
     }
-    const uint32_t base = totals[threadIdx.x] - mine;
-    for (int b = 0; b < blocks_per_seg; ++b) h[b] += base;
+    if (lane == 0) totals[blockIdx.x] = carry;
 }
 
 __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const uint32_t* __restrict__ keys_in,
                                                               const uint32_t* __restrict__ vals_in,
                                                               uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
                                                               int count, int blocks_per_seg, int shift,
-                                                              const uint32_t* __restrict__ hist) {
+                                                              const uint32_t* __restrict__ hist,
+                                                              const uint32_t* __restrict__ totals) {
     __shared__ uint32_t running[256];        // next output slot of every digit for this block
     __shared__ uint32_t wave_count[4][256];
     const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    running[threadIdx.x] = hist[(size_t(seg) * 256 + threadIdx.x) * blocks_per_seg + blk];
+    // exclusive scan of the segment's digit totals (Hillis-Steele on LDS) = first slot of every digit
+    const uint32_t mine = totals[size_t(seg) * 256 + threadIdx.x];
+    running[threadIdx.x] = mine;
 #pragma unroll
     for (int w = 0; w < 4; ++w) wave_count[w][threadIdx.x] = 0;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+        const uint32_t add = int(threadIdx.x) >= off ? running[threadIdx.x - off] : 0u;
+        __syncthreads();
+        running[threadIdx.x] += add;
+        __syncthreads();
+    }
+    running[threadIdx.x] += hist[(size_t(seg) * 256 + threadIdx.x) * blocks_per_seg + blk] - mine;
     __syncthreads();
     const size_t seg_off = size_t(seg) * count;
     const int begin = blk * kSortChunk;
@@ -489,32 +516,39 @@ __global__ __launch_bounds__(kBlock) void bvh_tree_kernel(const uint32_t* __rest
     if (i == 0) par[0] = -1;
 }
 
+// Bottom-up boxes: one lane per leaf walks towards the root.  A node's box is handed to its parent's child_box
+// slot; the first lane to arrive at a parent stops, the second one finds both child boxes, forms their union and
+// carries it further up.  Release/acquire fences around the arrival counter order the box stores and loads.
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int2* __restrict__ children, const int* __restrict__ parent,
-                                                          T* node_box, int* visit, int M, size_t total) {
+                                                          T* node_box, T* child_box, int* visit, int M, size_t total) {
     const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
     if (t >= total) return;
     const size_t bl = t / M;
     const int leaf = int(t - bl * M);
     const size_t nbase = bl * (2 * size_t(M) - 1);
     T* boxes = node_box + nbase * 2 * D;
+    T* cboxes = child_box + bl * (M - 1) * 4 * D;
+    const int2* kids = children + bl * (M - 1);
+    int self = ~leaf;                                     // encoded like a child link
+    T box[2 * D];
+    for (int d = 0; d < 2 * D; ++d) box[d] = boxes[size_t((M - 1) + leaf) * 2 * D + d];
     int node = parent[nbase + (M - 1) + leaf];
     // a leaf is at most M - 1 levels below the root; the bound also ends the walk on a malformed parent chain
     for (int level = 0; node >= 0 && node < M - 1 && level < M; ++level) {
-        __threadfence();                                   // publish this lane's box before announcing arrival
+        const int side = kids[node].x == self ? 0 : 1;
+        for (int d = 0; d < 2 * D; ++d) cboxes[(size_t(node) * 2 + side) * 2 * D + d] = box[d];
+        __threadfence();                                   // publish the box before announcing the arrival
         if (atomicAdd(&visit[bl * (M - 1) + node], 1) == 0) return;   // first arrival: the sibling will finish
         __threadfence();
-        const int2 ch = children[bl * (M - 1) + node];
-        const int l = ch.x >= 0 ? ch.x : (M - 1) + ~ch.x, r = ch.y >= 0 ? ch.y : (M - 1) + ~ch.y;
-        // child boxes were written by other lanes; the fence pair around the counter orders them before these loads
+        const T* other = cboxes + (size_t(node) * 2 + (1 - side)) * 2 * D;
         for (int d = 0; d < D; ++d) {
-            const T a = boxes[size_t(l) * 2 * D + d];
-            const T b = boxes[size_t(r) * 2 * D + d];
-            const T c = boxes[size_t(l) * 2 * D + D + d];
-            const T e = boxes[size_t(r) * 2 * D + D + d];
-            boxes[size_t(node) * 2 * D + d] = a < b ? a : b;
-            boxes[size_t(node) * 2 * D + D + d] = c > e ? c : e;
+            const T a = other[d], b = other[D + d];
+            box[d] = a < box[d] ? a : box[d];
+            box[D + d] = b > box[D + d] ? b : box[D + d];
         }
+        for (int d = 0; d < 2 * D; ++d) boxes[size_t(node) * 2 * D + d] = box[d];
+        self = node;
         node = parent[nbase + node];
     }
 }
@@ -522,11 +556,13 @@ __global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int2* __restric
 // ---------------------------------------------------------------------------------------------------------------
 // traversal
 // ---------------------------------------------------------------------------------------------------------------
+// closed-interval test of a point against a box given as (lower[D], upper[D]); every comparison is evaluated
+// (no short-circuit), so the box scalars can be fetched with one wide load before the test
 template <typename T, int D>
-__device__ __forceinline__ bool inside_box(const T (&x)[D], const T* __restrict__ box) {
+__device__ __forceinline__ bool inside_box(const T (&x)[D], const T* box) {
     bool in = true;
 #pragma unroll
-    for (int d = 0; d < D; ++d) in = in && !(x[d] < box[d]) && !(x[d] > box[D + d]) && (x[d] == x[d]);
+    for (int d = 0; d < D; ++d) in = in & (x[d] >= box[d]) & (x[d] <= box[D + d]);
     return in;
 }
 
@@ -553,11 +589,13 @@ __device__ __forceinline__ T leaf_terms(const T* __restrict__ r, const T (&x)[D]
 template <int D> struct BvhSums { static constexpr int k = 1 + D + D * (D + 1) / 2; };
 
 // MODE 0: forward.  MODE 1: backward (grad_out given; accumulates per-Gaussian sums and dL/dx).
-template <typename T, int D, int MODE, bool NEED_GM, bool NEED_GX>
+// W = points per wavefront (lanes W..63 idle).  The traversal is bound by the latency of dependent node loads,
+// not by lanes, so small inputs use W < 64: more wavefronts in flight and smaller node unions per wavefront.
+template <typename T, int D, int MODE, bool NEED_GM, bool NEED_GX, int W>
 __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
         const T* __restrict__ xes, const int* __restrict__ p_order, const T* __restrict__ node_box,
-        const int2* __restrict__ children, const T* __restrict__ leaf_rec, T* __restrict__ out,
-        const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes,
+        const T* __restrict__ child_box, const int2* __restrict__ children, const T* __restrict__ leaf_rec,
+        T* __restrict__ out, const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes,
         int L, int M, int N, int Bx, int Lx, int chunks, int xes_shared) {
     constexpr int RS = LeafRec<D>::kStride;
     constexpr int NR = BvhSums<D>::k;
@@ -570,8 +608,9 @@ __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
     const int wave = threadIdx.x >> 6;
     int* stack = stack_mem[wave];
 
-    const int j = chunk * kBlock + threadIdx.x;
-    const bool valid = j < N;
+    const int lane = threadIdx.x & 63;
+    const int j = (chunk * (kBlock / kWave) + wave) * W + lane;
+    const bool valid = lane < W && j < N;
     const int pid = valid ? p_order[xseg * N + j] : 0;
     T x[D];
 #pragma unroll
@@ -580,6 +619,7 @@ __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
     if (MODE == 1) g = valid ? grad_out[size_t(bl) * N + pid] : T(0);
 
     const T* boxes = node_box + size_t(bl) * (2 * size_t(M) - 1) * 2 * D;
+    const T* cboxes = child_box + size_t(bl) * (M - 1) * 4 * D;
     const int2* kids = children + size_t(bl) * (M - 1);
     const T* recs = leaf_rec + size_t(bl) * M * RS;
     T acc = T(0);
@@ -611,9 +651,11 @@ __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
                 for (int a = 0; a < D; ++a)
 #pragma unroll
                     for (int c = a; c < D; ++c) rs[k++] = rs[1 + a] * t[c];
+                // lanes W..63 hold zeros; with W == 16 all points sit in the first DPP row
+                constexpr int kLast = W == 16 ? 15 : 63;
 #pragma unroll
-                for (int i = 0; i < NR; ++i) rs[i] = wave_sum_to_lane63(rs[i]);
-                if ((threadIdx.x & 63) == 63) {
+                for (int i = 0; i < NR; ++i) rs[i] = W == 16 ? row_sum_to_lane15(rs[i]) : wave_sum_to_lane63(rs[i]);
+                if ((threadIdx.x & 63) == kLast) {
                     const int comp = reinterpret_cast<const int*>(r + D + D * (D + 1) / 2 + 1)[0];
                     T* dst = sums + (size_t(bl) * M + comp) * NR;
 #pragma unroll
@@ -624,7 +666,10 @@ __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
     };
 
     if (M == 1) {
-        const bool in = valid && inside_box<T, D>(x, boxes);
+        T bx[2 * D];
+#pragma unroll
+        for (int i = 0; i < 2 * D; ++i) bx[i] = boxes[i];
+        const bool in = valid & inside_box<T, D>(x, bx);
         if (__ballot(in) != 0ull) visit_leaf(0, in);
     } else {
         int sp = 0;
@@ -633,13 +678,17 @@ __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
         for (int iter = 0; sp > 0 && iter < M; ++iter) {
             const int node = __builtin_amdgcn_readfirstlane(stack[--sp]);
             const int2 ch = kids[node];
+            // both child boxes in one go: 4 D wave-uniform scalars, independent of the link load above
+            T cb[4 * D];
+#pragma unroll
+            for (int i = 0; i < 4 * D; ++i) cb[i] = cboxes[size_t(node) * 4 * D + i];
             const int c0 = __builtin_amdgcn_readfirstlane(ch.x), c1 = __builtin_amdgcn_readfirstlane(ch.y);
+            const bool in0 = valid & inside_box<T, D>(x, cb), in1 = valid & inside_box<T, D>(x, cb + 2 * D);
 #pragma unroll
             for (int side = 0; side < 2; ++side) {
                 const int c = side == 0 ? c0 : c1;
                 if (c >= M - 1 || ~c >= M) continue;                 // not a node of this tree
-                const int cnode = c >= 0 ? c : (M - 1) + ~c;
-                const bool in = valid && inside_box<T, D>(x, boxes + size_t(cnode) * 2 * D);
+                const bool in = side == 0 ? in0 : in1;
                 if (__ballot(in) != 0ull) {
                     if (c < 0) visit_leaf(~c, in);
                     else if (sp < kStackDepth) stack[sp++] = c;
@@ -748,22 +797,32 @@ __global__ void iota_segments_kernel(int* __restrict__ dst, int count, size_t to
 // ---------------------------------------------------------------------------------------------------------------
 static unsigned grid_for(size_t n) { return unsigned((n + kBlock - 1) / kBlock); }
 
-// sorts `segments` segments of `count` (key, value) pairs held in (ka, va) on bits [0, 8*passes); returns 0 if the
-// result is in the a buffers, 1 if in the b buffers
-static int radix_sort(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* hist, int segments, int count,
-                      int passes, hipStream_t st) {
+// sorts `segments` segments of `count` (key, value) pairs held in (ka, va) on the key bits
+// [first_bit, first_bit + 8 * passes); returns 0 if the result is in the a buffers, 1 if in the b buffers
+static int radix_sort(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* hist, uint32_t* totals,
+                      int segments, int count, int first_bit, int passes, hipStream_t st) {
     const int bps = (count + kSortChunk - 1) / kSortChunk;
     const dim3 grid(unsigned(size_t(segments) * bps));
     int cur = 0;
     for (int p = 0; p < passes; ++p) {
         uint32_t* kin = cur ? kb : ka; uint32_t* vin = cur ? vb : va;
         uint32_t* kout = cur ? ka : kb; uint32_t* vout = cur ? va : vb;
-        radix_hist_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, count, bps, 8 * p, hist);
-        radix_scan_kernel<<<dim3(unsigned(segments)), dim3(kBlock), 0, st>>>(hist, bps);
-        radix_scatter_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, vin, kout, vout, count, bps, 8 * p, hist);
+        const int shift = first_bit + 8 * p;
+        radix_hist_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, count, bps, shift, hist);
+        radix_scan_kernel<<<dim3(unsigned(segments) * 256), dim3(kWave), 0, st>>>(hist, totals, bps);
+        radix_scatter_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, vin, kout, vout, count, bps, shift, hist, totals);
         cur ^= 1;
     }
     return cur;
+}
+
+template <typename T, int D>
+static void launch_bounds_of(const T* pts, int stride, int offset, int count, size_t segments, T* parts, T* out,
+                             hipStream_t st) {
+    const int nb = (count + kBoundsChunk - 1) / kBoundsChunk;
+    bounds_kernel<T, D><<<dim3(unsigned(segments * nb)), dim3(kBlock), 0, st>>>(pts, stride, offset, 0, count, kBoundsChunk,
+                                                                              nb, parts);
+    bounds_kernel<T, D><<<dim3(unsigned(segments)), dim3(kBlock), 0, st>>>(parts, 2 * D, 0, D, nb, nb, 1, out);
 }
 
 template <typename T, int D>
@@ -780,14 +839,17 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     uint32_t* ka = (uint32_t*)(bvh + lay.keys_a); uint32_t* kb = (uint32_t*)(bvh + lay.keys_b);
     uint32_t* va = (uint32_t*)(bvh + lay.vals_a); uint32_t* vb = (uint32_t*)(bvh + lay.vals_b);
     uint32_t* hist = (uint32_t*)(bvh + lay.hist);
+    uint32_t* totals = (uint32_t*)(bvh + lay.hist_totals);
+    T* parts = (T*)(bvh + lay.part_bounds);
+    T* child_box = (T*)(bvh + lay.child_box);
     if (BL > 0 && M > 0) {
         const size_t n = BL * M;
         bvh_boxes_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, n,
                                                                           double(cfg.aabb_threshold), cfg.aabb_mode);
         T* gb = (T*)(bvh + lay.g_bounds);
-        bounds_kernel<T, D><<<dim3(unsigned(BL)), dim3(kBlock), 0, st>>>(mixture, G, 1, M, gb);
+        launch_bounds_of<T, D>(mixture, G, 1, M, BL, parts, gb, st);
         morton_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, G, 1, M, gb, ka, va, n);
-        const int where = radix_sort(ka, va, kb, vb, hist, int(BL), M, 4, st);
+        const int where = radix_sort(ka, va, kb, vb, hist, totals, int(BL), M, 0, 4, st);
         uint32_t* g_keys = (uint32_t*)(bvh + lay.g_keys);
         copy_kernel<uint32_t><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(where ? kb : ka, g_keys, n);
         bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, where ? vb : va, node_box,
@@ -795,7 +857,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         if (M > 1) {
             const size_t ni = BL * (M - 1);
             bvh_tree_kernel<<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(g_keys, children, parent, M, ni);
-            bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(children, parent, node_box, visit, M, n);
+            bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(children, parent, node_box, child_box, visit, M, n);
         }
     }
     if (XL > 0 && N > 0) {
@@ -803,9 +865,10 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         const size_t n = XL * N;
         if (xes) {
             T* pb = (T*)(bvh + lay.p_bounds);
-            bounds_kernel<T, D><<<dim3(unsigned(XL)), dim3(kBlock), 0, st>>>(xes, D, 0, N, pb);
+            launch_bounds_of<T, D>(xes, D, 0, N, XL, parts, pb, st);
             morton_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(xes, D, 0, N, pb, ka, va, n);
-            const int where = radix_sort(ka, va, kb, vb, hist, int(XL), N, 4, st);
+            // 16 Morton bits (65536 cells) are enough to make 64 consecutive points neighbours
+            const int where = radix_sort(ka, va, kb, vb, hist, totals, int(XL), N, 14, 2, st);
             copy_kernel<uint32_t><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(
                 where ? vb : va, (uint32_t*)p_order, n);
         } else {
@@ -813,6 +876,14 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         }
     }
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
+
+// points per wavefront of the traversal: keep at least ~8 wavefronts per SIMD (256 CUs x 4 SIMDs) in flight
+static int points_per_wave(size_t n_mixtures, int n_points) {
+    const size_t pts = n_mixtures * size_t(n_points);
+    if (pts >= size_t(64) * 8192) return 64;
+    if (pts >= size_t(32) * 8192) return 32;
+    return 16;
 }
 
 template <typename T, int D>
@@ -825,10 +896,15 @@ static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, 
         fill_zero_kernel<T><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(out, n);
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    const int chunks = (s.N + kBlock - 1) / kBlock;
-    bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kBlock), 0, st>>>(
-        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const int2*)(bvh + lay.children),
-        (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N, s.Bx, s.Lx, chunks, 0);
+    const int W = points_per_wave(BL, s.N);
+    const int chunks = (s.N + 4 * W - 1) / (4 * W);
+    const dim3 grid(unsigned(BL * chunks));
+#define GMC_TRAV(WW) bvh_traverse_kernel<T, D, 0, false, false, WW><<<grid, dim3(kBlock), 0, st>>>( \
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const T*)(bvh + lay.child_box), \
+        (const int2*)(bvh + lay.children), (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N, \
+        s.Bx, s.Lx, chunks, 0)
+    if (W == 64) GMC_TRAV(64); else if (W == 32) GMC_TRAV(32); else GMC_TRAV(16);
+#undef GMC_TRAV
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
@@ -852,14 +928,18 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, const ch
     }
     if (gm) zero(sums, n_g * NR);
     if (gx && xes_shared) zero(grad_xes, n_x);
-    const int chunks = (s.N + kBlock - 1) / kBlock;
+    const int W = points_per_wave(BL, s.N);
+    const int chunks = (s.N + 4 * W - 1) / (4 * W);
     const dim3 grid(unsigned(BL * chunks));
-#define GMC_TRAV(GM, GX) bvh_traverse_kernel<T, D, 1, GM, GX><<<grid, dim3(kBlock), 0, st>>>( \
-        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const int2*)(bvh + lay.children), \
-        (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared)
-    if (gm && gx) GMC_TRAV(true, true);
-    else if (gm) GMC_TRAV(true, false);
-    else if (gx) GMC_TRAV(false, true);
+#define GMC_TRAV(GM, GX, WW) bvh_traverse_kernel<T, D, 1, GM, GX, WW><<<grid, dim3(kBlock), 0, st>>>( \
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const T*)(bvh + lay.child_box), \
+        (const int2*)(bvh + lay.children), (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, s.L, s.M, s.N, \
+        s.Bx, s.Lx, chunks, xes_shared)
+#define GMC_TRAV_W(GM, GX) do { if (W == 64) GMC_TRAV(GM, GX, 64); else if (W == 32) GMC_TRAV(GM, GX, 32); else GMC_TRAV(GM, GX, 16); } while (0)
+    if (gm && gx) GMC_TRAV_W(true, true);
+    else if (gm) GMC_TRAV_W(true, false);
+    else if (gx) GMC_TRAV_W(false, true);
+#undef GMC_TRAV_W
 #undef GMC_TRAV
     if (gm) bvh_bwd_epilogue_kernel<T, D><<<dim3(grid_for(n_g)), dim3(kBlock), 0, st>>>(mixture, sums, grad_mixture, n_g);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;

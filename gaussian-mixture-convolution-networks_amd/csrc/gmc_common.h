@@ -209,7 +209,17 @@ __device__ __forceinline__ float dpp_mov(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
 }
 
-__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ double dpp_mov(double v) {
+    // a 64-bit value moves as its two halves; lanes without a source receive 0.0
+    const long long bits = __builtin_bit_cast(long long, v);
+    const int lo = __builtin_amdgcn_update_dpp(0, int(bits), CTRL, ROW_MASK, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, int(bits >> 32), CTRL, ROW_MASK, 0xf, false);
+    return __builtin_bit_cast(double, (long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned)lo));
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_sum_to_lane63(T v) {
     v += dpp_mov<0x111>(v);          // row_shr:1
     v += dpp_mov<0x112>(v);          // row_shr:2
     v += dpp_mov<0x114>(v);          // row_shr:4
@@ -219,30 +229,13 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
     return v;
 }
 
-__device__ __forceinline__ double wave_sum_to_lane63(double v) {
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const double o = __shfl_up(v, off, 64);
-        if ((threadIdx.x & 63) >= off) v += o;
-    }
-    return v;
-}
-
 // ---- sum over the 16 lanes of a DPP row; the total arrives in lane 15 of the row ---------------------------
-__device__ __forceinline__ float row_sum_to_lane15(float v) {
+template <typename T>
+__device__ __forceinline__ T row_sum_to_lane15(T v) {
     v += dpp_mov<0x111>(v);
     v += dpp_mov<0x112>(v);
     v += dpp_mov<0x114>(v);
     v += dpp_mov<0x118>(v);
-    return v;
-}
-
-__device__ __forceinline__ double row_sum_to_lane15(double v) {
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
-        const double o = __shfl_up(v, off, 16);
-        if ((threadIdx.x & 15) >= off) v += o;
-    }
     return v;
 }
 

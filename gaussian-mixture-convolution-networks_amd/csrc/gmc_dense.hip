@@ -18,6 +18,27 @@ namespace gmc {
 
 constexpr int kTile = 256;   // Gaussians staged per LDS tile (one per lane)
 
+// Workgroups are dealt round-robin to the 8 XCDs.  With at least kXcdAffineMin mixtures all point chunks of one
+// mixture go to one XCD, so that its L2 serves the repeated reads of the Gaussians (the grid then has
+// ceil(n_mixtures / 8) * 8 * chunks workgroups, surplus ones exit); with fewer mixtures chunks are dealt
+// plainly, otherwise a single mixture would occupy one XCD only.
+constexpr int kXcdAffineMin = 64;
+
+__device__ __forceinline__ void map_workgroup(int id, int chunks, int n_mixtures, int& bl, int& chunk) {
+    if (n_mixtures >= kXcdAffineMin) {
+        const int xcd = id & 7, slot = id >> 3;
+        bl = (slot / chunks) * 8 + xcd;
+        chunk = slot % chunks;
+    } else {
+        bl = id / chunks;
+        chunk = id - bl * chunks;
+    }
+}
+
+static size_t grid_mixtures(size_t n_mixtures) {
+    return n_mixtures >= size_t(kXcdAffineMin) ? (n_mixtures + 7) / 8 * 8 : n_mixtures;
+}
+
 template <typename T, int D, int P, bool CENTRED>
 __device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, int begin, int end, const T (&x)[P][D], T (&acc)[P]) {
     constexpr int S = Rec<T, D>::kStride;
@@ -44,11 +65,8 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
     __shared__ __attribute__((aligned(16))) T lds[kTile * S];
     __shared__ int counts[10];
 
-    // workgroups are dealt round-robin to the 8 XCDs; keep all point chunks of one mixture on one XCD so that
-    // its L2 serves the repeated reads of the Gaussians
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int bl = (slot / chunks) * 8 + xcd;
-    const int chunk = slot % chunks;
+    int bl, chunk;
+    map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
     if (bl >= n_mixtures) return;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
@@ -161,11 +179,8 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_rc_kernel(const T* __restrict
     __shared__ T block_sums[NEED_GM ? kTile * NR : 1];
     __shared__ int counts[10];
 
-    // workgroups are dealt round-robin to the 8 XCDs; keep all point chunks of one mixture on one XCD so that
-    // its L2 serves the repeated reads of the Gaussians
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int bl = (slot / chunks) * 8 + xcd;
-    const int chunk = slot % chunks;
+    int bl, chunk;
+    map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
     if (bl >= n_mixtures) return;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
@@ -359,7 +374,7 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
     if (s.M == 0) { zero_async(out, BL * s.N, stream); return GMC_OK; }
     const int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
     const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
-    const dim3 grid(unsigned((BL + 7) / 8 * 8 * chunks));
+    const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
 #define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks, int(BL))
     switch (P) {
         case 8: GMC_FWD(8); break;
@@ -386,8 +401,7 @@ static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T
     }
     const int span = 64 * P;
     const int chunks = (s.N + span - 1) / span;
-    const size_t bl8 = (BL + 7) / 8 * 8;
-    const dim3 grid(unsigned(bl8 * chunks));
+    const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
 #define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL))
     switch (P) {
         case 16: GMC_BWD(16); break;
