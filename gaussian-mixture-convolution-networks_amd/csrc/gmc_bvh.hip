@@ -10,7 +10,7 @@
 //   boxes + centre bounds -> 30-bit Morton codes of the centres (lbvh/morton_code.h:77-85,145-168) -> segmented LSD
 //   radix sort (8 bits per pass, stable, keys uint32 + index payload) -> leaves in Morton order with their
 //   evaluation records -> Karras radix tree over the unique keys (morton << 32 | rank), as lbvh/building.h:11-103
-//   -> bottom-up union of boxes with one visit counter per internal node.
+//   -> bottom-up union of boxes with integer atomic min/max on order-preserving encodings.
 // Query points are Morton-sorted the same way so that a wavefront owns 64 neighbouring points.
 //
 // Traversal: one wavefront per 64 sorted points, ONE stack per wavefront (LDS).  A node is entered when any
@@ -37,7 +37,7 @@ struct BvhLayout {
     size_t children;            // int2 [BL][M-1]          left, right: >= 0 internal node, < 0 leaf ~index
     size_t parent;              // int [BL][2M-1]
     size_t leaf_comp;           // int [BL][M]             component id of each leaf
-    size_t visit;               // int [BL][M-1]           arrival counters of the bottom-up pass
+    size_t enc_box;             // int64 [BL][M-1][2D]     boxes of the internal nodes as order-preserving integers
     size_t g_bounds;            // T [BL][2D]              bounds of the centres
     size_t p_bounds;            // T [BxLx][2D]            bounds of the query points
     size_t part_bounds;         // T [segments][blocks][2D] per-block partial bounds
@@ -75,7 +75,7 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.children = take(BL * (M > 0 ? M - 1 : 0) * 8);
     l.parent = take(BL * nodes * 4);
     l.leaf_comp = take(BL * M * 4);
-    l.visit = take(BL * (M > 0 ? M - 1 : 0) * 4);
+    l.enc_box = take(BL * (M > 0 ? M - 1 : 0) * 2 * D * 8);
     l.g_bounds = take(BL * 2 * D * e);
     l.p_bounds = take(XL * 2 * D * e);
     {
@@ -425,11 +425,21 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const uint32_t* _
 // ---------------------------------------------------------------------------------------------------------------
 // leaves, radix tree, bottom-up boxes
 // ---------------------------------------------------------------------------------------------------------------
+// Order-preserving map from a floating-point value to a signed 64-bit integer (a < b <=> ordered(a) < ordered(b)),
+// so that box unions can be formed with integer atomic min/max.
+__device__ __forceinline__ long long ordered_bits(double v) {
+    const long long b = __builtin_bit_cast(long long, v);
+    return b ^ ((b >> 63) & 0x7fffffffffffffffll);
+}
+__device__ __forceinline__ double from_ordered_bits(long long k) {
+    return __builtin_bit_cast(double, k ^ ((k >> 63) & 0x7fffffffffffffffll));
+}
+
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, const T* __restrict__ box_lo,
                                                            const T* __restrict__ box_hi, const uint32_t* __restrict__ order,
                                                            T* __restrict__ node_box, T* __restrict__ leaf_rec,
-                                                           int* __restrict__ leaf_comp, int* __restrict__ visit,
+                                                           int* __restrict__ leaf_comp, long long* __restrict__ enc_box,
                                                            int* __restrict__ parent, int M, size_t total) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
@@ -446,7 +456,11 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         node_box[node * 2 * D + D + d] = box_hi[gi * D + d];
     }
     leaf_comp[i] = comp;
-    if (leaf < M - 1) visit[bl * (M - 1) + leaf] = 0;
+    if (leaf < M - 1) {
+        // empty box of internal node `leaf`: lower = +inf, upper = -inf in the ordered-integer encoding
+        long long* e = enc_box + (bl * (M - 1) + leaf) * 2 * D;
+        for (int d = 0; d < D; ++d) { e[d] = ordered_bits(double(INFINITY)); e[D + d] = ordered_bits(double(-INFINITY)); }
+    }
     if (M == 1) parent[node] = -1;                  // a single leaf is its own root
     const T* g = mixture + gi * G;
     T* r = leaf_rec + i * RS;
@@ -516,40 +530,60 @@ __global__ __launch_bounds__(kBlock) void bvh_tree_kernel(const uint32_t* __rest
     if (i == 0) par[0] = -1;
 }
 
-// Bottom-up boxes: one lane per leaf walks towards the root.  A node's box is handed to its parent's child_box
-// slot; the first lane to arrive at a parent stops, the second one finds both child boxes, forms their union and
-// carries it further up.  Release/acquire fences around the arrival counter order the box stores and loads.
+// Bottom-up boxes without inter-lane ordering: one lane per leaf walks towards the root and merges ITS OWN leaf
+// box into every ancestor with atomic min/max, as long as it still enlarges the ancestor; it stops at the first
+// ancestor that already contains it.  Every extreme of that ancestor was set by some leaf that enlarged it and
+// therefore walks on itself, so all higher ancestors end up containing the stopped leaf as well: the final boxes
+// are the exact unions of the leaves below each node.  Nothing is read back except the atomics' own return
+// values, so no fences are needed; the decoded boxes are produced by the next kernel.
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int2* __restrict__ children, const int* __restrict__ parent,
-                                                          T* node_box, T* child_box, int* visit, int M, size_t total) {
+__global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int* __restrict__ parent, const T* __restrict__ node_box,
+                                                          long long* enc_box, int M, size_t total) {
     const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
     if (t >= total) return;
     const size_t bl = t / M;
     const int leaf = int(t - bl * M);
     const size_t nbase = bl * (2 * size_t(M) - 1);
-    T* boxes = node_box + nbase * 2 * D;
-    T* cboxes = child_box + bl * (M - 1) * 4 * D;
-    const int2* kids = children + bl * (M - 1);
-    int self = ~leaf;                                     // encoded like a child link
-    T box[2 * D];
-    for (int d = 0; d < 2 * D; ++d) box[d] = boxes[size_t((M - 1) + leaf) * 2 * D + d];
+    const T* box = node_box + (nbase + (M - 1) + leaf) * 2 * D;
+    long long* enc = enc_box + bl * (M - 1) * 2 * D;
+    long long lo[D], hi[D];
+    for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(double(box[d])); hi[d] = ordered_bits(double(box[D + d])); }
     int node = parent[nbase + (M - 1) + leaf];
-    // a leaf is at most M - 1 levels below the root; the bound also ends the walk on a malformed parent chain
-    for (int level = 0; node >= 0 && node < M - 1 && level < M; ++level) {
-        const int side = kids[node].x == self ? 0 : 1;
-        for (int d = 0; d < 2 * D; ++d) cboxes[(size_t(node) * 2 + side) * 2 * D + d] = box[d];
-        __threadfence();                                   // publish the box before announcing the arrival
-        if (atomicAdd(&visit[bl * (M - 1) + node], 1) == 0) return;   // first arrival: the sibling will finish
-        __threadfence();
-        const T* other = cboxes + (size_t(node) * 2 + (1 - side)) * 2 * D;
+    // the radix tree over 64-bit keys is at most 64 levels deep; the bound also ends a walk on a malformed chain
+    for (int level = 0; node >= 0 && node < M - 1 && level < 128; ++level) {
+        bool grew = false;
+        long long* e = enc + size_t(node) * 2 * D;
         for (int d = 0; d < D; ++d) {
-            const T a = other[d], b = other[D + d];
-            box[d] = a < box[d] ? a : box[d];
-            box[D + d] = b > box[D + d] ? b : box[D + d];
+            grew |= lo[d] < atomicMin(&e[d], lo[d]);
+            grew |= hi[d] > atomicMax(&e[D + d], hi[d]);
         }
-        for (int d = 0; d < 2 * D; ++d) boxes[size_t(node) * 2 * D + d] = box[d];
-        self = node;
+        if (!grew) break;
         node = parent[nbase + node];
+    }
+}
+
+// decodes the internal boxes and stores, with every internal node, the boxes of its two children
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __restrict__ children,
+                                                                const long long* __restrict__ enc_box, T* node_box,
+                                                                T* __restrict__ child_box, int M, size_t total) {
+    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= total) return;
+    const size_t bl = t / (M - 1);
+    const int node = int(t - bl * (M - 1));
+    const size_t nbase = bl * (2 * size_t(M) - 1);
+    const int2 ch = children[t];
+    for (int d = 0; d < 2 * D; ++d) node_box[(nbase + node) * 2 * D + d] = T(from_ordered_bits(enc_box[t * 2 * D + d]));
+    for (int side = 0; side < 2; ++side) {
+        const int c = side == 0 ? ch.x : ch.y;
+        T* dst = child_box + (t * 2 + side) * 2 * D;
+        if (c < 0) {
+            const T* src = node_box + (nbase + (M - 1) + ~c) * 2 * D;       // leaf boxes were written by an earlier kernel
+            for (int d = 0; d < 2 * D; ++d) dst[d] = src[d];
+        } else {
+            const long long* src = enc_box + (bl * (M - 1) + c) * 2 * D;
+            for (int d = 0; d < 2 * D; ++d) dst[d] = T(from_ordered_bits(src[d]));
+        }
     }
 }
 
@@ -835,7 +869,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     T* box_lo = (T*)(bvh + lay.box_lo); T* box_hi = (T*)(bvh + lay.box_hi);
     T* node_box = (T*)(bvh + lay.node_box); T* leaf_rec = (T*)(bvh + lay.leaf_rec);
     int2* children = (int2*)(bvh + lay.children); int* parent = (int*)(bvh + lay.parent);
-    int* leaf_comp = (int*)(bvh + lay.leaf_comp); int* visit = (int*)(bvh + lay.visit);
+    int* leaf_comp = (int*)(bvh + lay.leaf_comp); long long* enc_box = (long long*)(bvh + lay.enc_box);
     uint32_t* ka = (uint32_t*)(bvh + lay.keys_a); uint32_t* kb = (uint32_t*)(bvh + lay.keys_b);
     uint32_t* va = (uint32_t*)(bvh + lay.vals_a); uint32_t* vb = (uint32_t*)(bvh + lay.vals_b);
     uint32_t* hist = (uint32_t*)(bvh + lay.hist);
@@ -853,11 +887,12 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         uint32_t* g_keys = (uint32_t*)(bvh + lay.g_keys);
         copy_kernel<uint32_t><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(where ? kb : ka, g_keys, n);
         bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, where ? vb : va, node_box,
-                                                                           leaf_rec, leaf_comp, visit, parent, M, n);
+                                                                           leaf_rec, leaf_comp, enc_box, parent, M, n);
         if (M > 1) {
             const size_t ni = BL * (M - 1);
             bvh_tree_kernel<<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(g_keys, children, parent, M, ni);
-            bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(children, parent, node_box, child_box, visit, M, n);
+            bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(parent, node_box, enc_box, M, n);
+            bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(children, enc_box, node_box, child_box, M, ni);
         }
     }
     if (XL > 0 && N > 0) {
