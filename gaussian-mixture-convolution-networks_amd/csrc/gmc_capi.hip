@@ -3,10 +3,12 @@
 #include "gmc_common.h"
 
 namespace gmc {
-int dense_forward(const void* mixture, const void* xes, void* out, const gmc_shape& s, hipStream_t stream);
+int dense_forward(const void* mixture, const void* xes, void* out, const gmc_shape& s, bool covariance_form,
+                  hipStream_t stream);
 size_t dense_backward_workspace_bytes(const gmc_shape& s);
 int dense_backward(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
-                   void* workspace, const gmc_shape& s, bool need_gm, bool need_gx, hipStream_t stream);
+                   void* workspace, const gmc_shape& s, bool need_gm, bool need_gx, bool covariance_form,
+                   hipStream_t stream);
 
 int check_shape(const gmc_shape* s) {
     if (!s) return GMC_E_NULL;
@@ -24,7 +26,7 @@ int check_shape(const gmc_shape* s) {
 
 extern "C" {
 
-int gmc_abi_version(void) { return 1; }
+int gmc_abi_version(void) { return 2; }
 
 const char* gmc_error_string(int code) {
     switch (code) {
@@ -40,13 +42,22 @@ const char* gmc_error_string(int code) {
     }
 }
 
-int gmc_eval_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream) {
+static int eval_fwd_impl(const void* mixture, const void* xes, void* out, const gmc_shape* shape, bool covariance_form,
+                         void* stream) {
     const int rc = gmc::check_shape(shape);
     if (rc != GMC_OK) return rc;
     const size_t n_out = size_t(shape->B) * shape->L * shape->N;
     if (n_out == 0) return GMC_OK;
     if (!out || !xes || (!mixture && shape->M > 0)) return GMC_E_NULL;
-    return gmc::dense_forward(mixture, xes, out, *shape, (hipStream_t)stream);
+    return gmc::dense_forward(mixture, xes, out, *shape, covariance_form, (hipStream_t)stream);
+}
+
+int gmc_eval_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream) {
+    return eval_fwd_impl(mixture, xes, out, shape, false, stream);
+}
+
+int gmc_eval_cov_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream) {
+    return eval_fwd_impl(mixture, xes, out, shape, true, stream);
 }
 
 size_t gmc_eval_bwd_workspace_bytes(const gmc_shape* shape) {
@@ -54,9 +65,9 @@ size_t gmc_eval_bwd_workspace_bytes(const gmc_shape* shape) {
     return gmc::dense_backward_workspace_bytes(*shape);
 }
 
-int gmc_eval_bwd(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
-                 void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
-                 int need_grad_xes, void* stream) {
+static int eval_bwd_impl(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                         void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
+                         int need_grad_xes, bool covariance_form, void* stream) {
     const int rc = gmc::check_shape(shape);
     if (rc != GMC_OK) return rc;
     const bool gm = need_grad_mixture != 0, gx = need_grad_xes != 0;
@@ -70,8 +81,22 @@ int gmc_eval_bwd(const void* grad_out, const void* mixture, const void* xes, voi
         if (workspace_bytes < gmc::dense_backward_workspace_bytes(*shape)) return GMC_E_WORKSPACE;
         if (!workspace) return GMC_E_NULL;
     }
-    return gmc::dense_backward(grad_out, mixture, xes, grad_mixture, grad_xes, workspace, *shape, gm, gx,
+    return gmc::dense_backward(grad_out, mixture, xes, grad_mixture, grad_xes, workspace, *shape, gm, gx, covariance_form,
                                (hipStream_t)stream);
+}
+
+int gmc_eval_bwd(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                 void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
+                 int need_grad_xes, void* stream) {
+    return eval_bwd_impl(grad_out, mixture, xes, grad_mixture, grad_xes, workspace, workspace_bytes, shape,
+                         need_grad_mixture, need_grad_xes, false, stream);
+}
+
+int gmc_eval_cov_bwd(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                     void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
+                     int need_grad_xes, void* stream) {
+    return eval_bwd_impl(grad_out, mixture, xes, grad_mixture, grad_xes, workspace, workspace_bytes, shape,
+                         need_grad_mixture, need_grad_xes, true, stream);
 }
 
 }  // extern "C"

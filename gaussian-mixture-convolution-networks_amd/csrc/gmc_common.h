@@ -37,13 +37,49 @@ template <int D> struct Derived {
     double w;
 };
 
+// `covariance_form`: the record stores the covariance; its inverse (transposed, as gm.evaluate packs it,
+// src/gmc/mixture.py:149) is formed here in double, so the covariance-form API needs no separate inversion pass.
 template <typename T, int D>
-__device__ __forceinline__ Derived<D> derive(const T* __restrict__ g) {
+__device__ __forceinline__ void load_inverse_covariance(const T* __restrict__ c, bool covariance_form, double (&m)[D][D]) {
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+#pragma unroll
+        for (int j = 0; j < D; ++j) m[i][j] = double(c[i * D + j]);
+    if (!covariance_form) return;
+    if constexpr (D == 2) {
+        const double det = m[0][0] * m[1][1] - m[0][1] * m[1][0];
+        const double a = m[0][0], b = m[0][1], cc = m[1][0], d = m[1][1];
+        // (S^-1)^T
+        m[0][0] = d / det; m[0][1] = -cc / det; m[1][0] = -b / det; m[1][1] = a / det;
+    } else {
+        double k[3][3];
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int i1 = i == 0 ? 1 : 0, i2 = i == 2 ? 1 : 2;
+#pragma unroll
+            for (int j = 0; j < 3; ++j) {
+                const int j1 = j == 0 ? 1 : 0, j2 = j == 2 ? 1 : 2;
+                const double minor = m[i1][j1] * m[i2][j2] - m[i1][j2] * m[i2][j1];
+                k[i][j] = ((i + j) & 1) ? -minor : minor;
+            }
+        }
+        const double det = m[0][0] * k[0][0] + m[0][1] * k[0][1] + m[0][2] * k[0][2];
+        // S^-1 = cofactor^T / det, hence (S^-1)^T = cofactor / det
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+#pragma unroll
+            for (int j = 0; j < 3; ++j) m[i][j] = k[i][j] / det;
+    }
+}
+
+template <typename T, int D>
+__device__ __forceinline__ Derived<D> derive(const T* __restrict__ g, bool covariance_form = false) {
     Derived<D> r;
     r.w = double(g[0]);
-    const T* c = g + 1 + D;
+    double cm[D][D];
+    load_inverse_covariance<T, D>(g + 1 + D, covariance_form, cm);
     if constexpr (D == 2) {
-        const double c00 = c[0], c01 = c[1], c10 = c[2], c11 = c[3];
+        const double c00 = cm[0][0], c01 = cm[0][1], c10 = cm[1][0], c11 = cm[1][1];
         const double det = c00 * c11 - c01 * c10;
         const double a00 = kHalfLog2e * c00, a01 = kHalfLog2e * 0.5 * (c01 + c10), a11 = kHalfLog2e * c11;
         const double u00 = sqrt(a00);
@@ -57,8 +93,8 @@ __device__ __forceinline__ Derived<D> derive(const T* __restrict__ g) {
         r.bound = fmax(fabs(u00 * b0) + fabs(u01 * b1), fabs(u11 * b1));
         r.norm = Kappa<2>::v * sqrt(det);
     } else {
-        const double c00 = c[0], c01 = c[1], c02 = c[2], c10 = c[3], c11 = c[4], c12 = c[5], c20 = c[6], c21 = c[7],
-                     c22 = c[8];
+        const double c00 = cm[0][0], c01 = cm[0][1], c02 = cm[0][2], c10 = cm[1][0], c11 = cm[1][1], c12 = cm[1][2],
+                     c20 = cm[2][0], c21 = cm[2][1], c22 = cm[2][2];
         const double det = c00 * (c11 * c22 - c12 * c21) - c01 * (c10 * c22 - c12 * c20) + c02 * (c10 * c21 - c11 * c20);
         const double a00 = kHalfLog2e * c00, a11 = kHalfLog2e * c11, a22 = kHalfLog2e * c22;
         const double a01 = kHalfLog2e * 0.5 * (c01 + c10), a02 = kHalfLog2e * 0.5 * (c02 + c20),
@@ -154,7 +190,7 @@ __device__ __forceinline__ T quad_form(const T* __restrict__ r, const T* __restr
 // caller needs no barrier of its own.
 template <typename T, int D, int GROUP = 1>
 __device__ __forceinline__ void stage_tile(const T* __restrict__ gaussians, int cnt, double amp_scale, T* lds,
-                                           int* counts /* LDS int[10] */) {
+                                           int* counts /* LDS int[10] */, bool covariance_form) {
     constexpr int S = Rec<T, D>::kStride;
     constexpr int G = 1 + D + D * D;
     const int tid = threadIdx.x;
@@ -163,7 +199,7 @@ __device__ __forceinline__ void stage_tile(const T* __restrict__ gaussians, int 
     Derived<D> dv;
     bool centred = false;
     if (active) {
-        dv = derive<T, D>(gaussians + size_t(tid) * G);
+        dv = derive<T, D>(gaussians + size_t(tid) * G, covariance_form);
         centred = !(dv.bound <= ShiftedBound<T>::v);
     }
     const unsigned long long mc = __ballot(active && centred);

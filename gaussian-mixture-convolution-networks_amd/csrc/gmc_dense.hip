@@ -59,7 +59,7 @@ __device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, int begin, 
 template <typename T, int D, int P>
 __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ mixture, const T* __restrict__ xes,
                                                           T* __restrict__ out, int L, int M, int N, int Bx, int Lx,
-                                                          int chunks, int n_mixtures) {
+                                                          int chunks, int n_mixtures, bool covariance_form) {
     constexpr int G = 1 + D + D * D;
     constexpr int S = Rec<T, D>::kStride;
     __shared__ __attribute__((aligned(16))) T lds[kTile * S];
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
 
     for (int g0 = 0; g0 < M; g0 += kTile) {
         const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
-        stage_tile<T, D>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts);
+        stage_tile<T, D>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts, covariance_form);
         const int n_shifted = counts[8];
         fwd_pairs<T, D, P, false>(lds, 0, n_shifted, x, acc);
         fwd_pairs<T, D, P, true>(lds, n_shifted, cnt, x, acc);
@@ -170,7 +170,8 @@ template <typename T, int D, int P, bool NEED_GM, bool NEED_GX>
 __global__ __launch_bounds__(kBlock) void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture,
                                                              const T* __restrict__ xes, T* __restrict__ sums,
                                                              T* __restrict__ grad_xes, int L, int M, int N, int Bx, int Lx,
-                                                             int chunks, int xes_shared, int n_mixtures) {
+                                                             int chunks, int xes_shared, int n_mixtures,
+                                                             bool covariance_form) {
     constexpr int G = 1 + D + D * D;
     constexpr int S = Rec<T, D>::kStride;
     constexpr int NR = Sums<D>::k;
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_rc_kernel(const T* __restrict
 
     for (int g0 = 0; g0 < M; g0 += kTile) {
         const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
-        stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0 / kHalfLog2e, lds, counts);
+        stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0 / kHalfLog2e, lds, counts, covariance_form);
         const int centred_start = counts[8], padded_total = counts[9];
         bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, false>(lds, block_sums, 0, centred_start, row, x, go, gx);
         bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, true>(lds, block_sums, centred_start, padded_total, row, x, go, gx);
@@ -257,10 +258,14 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_rc_kernel(const T* __restrict
 //   dw  = norm R0
 //   db  = w norm / (0.5 log2 e) * u^T R1
 //   dC  = -1/2 w norm * u^-1 R2 u^-T  +  cofactor(C) * w kappa R0 / (2 sqrt(det C))
+// In covariance form C = (S^-1)^T was formed on the fly from the stored covariance S and the matrix gradient is
+// carried on to S as the reference's Python layer does (transpose of pack_mixture's argument, then
+// MatrixInverse.backward, src/gmc/cpp/extensions/math/matrix_inverse.py:30-33):  dS = -S^-1 dC^T S^-1.
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void eval_bwd_epilogue_kernel(const T* __restrict__ mixture,
                                                                    const T* __restrict__ sums,
-                                                                   T* __restrict__ grad_mixture, size_t n_gaussians) {
+                                                                   T* __restrict__ grad_mixture, size_t n_gaussians,
+                                                                   bool covariance_form) {
     constexpr int G = 1 + D + D * D;
     constexpr int NR = Sums<D>::k;
     const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
@@ -268,73 +273,111 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_epilogue_kernel(const T* __re
     const T* g = mixture + i * G;
     const T* rs = sums + i * NR;
     T* o = grad_mixture + i * G;
-    const Derived<D> dv = derive<T, D>(g);
+    const Derived<D> dv = derive<T, D>(g, covariance_form);
+    double c[D][D];
+    load_inverse_covariance<T, D>(g + 1 + D, covariance_form, c);
     const double R0 = double(rs[0]);
     const double wn = dv.w * dv.norm;
     o[0] = T(dv.norm * R0);
-    const T* c = g + 1 + D;
+
+    // u as a full upper-triangular matrix, V = u^-1
+    double U[D][D], V[D][D];
+#pragma unroll
+    for (int r = 0; r < D; ++r)
+#pragma unroll
+        for (int q = 0; q < D; ++q) { U[r][q] = 0.0; V[r][q] = 0.0; }
     if constexpr (D == 2) {
-        const double u00 = dv.u[0], u01 = dv.u[1], u11 = dv.u[2];
-        const double r1[2] = {double(rs[1]), double(rs[2])};
-        const double k = wn / kHalfLog2e;
-        o[1] = T(k * (u00 * r1[0]));
-        o[2] = T(k * (u01 * r1[0] + u11 * r1[1]));
-        // V = u^-1 (upper triangular)
-        const double v00 = 1.0 / u00, v11 = 1.0 / u11, v01 = -u01 * v00 * v11;
-        const double s00 = double(rs[3]), s01 = double(rs[4]), s11 = double(rs[5]);
-        // A = V S V^T
-        const double m00 = v00 * s00 + v01 * s01, m01 = v00 * s01 + v01 * s11, m11 = v11 * s11;
-        const double a00 = m00 * v00 + m01 * v01, a01 = m01 * v11, a11 = m11 * v11;
-        const double det = double(c[0]) * double(c[3]) - double(c[1]) * double(c[2]);
-        const double kd = dv.w * Kappa<2>::v * R0 / (2.0 * sqrt(det));
-        o[3] = T(-0.5 * wn * a00 + double(c[3]) * kd);
-        o[4] = T(-0.5 * wn * a01 - double(c[2]) * kd);
-        o[5] = T(-0.5 * wn * a01 - double(c[1]) * kd);
-        o[6] = T(-0.5 * wn * a11 + double(c[0]) * kd);
+        U[0][0] = dv.u[0]; U[0][1] = dv.u[1]; U[1][1] = dv.u[2];
+        V[0][0] = 1.0 / U[0][0]; V[1][1] = 1.0 / U[1][1];
+        V[0][1] = -U[0][1] * V[0][0] * V[1][1];
     } else {
-        const double u00 = dv.u[0], u01 = dv.u[1], u02 = dv.u[2], u11 = dv.u[3], u12 = dv.u[4], u22 = dv.u[5];
-        const double r1[3] = {double(rs[1]), double(rs[2]), double(rs[3])};
-        const double k = wn / kHalfLog2e;
-        o[1] = T(k * (u00 * r1[0]));
-        o[2] = T(k * (u01 * r1[0] + u11 * r1[1]));
-        o[3] = T(k * (u02 * r1[0] + u12 * r1[1] + u22 * r1[2]));
-        const double v00 = 1.0 / u00, v11 = 1.0 / u11, v22 = 1.0 / u22;
-        const double v01 = -u01 * v00 * v11;
-        const double v12 = -u12 * v11 * v22;
-        const double v02 = -(u01 * v12 + u02 * v22) * v00;
-        const double s[3][3] = {{double(rs[4]), double(rs[5]), double(rs[6])},
-                                {double(rs[5]), double(rs[7]), double(rs[8])},
-                                {double(rs[6]), double(rs[8]), double(rs[9])}};
-        const double V[3][3] = {{v00, v01, v02}, {0.0, v11, v12}, {0.0, 0.0, v22}};
-        double m[3][3], a[3][3];
+        U[0][0] = dv.u[0]; U[0][1] = dv.u[1]; U[0][2] = dv.u[2]; U[1][1] = dv.u[3]; U[1][2] = dv.u[4]; U[2][2] = dv.u[5];
+        V[0][0] = 1.0 / U[0][0]; V[1][1] = 1.0 / U[1][1]; V[2][2] = 1.0 / U[2][2];
+        V[0][1] = -U[0][1] * V[0][0] * V[1][1];
+        V[1][2] = -U[1][2] * V[1][1] * V[2][2];
+        V[0][2] = -(U[0][1] * V[1][2] + U[0][2] * V[2][2]) * V[0][0];
+    }
+    // db = k u^T R1
+    const double k = wn / kHalfLog2e;
 #pragma unroll
-        for (int r = 0; r < 3; ++r)
+    for (int r = 0; r < D; ++r) {
+        double acc = 0.0;
 #pragma unroll
-            for (int q = 0; q < 3; ++q) m[r][q] = V[r][0] * s[0][q] + V[r][1] * s[1][q] + V[r][2] * s[2][q];
+        for (int q = 0; q <= r; ++q) acc += U[q][r] * double(rs[1 + q]);
+        o[1 + r] = T(k * acc);
+    }
+    // A = V R2 V^T
+    double s2[D][D], m[D][D], a[D][D];
+    {
+        int idx = 1 + D;
 #pragma unroll
-        for (int r = 0; r < 3; ++r)
+        for (int r = 0; r < D; ++r)
 #pragma unroll
-            for (int q = 0; q < 3; ++q) a[r][q] = m[r][0] * V[q][0] + m[r][1] * V[q][1] + m[r][2] * V[q][2];
-        double cc[3][3];
+            for (int q = r; q < D; ++q) { s2[r][q] = double(rs[idx]); s2[q][r] = s2[r][q]; ++idx; }
+    }
 #pragma unroll
-        for (int r = 0; r < 3; ++r)
+    for (int r = 0; r < D; ++r)
 #pragma unroll
-            for (int q = 0; q < 3; ++q) cc[r][q] = double(c[r * 3 + q]);
-        const double det = cc[0][0] * (cc[1][1] * cc[2][2] - cc[1][2] * cc[2][1]) -
-                           cc[0][1] * (cc[1][0] * cc[2][2] - cc[1][2] * cc[2][0]) +
-                           cc[0][2] * (cc[1][0] * cc[2][1] - cc[1][1] * cc[2][0]);
-        const double kd = dv.w * Kappa<3>::v * R0 / (2.0 * sqrt(det));
+        for (int q = 0; q < D; ++q) {
+            double acc = 0.0;
 #pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            const int r1i = r == 0 ? 1 : 0, r2i = r == 2 ? 1 : 2;
-#pragma unroll
-            for (int q = 0; q < 3; ++q) {
-                const int q1 = q == 0 ? 1 : 0, q2 = q == 2 ? 1 : 2;
-                const double sign = ((r + q) & 1) ? -1.0 : 1.0;
-                const double cof = sign * (cc[r1i][q1] * cc[r2i][q2] - cc[r1i][q2] * cc[r2i][q1]);
-                o[4 + r * 3 + q] = T(-0.5 * wn * a[r][q] + cof * kd);
-            }
+            for (int t = 0; t < D; ++t) acc += V[r][t] * s2[t][q];
+            m[r][q] = acc;
         }
+#pragma unroll
+    for (int r = 0; r < D; ++r)
+#pragma unroll
+        for (int q = 0; q < D; ++q) {
+            double acc = 0.0;
+#pragma unroll
+            for (int t = 0; t < D; ++t) acc += m[r][t] * V[q][t];
+            a[r][q] = acc;
+        }
+    double det;
+    if constexpr (D == 2) det = c[0][0] * c[1][1] - c[0][1] * c[1][0];
+    else det = c[0][0] * (c[1][1] * c[2][2] - c[1][2] * c[2][1]) - c[0][1] * (c[1][0] * c[2][2] - c[1][2] * c[2][0]) +
+               c[0][2] * (c[1][0] * c[2][1] - c[1][1] * c[2][0]);
+    const double kd = dv.w * Kappa<D>::v * R0 / (2.0 * sqrt(det));
+    double gc[D][D];
+#pragma unroll
+    for (int r = 0; r < D; ++r)
+#pragma unroll
+        for (int q = 0; q < D; ++q) {
+            double cof;
+            if constexpr (D == 2) {
+                cof = (r == q) ? c[1 - r][1 - q] : -c[q][r];
+            } else {
+                const int r1i = r == 0 ? 1 : 0, r2i = r == 2 ? 1 : 2, q1 = q == 0 ? 1 : 0, q2 = q == 2 ? 1 : 2;
+                cof = (((r + q) & 1) ? -1.0 : 1.0) * (c[r1i][q1] * c[r2i][q2] - c[r1i][q2] * c[r2i][q1]);
+            }
+            gc[r][q] = -0.5 * wn * a[r][q] + cof * kd;
+        }
+    if (!covariance_form) {
+#pragma unroll
+        for (int r = 0; r < D; ++r)
+#pragma unroll
+            for (int q = 0; q < D; ++q) o[1 + D + r * D + q] = T(gc[r][q]);
+    } else {
+        // X = C gC C, dS = -X^T
+        double x1[D][D];
+#pragma unroll
+        for (int r = 0; r < D; ++r)
+#pragma unroll
+            for (int q = 0; q < D; ++q) {
+                double acc = 0.0;
+#pragma unroll
+                for (int t = 0; t < D; ++t) acc += c[r][t] * gc[t][q];
+                x1[r][q] = acc;
+            }
+#pragma unroll
+        for (int r = 0; r < D; ++r)
+#pragma unroll
+            for (int q = 0; q < D; ++q) {
+                double acc = 0.0;
+#pragma unroll
+                for (int t = 0; t < D; ++t) acc += x1[r][t] * c[t][q];
+                o[1 + D + q * D + r] = T(-acc);
+            }
     }
 }
 
@@ -368,14 +411,14 @@ static void zero_async(T* p, size_t n, hipStream_t stream) {
 }
 
 template <typename T, int D>
-static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s, hipStream_t stream) {
+static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s, bool cov, hipStream_t stream) {
     const size_t BL = size_t(s.B) * s.L;
     if (BL == 0 || s.N == 0) return GMC_OK;
     if (s.M == 0) { zero_async(out, BL * s.N, stream); return GMC_OK; }
     const int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
     const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
     const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
-#define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks, int(BL))
+#define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks, int(BL), cov)
     switch (P) {
         case 8: GMC_FWD(8); break;
         case 4: GMC_FWD(4); break;
@@ -388,7 +431,7 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
 
 template <typename T, int D, bool GM, bool GX>
 static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T* sums, T* grad_xes, const gmc_shape& s,
-                            int xes_shared, hipStream_t stream) {
+                            int xes_shared, bool cov, hipStream_t stream) {
     const size_t BL = size_t(s.B) * s.L;
     // a workgroup covers 4 wavefronts x 16 P points; pick the largest P that wastes little of the last chunk
     int P = 16;
@@ -402,7 +445,7 @@ static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T
     const int span = 64 * P;
     const int chunks = (s.N + span - 1) / span;
     const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
-#define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL))
+#define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL), cov)
     switch (P) {
         case 16: GMC_BWD(16); break;
         case 8: GMC_BWD(8); break;
@@ -414,7 +457,7 @@ static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T
 
 template <typename T, int D>
 static int launch_bwd(const T* grad_out, const T* mixture, const T* xes, T* grad_mixture, T* grad_xes, T* sums,
-                      const gmc_shape& s, bool need_gm, bool need_gx, hipStream_t stream) {
+                      const gmc_shape& s, bool need_gm, bool need_gx, bool cov, hipStream_t stream) {
     constexpr int G = 1 + D + D * D;
     const size_t BL = size_t(s.B) * s.L;
     const size_t n_gauss = BL * s.M;
@@ -428,23 +471,25 @@ static int launch_bwd(const T* grad_out, const T* mixture, const T* xes, T* grad
     }
     if (need_gm) zero_async(sums, n_gauss * Sums<D>::k, stream);
     if (need_gx && xes_shared) zero_async(grad_xes, n_x, stream);
-    if (need_gm && need_gx) launch_bwd_main<T, D, true, true>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, stream);
-    else if (need_gm) launch_bwd_main<T, D, true, false>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, stream);
-    else if (need_gx) launch_bwd_main<T, D, false, true>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, stream);
+    if (need_gm && need_gx) launch_bwd_main<T, D, true, true>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, cov, stream);
+    else if (need_gm) launch_bwd_main<T, D, true, false>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, cov, stream);
+    else if (need_gx) launch_bwd_main<T, D, false, true>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, cov, stream);
     if (need_gm) {
         const size_t blocks = (n_gauss + kBlock - 1) / kBlock;
-        eval_bwd_epilogue_kernel<T, D><<<dim3(unsigned(blocks)), dim3(kBlock), 0, stream>>>(mixture, sums, grad_mixture, n_gauss);
+        eval_bwd_epilogue_kernel<T, D><<<dim3(unsigned(blocks)), dim3(kBlock), 0, stream>>>(mixture, sums, grad_mixture, n_gauss, cov);
     }
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
-int dense_forward(const void* mixture, const void* xes, void* out, const gmc_shape& s, hipStream_t stream) {
+int dense_forward(const void* mixture, const void* xes, void* out, const gmc_shape& s, bool covariance_form,
+                  hipStream_t stream) {
+    const bool cov = covariance_form;
     if (s.dtype == GMC_F32) {
-        if (s.D == 2) return launch_fwd<float, 2>((const float*)mixture, (const float*)xes, (float*)out, s, stream);
-        return launch_fwd<float, 3>((const float*)mixture, (const float*)xes, (float*)out, s, stream);
+        if (s.D == 2) return launch_fwd<float, 2>((const float*)mixture, (const float*)xes, (float*)out, s, cov, stream);
+        return launch_fwd<float, 3>((const float*)mixture, (const float*)xes, (float*)out, s, cov, stream);
     }
-    if (s.D == 2) return launch_fwd<double, 2>((const double*)mixture, (const double*)xes, (double*)out, s, stream);
-    return launch_fwd<double, 3>((const double*)mixture, (const double*)xes, (double*)out, s, stream);
+    if (s.D == 2) return launch_fwd<double, 2>((const double*)mixture, (const double*)xes, (double*)out, s, cov, stream);
+    return launch_fwd<double, 3>((const double*)mixture, (const double*)xes, (double*)out, s, cov, stream);
 }
 
 size_t dense_backward_workspace_bytes(const gmc_shape& s) {
@@ -454,8 +499,9 @@ size_t dense_backward_workspace_bytes(const gmc_shape& s) {
 }
 
 int dense_backward(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
-                   void* workspace, const gmc_shape& s, bool need_gm, bool need_gx, hipStream_t stream) {
-#define GMC_CALL(T, DD) launch_bwd<T, DD>((const T*)grad_out, (const T*)mixture, (const T*)xes, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, s, need_gm, need_gx, stream)
+                   void* workspace, const gmc_shape& s, bool need_gm, bool need_gx, bool covariance_form,
+                   hipStream_t stream) {
+#define GMC_CALL(T, DD) launch_bwd<T, DD>((const T*)grad_out, (const T*)mixture, (const T*)xes, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, s, need_gm, need_gx, covariance_form, stream)
     if (s.dtype == GMC_F32) return s.D == 2 ? GMC_CALL(float, 2) : GMC_CALL(float, 3);
     return s.D == 2 ? GMC_CALL(double, 2) : GMC_CALL(double, 3);
 #undef GMC_CALL

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class Shape(ctypes.Structure):
@@ -57,6 +57,8 @@ def lib() -> ctypes.CDLL:
     l.gmc_eval_bwd_workspace_bytes.restype = sz
     l.gmc_eval_bwd_workspace_bytes.argtypes = [shp]
     l.gmc_eval_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
+    l.gmc_eval_cov_fwd.argtypes = [vp, vp, vp, shp, vp]
+    l.gmc_eval_cov_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
     if hasattr(l, "gmc_bvh_bytes"):
         l.gmc_bvh_bytes.restype = sz
         l.gmc_bvh_bytes.argtypes = [shp]
@@ -125,15 +127,17 @@ def _p(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else ctypes.c_void_p(0)
 
 
-def eval_fwd(mixture: torch.Tensor, xes: torch.Tensor) -> torch.Tensor:
+def eval_fwd(mixture: torch.Tensor, xes: torch.Tensor, covariance_form: bool = False) -> torch.Tensor:
+    """`covariance_form`: the mixture holds covariances and the inversion happens inside the kernel"""
     shape = check_input(mixture, xes)
     out = torch.empty((shape.B, shape.L, shape.N), dtype=mixture.dtype, device=mixture.device)
+    fn = lib().gmc_eval_cov_fwd if covariance_form else lib().gmc_eval_fwd
     with torch.cuda.device(mixture.device):
-        check(lib().gmc_eval_fwd(_p(mixture), _p(xes), _p(out), ctypes.byref(shape), _stream(mixture.device)))
+        check(fn(_p(mixture), _p(xes), _p(out), ctypes.byref(shape), _stream(mixture.device)))
     return out
 
 
-def eval_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool):
+def eval_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool, covariance_form: bool = False):
     shape = check_input(mixture, xes)
     if grad_output.dim() != 3:
         raise RuntimeError("grad_output has wrong number of dimensions")
@@ -156,8 +160,9 @@ def eval_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool):
     with torch.cuda.device(dev):
         ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
         ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
-        check(lib().gmc_eval_bwd(_p(grad_output), _p(mixture), _p(xes), _p(grad_mixture), _p(grad_xes), _p(ws),
-                                 ws_bytes, ctypes.byref(shape), int(need_mixture), int(need_xes), _stream(dev)))
+        fn = lib().gmc_eval_cov_bwd if covariance_form else lib().gmc_eval_bwd
+        check(fn(_p(grad_output), _p(mixture), _p(xes), _p(grad_mixture), _p(grad_xes), _p(ws), ws_bytes,
+                 ctypes.byref(shape), int(need_mixture), int(need_xes), _stream(dev)))
     return grad_mixture, grad_xes
 
 

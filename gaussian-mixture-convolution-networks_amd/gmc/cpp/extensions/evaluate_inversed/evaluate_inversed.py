@@ -49,4 +49,27 @@ class EvaluateInversed(torch.autograd.Function):
         return (grad_mixture if want_mixture else None), (grad_xes if want_xes else None)
 
 
+class EvaluateCovariance(torch.autograd.Function):
+    """Same sum for a mixture that holds COVARIANCES: what gm.evaluate computes (src/gmc/mixture.py:144-149), with
+    the small-matrix inversion, its transpose and the repacking fused into the kernels, and the matrix gradient
+    carried on to the covariance in the backward kernel (-S^-1 g S^-1, math/matrix_inverse.py:30-33)."""
+
+    @staticmethod
+    def forward(ctx, mixture: torch.Tensor, xes: torch.Tensor):
+        mixture, xes = mixture.contiguous(), xes.contiguous()
+        values = _native.eval_fwd(mixture, xes, covariance_form=True)
+        ctx.save_for_backward(mixture, xes)
+        return values
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_output):
+        mixture, xes = ctx.saved_tensors
+        want_mixture, want_xes = ctx.needs_input_grad[:2]
+        grad_mixture, grad_xes = _native.eval_bwd(grad_output.contiguous(), mixture, xes, bool(want_mixture),
+                                                  bool(want_xes), covariance_form=True)
+        return (grad_mixture if want_mixture else None), (grad_xes if want_xes else None)
+
+
 apply = EvaluateInversed.apply
+apply_covariance = EvaluateCovariance.apply

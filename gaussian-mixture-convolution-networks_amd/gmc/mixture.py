@@ -99,7 +99,11 @@ def evaluate_inversed_with_amplitude_mixture(mixture: Tensor, xes: Tensor) -> Te
 
 
 def evaluate(mixture: Tensor, xes: Tensor, bvh: typing.Optional[BvhConfig] = None) -> Tensor:
-    """mixture holds covariances; returns [batch, layers, n_points]"""
+    """mixture holds covariances; returns [batch, layers, n_points].  The dense path inverts the covariances
+    inside the evaluation kernels (one read of the mixture, no intermediate tensors); the culled path inverts and
+    repacks first, as the reference does."""
+    if bvh is None:
+        return cppExtensionsEvaluateInversed.apply_covariance(mixture, xes)
     inv = mat_tools.inverse(covariances(mixture)).transpose(-1, -2)
     return evaluate_inversed(pack_mixture(weights(mixture), positions(mixture), inv), xes, bvh)
 

@@ -63,6 +63,18 @@ int gmc_eval_bwd(const void* grad_out, const void* mixture, const void* xes, voi
                  void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
                  int need_grad_xes, void* stream);
 
+/* ---- covariance-form evaluation ------------------------------------------------------------------
+ * gmc_eval_cov_fwd / gmc_eval_cov_bwd replace gm.evaluate (src/gmc/mixture.py:144-149) as a whole: `mixture` holds
+ * COVARIANCES; the inversion of src/gmc/mat_tools.py:34-36 (math/matrix_inverse_cuda.cu:18-31), its transpose and
+ * pack_mixture are fused into the Gaussian staging of the kernels, and the backward pass carries the matrix
+ * gradient on to the covariance as MatrixInverse.backward does (math/matrix_inverse.py:30-33: -S^-1 g S^-1).
+ * Same shapes, workspace and rules as gmc_eval_fwd / gmc_eval_bwd.
+ */
+int gmc_eval_cov_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream);
+int gmc_eval_cov_bwd(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                     void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
+                     int need_grad_xes, void* stream);
+
 /* ---- LBVH-culled evaluation ------------------------------------------------------------------------
  * Replaces lbvh::Bvh<D,T> (src/gmc/cpp/extensions/lbvh/bvh.h:97-148, bvh.cu:24-144: per-Gaussian boxes from
  * the contribution cutoff, Morton codes, sort, Karras node build, bottom-up box merge) and the point query

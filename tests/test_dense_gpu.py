@@ -169,6 +169,48 @@ def test_evaluate_covariance_form(golden_dir):
         assert rel_l2(got, ref) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_evaluate_covariance_form_fused_inverse(dtype, D):
+    """gm.evaluate with the inversion fused into the kernels: forward and all gradients against the oracle's
+    evaluate and its chain rule dS = -C dC C, and against the unfused composition (inverse + pack + evaluate)"""
+    g = torch.Generator().manual_seed(77 + D)
+    B, L, M, N = 3, 2, 70, 300
+    a = torch.rand((B, L, M, D, D), generator=g, dtype=torch.float64) * 2 - 1
+    cov = a @ a.transpose(-1, -2) + 0.05 * torch.eye(D, dtype=torch.float64)
+    w = torch.rand((B, L, M), generator=g, dtype=torch.float64) * 2 - 1
+    pos = torch.rand((B, L, M, D), generator=g, dtype=torch.float64) * 6 - 3
+    mix = gm.pack_mixture(w, pos, cov).to(dtype)
+    xes = (torch.rand((B, L, N, D), generator=g, dtype=torch.float64) * 8 - 4).to(dtype)
+    gout = torch.randn((B, L, N), generator=g, dtype=torch.float64).to(dtype)
+    m = mix.to(DEV).requires_grad_(True)
+    x = xes.to(DEV).requires_grad_(True)
+    out = gm.evaluate(m, x)
+    out.backward(gout.to(DEV))
+    # oracle on the rounded inputs
+    m64 = mix.numpy().astype(np.float64)
+    ref = o.evaluate(m64, xes.numpy())
+    c = np.linalg.inv(o.split(m64)[2])
+    inv_mix = np.concatenate([m64[..., :1 + D], c.reshape(B, L, M, D * D)], axis=-1)
+    rgm, rgx = o.evaluate_inversed_backward(gout.numpy(), inv_mix, xes.numpy())
+    gc = rgm[..., 1 + D:].reshape(B, L, M, D, D)
+    gs = -(c @ np.swapaxes(gc, -1, -2) @ c)
+    tol, fl = TOL[dtype], FLOOR[dtype]
+    gmix = m.grad.cpu().numpy()
+    assert rel_l2(out.detach().cpu().numpy(), ref, fl) <= tol
+    assert rel_l2(gmix[..., :1 + D], rgm[..., :1 + D], fl) <= tol
+    assert rel_l2(gmix[..., 1 + D:], gs.reshape(B, L, M, D * D), fl) <= tol * 2
+    assert rel_l2(x.grad.cpu().numpy(), rgx, fl) <= tol
+    # unfused composition through the inverse-covariance entry point
+    from gmc import mat_tools
+    m2 = mix.to(DEV).requires_grad_(True)
+    inv = mat_tools.inverse(gm.covariances(m2)).transpose(-1, -2)
+    out2 = gm.evaluate_inversed(gm.pack_mixture(gm.weights(m2), gm.positions(m2), inv), x.detach())
+    out2.backward(gout.to(DEV))
+    assert rel_l2(out2.detach().cpu().numpy(), out.detach().cpu().numpy(), fl) <= tol
+    assert rel_l2(m2.grad.cpu().numpy(), gmix, fl) <= tol * 2
+
+
 def _workload_check(name, **kw):
     wl, mix, xes, gout = synthetic.make_workload(name, **kw)
     out, gmix, gxes = _run(mix.numpy(), xes.numpy(), gout.numpy(), wl.dtype)

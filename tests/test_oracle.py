@@ -206,6 +206,35 @@ def test_backward_on_reference_literal_collections(golden_dir, D):
             assert np.abs(gx - xt.grad.numpy()).max() < 1e-12
 
 
+def test_covariance_form_chain_rule_by_central_differences():
+    """gm.evaluate = evaluate_inversed o inverse (src/gmc/mixture.py:144-149); its covariance gradient is
+    -S^-1 g S^-1 (math/matrix_inverse.py:30-33).  Checked here against central differences of o.evaluate."""
+    rng = np.random.default_rng(61)
+    for D in (2, 3):
+        a = rng.random((1, 1, 3, D, D)) * 2 - 1
+        cov = a @ np.swapaxes(a, -1, -2) + 0.3 * np.eye(D)
+        mix = np.concatenate([rng.random((1, 1, 3, 1)) + 0.2, rng.normal(size=(1, 1, 3, D)), cov.reshape(1, 1, 3, D * D)], -1)
+        xes = rng.normal(size=(1, 1, 5, D))
+        gout = rng.normal(size=(1, 1, 5))
+        c = np.linalg.inv(cov)
+        inv_mix = np.concatenate([mix[..., :1 + D], c.reshape(1, 1, 3, D * D)], -1)
+        gm_, _ = o.evaluate_inversed_backward(gout, inv_mix, xes)
+        gc = gm_[..., 1 + D:].reshape(1, 1, 3, D, D)
+        gs = -(c @ np.swapaxes(gc, -1, -2) @ c).reshape(1, 1, 3, D * D)
+        dx = 1e-6
+        for m in range(3):
+            for k in range(D * D):
+                i, j = divmod(k, D)
+                # symmetric perturbation keeps the matrix a covariance; it moves (i,j) and (j,i) together
+                mp, mm = mix.copy(), mix.copy()
+                for (r, q) in {(i, j), (j, i)}:
+                    mp[0, 0, m, 1 + D + r * D + q] += dx
+                    mm[0, 0, m, 1 + D + r * D + q] -= dx
+                num = ((o.evaluate(mp, xes) - o.evaluate(mm, xes)) * gout).sum() / (2 * dx)
+                ana = gs[0, 0, m, i * D + j] + (gs[0, 0, m, j * D + i] if i != j else 0.0)
+                assert abs(num - ana) < 1e-6 * max(1.0, abs(ana))
+
+
 def test_position_grad_is_minus_matched_xes_grad():
     mix, xes, gout = _rand_case(1, 1, 1, 9, 3, seed=19)
     gm, gx = o.evaluate_inversed_backward(gout, mix, xes)
