@@ -481,6 +481,15 @@ static int launch_bwd(const T* grad_out, const T* mixture, const T* xes, T* grad
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
+void launch_bwd_epilogue(const void* mixture, const void* sums, void* grad_mixture, size_t n_gaussians, int D, int dtype,
+                         bool covariance_form, hipStream_t stream) {
+    const dim3 grid(unsigned((n_gaussians + kBlock - 1) / kBlock));
+#define GMC_EPI(T, DD) eval_bwd_epilogue_kernel<T, DD><<<grid, dim3(kBlock), 0, stream>>>((const T*)mixture, (const T*)sums, (T*)grad_mixture, n_gaussians, covariance_form)
+    if (dtype == GMC_F32) { if (D == 2) GMC_EPI(float, 2); else GMC_EPI(float, 3); }
+    else { if (D == 2) GMC_EPI(double, 2); else GMC_EPI(double, 3); }
+#undef GMC_EPI
+}
+
 int dense_forward(const void* mixture, const void* xes, void* out, const gmc_shape& s, bool covariance_form,
                   hipStream_t stream) {
     const bool cov = covariance_form;

@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
     l.gmc_eval_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
     l.gmc_eval_cov_fwd.argtypes = [vp, vp, vp, shp, vp]
     l.gmc_eval_cov_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
+    l.gmc_eval_componentwise_fwd.argtypes = [vp, vp, vp, shp, ci, vp]
+    l.gmc_eval_componentwise_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, ci, vp]
     if hasattr(l, "gmc_bvh_bytes"):
         l.gmc_bvh_bytes.restype = sz
         l.gmc_bvh_bytes.argtypes = [shp]
@@ -163,6 +165,38 @@ def eval_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool, cova
         fn = lib().gmc_eval_cov_bwd if covariance_form else lib().gmc_eval_bwd
         check(fn(_p(grad_output), _p(mixture), _p(xes), _p(grad_mixture), _p(grad_xes), _p(ws), ws_bytes,
                  ctypes.byref(shape), int(need_mixture), int(need_xes), _stream(dev)))
+    return grad_mixture, grad_xes
+
+
+def eval_componentwise_fwd(mixture: torch.Tensor, xes: torch.Tensor, covariance_form: bool = False) -> torch.Tensor:
+    """values [B, L, N, M] of every (point, component) pair"""
+    shape = check_input(mixture, xes)
+    out = torch.empty((shape.B, shape.L, shape.N, shape.M), dtype=mixture.dtype, device=mixture.device)
+    with torch.cuda.device(mixture.device):
+        check(lib().gmc_eval_componentwise_fwd(_p(mixture), _p(xes), _p(out), ctypes.byref(shape), int(covariance_form),
+                                               _stream(mixture.device)))
+    return out
+
+
+def eval_componentwise_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool, covariance_form: bool = False):
+    shape = check_input(mixture, xes)
+    if tuple(grad_output.shape) != (shape.B, shape.L, shape.N, shape.M):
+        raise RuntimeError("grad_output has wrong shape")
+    if grad_output.dtype != mixture.dtype:
+        raise RuntimeError("grad_output dtype does not match with mixture dtype")
+    if not grad_output.is_contiguous():
+        raise RuntimeError("grad_output must be contiguous")
+    dev = mixture.device
+    grad_mixture = torch.empty_like(mixture) if need_mixture else torch.zeros_like(mixture)
+    grad_xes = torch.empty_like(xes) if need_xes else torch.zeros_like(xes)
+    if not (need_mixture or need_xes):
+        return grad_mixture, grad_xes
+    with torch.cuda.device(dev):
+        ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
+        ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
+        check(lib().gmc_eval_componentwise_bwd(_p(grad_output), _p(mixture), _p(xes), _p(grad_mixture), _p(grad_xes),
+                                               _p(ws), ws_bytes, ctypes.byref(shape), int(need_mixture), int(need_xes),
+                                               int(covariance_form), _stream(dev)))
     return grad_mixture, grad_xes
 
 

@@ -71,5 +71,28 @@ class EvaluateCovariance(torch.autograd.Function):
         return (grad_mixture if want_mixture else None), (grad_xes if want_xes else None)
 
 
+class EvaluateComponentwise(torch.autograd.Function):
+    """values [batch, layers, n_points, n_components] of every pair, without the sum over components
+    (evaluate_componentwise_inversed / evaluate_componentwise, src/gmc/mixture.py:152-185)"""
+
+    @staticmethod
+    def forward(ctx, mixture: torch.Tensor, xes: torch.Tensor, covariance_form: bool):
+        mixture, xes = mixture.contiguous(), xes.contiguous()
+        values = _native.eval_componentwise_fwd(mixture, xes, covariance_form)
+        ctx.save_for_backward(mixture, xes)
+        ctx.covariance_form = covariance_form
+        return values
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_output):
+        mixture, xes = ctx.saved_tensors
+        want_mixture, want_xes = ctx.needs_input_grad[:2]
+        grad_mixture, grad_xes = _native.eval_componentwise_bwd(grad_output.contiguous(), mixture, xes, bool(want_mixture),
+                                                                bool(want_xes), ctx.covariance_form)
+        return (grad_mixture if want_mixture else None), (grad_xes if want_xes else None), None
+
+
 apply = EvaluateInversed.apply
 apply_covariance = EvaluateCovariance.apply
+apply_componentwise = EvaluateComponentwise.apply

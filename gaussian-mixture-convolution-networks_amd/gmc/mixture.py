@@ -108,6 +108,16 @@ def evaluate(mixture: Tensor, xes: Tensor, bvh: typing.Optional[BvhConfig] = Non
     return evaluate_inversed(pack_mixture(weights(mixture), positions(mixture), inv), xes, bvh)
 
 
+def evaluate_componentwise_inversed(gaussians: Tensor, xes: Tensor) -> Tensor:
+    """gaussians hold inverse covariances; returns [batch, layers, n_points, n_components]"""
+    return cppExtensionsEvaluateInversed.apply_componentwise(gaussians, xes, False)
+
+
+def evaluate_componentwise(mixture: Tensor, xes: Tensor) -> Tensor:
+    """mixture holds covariances; returns [batch, layers, n_points, n_components]"""
+    return cppExtensionsEvaluateInversed.apply_componentwise(mixture, xes, True)
+
+
 def convert_priors_to_amplitudes2(weights: Tensor, covariances: Tensor) -> Tensor:
     d = covariances.shape[-1]
     return weights / (covariances.det().sqrt() * math.sqrt((2 * math.pi) ** d))

@@ -75,6 +75,18 @@ int gmc_eval_cov_bwd(const void* grad_out, const void* mixture, const void* xes,
                      void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
                      int need_grad_xes, void* stream);
 
+/* ---- component-wise evaluation --------------------------------------------------------------------
+ * Replaces evaluate_componentwise_inversed / evaluate_componentwise (src/gmc/mixture.py:152-185, pure torch in the
+ * reference): out [B][L][N][M] holds every pair's value without the sum over components; grad_out of the backward
+ * pass has the same shape.  covariance_form != 0: the mixture holds covariances (as gmc_eval_cov_*).  The
+ * workspace of the backward pass is gmc_eval_bwd_workspace_bytes(shape).
+ */
+int gmc_eval_componentwise_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, int covariance_form,
+                               void* stream);
+int gmc_eval_componentwise_bwd(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture,
+                               void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
+                               int need_grad_mixture, int need_grad_xes, int covariance_form, void* stream);
+
 /* ---- LBVH-culled evaluation ------------------------------------------------------------------------
  * Replaces lbvh::Bvh<D,T> (src/gmc/cpp/extensions/lbvh/bvh.h:97-148, bvh.cu:24-144: per-Gaussian boxes from
  * the contribution cutoff, Morton codes, sort, Karras node build, bottom-up box merge) and the point query

@@ -211,6 +211,41 @@ def test_evaluate_covariance_form_fused_inverse(dtype, D):
     assert rel_l2(m2.grad.cpu().numpy(), gmix, fl) <= tol * 2
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_componentwise(dtype, D):
+    """evaluate_componentwise_inversed (src/gmc/mixture.py:152-180): every pair's value; its sum over components is
+    evaluate_inversed; gradients for a per-pair upstream gradient against the oracle with one component at a time"""
+    for B, L, M, N, bc in ((2, 3, 7, 9, False), (1, 2, 300, 70, True), (2, 1, 257, 130, False)):
+        mix, xes, _ = _case(B, L, M, N, D, 700 + M, bc)
+        npdt = np.float32 if dtype == torch.float32 else np.float64
+        mix, xes = mix.astype(npdt), xes.astype(npdt)
+        g = torch.Generator().manual_seed(M)
+        gout = torch.randn((B, L, N, M), generator=g, dtype=torch.float64).numpy().astype(npdt)
+        m = torch.tensor(mix, device=DEV, requires_grad=True)
+        x = torch.tensor(xes, device=DEV, requires_grad=True)
+        vals = gm.evaluate_componentwise_inversed(m, x)
+        assert vals.shape == (B, L, N, M)
+        vals.backward(torch.tensor(gout, device=DEV))
+        tol, fl = TOL[dtype], FLOOR[dtype]
+        ref = np.stack([o.evaluate_inversed(mix[:, :, k:k + 1], xes) for k in range(M)], axis=-1)
+        assert rel_l2(vals.detach().cpu().numpy(), ref, fl) <= tol
+        assert rel_l2(vals.sum(-1).detach().cpu().numpy(), o.evaluate_inversed(mix, xes), fl) <= tol
+        rgm = np.zeros_like(mix, dtype=np.float64)
+        rgx = np.zeros(xes.shape, dtype=np.float64)
+        for k in range(M):
+            a, b_ = o.evaluate_inversed_backward(gout[..., k], mix[:, :, k:k + 1], xes)
+            rgm[:, :, k:k + 1] = a
+            rgx += b_
+        assert rel_l2(m.grad.cpu().numpy(), rgm, fl) <= tol
+        assert rel_l2(x.grad.cpu().numpy(), rgx, fl) <= tol
+    # covariance form equals the inverse form on inverted covariances
+    cov = torch.linalg.inv(torch.tensor(mix[..., 1 + D:].reshape(B, L, M, D, D), dtype=torch.float64))
+    mc = torch.cat([torch.tensor(mix[..., :1 + D], dtype=torch.float64), cov.reshape(B, L, M, D * D)], -1).to(dtype).to(DEV)
+    v2 = gm.evaluate_componentwise(mc, torch.tensor(xes, device=DEV))
+    assert rel_l2(v2.cpu().numpy(), ref, fl) <= 20 * tol
+
+
 def _workload_check(name, **kw):
     wl, mix, xes, gout = synthetic.make_workload(name, **kw)
     out, gmix, gxes = _run(mix.numpy(), xes.numpy(), gout.numpy(), wl.dtype)

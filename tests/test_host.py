@@ -100,3 +100,40 @@ def test_small_matrix_inverse_and_its_gradient():
         a2 = a.detach().clone().requires_grad_(True)
         torch.linalg.inv(a2).backward(up)
         assert torch.allclose(a.grad, a2.grad, atol=1e-10)
+
+
+def test_on_disk_formats_roundtrip(tmp_path):
+    """container versions 3..6 and the ASCII PLY layout of src/gmc/inout.py:12-141"""
+    from gmc import inout
+    g = torch.Generator().manual_seed(3)
+    w = torch.rand(2, 1, 5, generator=g) + 0.1
+    p = torch.rand(2, 1, 5, 3, generator=g)
+    a = torch.rand(2, 1, 5, 3, 3, generator=g)
+    c = a @ a.transpose(-1, -2) + torch.eye(3)
+    m = gm.pack_mixture(w, p, c)
+    inout.save(m, tmp_path / "m6.torch", meta_info={"note": "x"})
+    back, meta = inout.load(tmp_path / "m6.torch")
+    assert torch.equal(back, m) and meta == {"note": "x"}
+    # older containers store amplitudes
+    amp = gm.convert_priors_to_amplitudes(m)
+    torch.save({"type": "gm.Mixture", "version": 5, "data": amp, "meta_info": None}, tmp_path / "m5.torch")
+    assert torch.allclose(inout.load(tmp_path / "m5.torch")[0], m, atol=1e-6)
+    torch.save({"type": "gm.Mixture", "version": 4, "weights": gm.weights(amp), "positions": p, "covariances": c,
+                "meta_info": None}, tmp_path / "m4.torch")
+    assert torch.allclose(inout.load(tmp_path / "m4.torch")[0], m, atol=1e-6)
+    torch.save({"type": "gm.Mixture", "version": 3, "weights": gm.weights(amp)[:, 0], "positions": p[:, 0],
+                "covariances": c[:, 0], "meta_info": None}, tmp_path / "m3.torch")
+    assert torch.allclose(inout.load(tmp_path / "m3.torch")[0], m, atol=1e-6)
+    with pytest.raises(RuntimeError):
+        torch.save({"type": "other"}, tmp_path / "bad.torch")
+        inout.load(tmp_path / "bad.torch")
+    # PLY
+    inout.write_gm_to_ply2(m, str(tmp_path / "ply" / "gm"))
+    text = open(tmp_path / "ply" / "gm_b1_l0.ply").read().splitlines()
+    assert text[0] == "ply" and text[2] == "element component 5" and text[3] == "property float x"
+    assert text[12] == "property float weight" and text[13] == "end_header" and len(text) == 14 + 5
+    r = inout.read_gm_from_ply(str(tmp_path / "ply" / "gm_b1_l0.ply"))
+    assert torch.allclose(r, m[1:2], atol=1e-6)
+    prior = inout.read_gm_from_ply(str(tmp_path / "ply" / "gm_b1_l0.ply"), ismodel=True)
+    wn = w[1:2] / w[1:2].sum()
+    assert torch.allclose(gm.weights(prior), gm.convert_priors_to_amplitudes2(wn, c[1:2]), atol=1e-6)
