@@ -433,14 +433,19 @@ template <typename T, int D, bool GM, bool GX>
 static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T* sums, T* grad_xes, const gmc_shape& s,
                             int xes_shared, bool cov, hipStream_t stream) {
     const size_t BL = size_t(s.B) * s.L;
-    // a workgroup covers 4 wavefronts x 16 P points; pick the largest P that wastes little of the last chunk
-    int P = 16;
-    if (sizeof(T) == 8) P = 8;
-    while (P > 2) {
-        const int span = 64 * P;
-        const int chunks = (s.N + span - 1) / span;
-        if (double(chunks) * span <= 1.15 * double(s.N) && size_t(chunks) * BL >= 512) break;
-        P >>= 1;
+    // A workgroup covers 4 wavefronts x 16 P points.  Larger P amortises the per-Gaussian row reductions (about
+    // 4 (1 + D + D(D+1)/2) instructions per step and lane) over more pairs but pads the last chunk more; pick the P
+    // with the least modelled work that still leaves enough workgroups for the 256 CUs.
+    const int p_max = sizeof(T) == 8 ? 8 : 16;
+    const double pair_cost = D == 2 ? 21.0 : 34.0, reduce_cost = 4.0 * Sums<D>::k;
+    int P = 2;
+    double best = 1e300;
+    for (int cand = p_max; cand >= 2; cand >>= 1) {
+        const int span = 64 * cand;
+        const size_t chunks = (size_t(s.N) + span - 1) / span;
+        if (cand > 2 && chunks * BL < 256) continue;
+        const double cost = double(chunks) * span * (pair_cost + reduce_cost / cand);
+        if (cost < best) { best = cost; P = cand; }
     }
     const int span = 64 * P;
     const int chunks = (s.N + span - 1) / span;
