@@ -13,17 +13,15 @@
 //   -> bottom-up union of boxes with integer atomic min/max on order-preserving encodings.
 // Query points are Morton-sorted the same way so that a wavefront owns 64 neighbouring points.
 //
-// Traversal: one wavefront per 64 sorted points, ONE stack per wavefront (LDS).  A node is entered when any
-// lane's point lies in its box (ballot); node data is wave-uniform; at a leaf every lane evaluates the Gaussian
-// and lanes outside the leaf's own box add zero, which reproduces the per-point rule exactly.  Backward reduces
-// the per-Gaussian sums over the wavefront and issues one atomic per scalar, leaf visit and wavefront.
+// Traversal: one wavefront per 64 sorted points with ONE node stack per wavefront (LDS); lanes work on tree nodes
+// while the tree is descended and on points while the gathered leaves are evaluated (see bvh_traverse_kernel).
+// Backward reduces the per-Gaussian sums over the wavefront and issues one atomic per scalar, leaf and wavefront.
 #include "gmc_common.h"
 
 namespace gmc {
 
 int check_shape(const gmc_shape* s);
 
-constexpr int kStackDepth = 80;         // the radix tree over 64-bit unique keys is at most 64 levels deep
 constexpr double kSqFloor = 5.991464547107982;   // -2 ln 0.05 (lbvh/bvh.cu:194)
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -622,35 +620,86 @@ __device__ __forceinline__ T leaf_terms(const T* __restrict__ r, const T (&x)[D]
 
 template <int D> struct BvhSums { static constexpr int k = 1 + D + D * (D + 1) / 2; };
 
+constexpr int kStackCap = 512;          // soft capacity of the node stack (the array has 128 more)
+constexpr int kLeafFlush = 512;         // candidate leaves are evaluated whenever this many have gathered
+constexpr int kLeafCap = kLeafFlush + 128;
+constexpr int kTravWaves = 8;           // wavefronts per workgroup of the traversal (one workgroup per 64 points)
+constexpr int kTravBlock = kTravWaves * kWave;
+constexpr int kStageBatch = 32;         // candidate leaves a wavefront stages in LDS at a time
+
+template <typename T>
+__device__ __forceinline__ T wave_min(T v) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) { const T o = __shfl_xor(v, off, 64); v = o < v ? o : v; }
+    return v;
+}
+template <typename T>
+__device__ __forceinline__ T wave_max(T v) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) { const T o = __shfl_xor(v, off, 64); v = o > v ? o : v; }
+    return v;
+}
+
+// orders the LDS traffic of one wavefront: stores of some lanes before loads of other lanes
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Traversal of one tree for 64 Morton-neighbouring points by one workgroup of 8 wavefronts, in two alternating
+// phases.
+//   Phase 1 (wavefront 0, lanes = tree nodes): ONE stack of internal nodes in LDS; up to 64 of them are popped at
+//   a time, each lane fetches the two child boxes of its node and tests them against the bounding box of the 64
+//   points (a node that contains any of the points overlaps that box).  Overlapping internal children go back on
+//   the stack, overlapping leaves into a candidate list (ballot + prefix-popcount compaction).
+//   Phase 2 (all wavefronts, lanes = points): the candidates are dealt to the wavefronts; each stages 32 of its
+//   candidates (own box + evaluation record) in LDS with one memory round trip, then tests every staged leaf
+//   against each point with the leaf's OWN box (closed interval, lbvh/aabb.h:39-47) and evaluates it where it
+//   contains the point.  The per-point partial results of the wavefronts are added at the end.
+// Phase 1 only filters, phase 2 applies the per-point rule, so the result is the sum over the Gaussians whose own
+// box contains the point.  Dependent memory round trips: about one per tree level plus one per 64 visited nodes,
+// instead of one per visited node; the candidate lists vary a lot between point groups (dense regions), which
+// is why one group gets a whole workgroup.
 // MODE 0: forward.  MODE 1: backward (grad_out given; accumulates per-Gaussian sums and dL/dx).
-// W = points per wavefront (lanes W..63 idle).  The traversal is bound by the latency of dependent node loads,
-// not by lanes, so small inputs use W < 64: more wavefronts in flight and smaller node unions per wavefront.
-template <typename T, int D, int MODE, bool NEED_GM, bool NEED_GX, int W>
-__global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
+template <typename T, int D, int MODE, bool NEED_GM, bool NEED_GX>
+__global__ __launch_bounds__(kTravBlock) void bvh_traverse_kernel(
         const T* __restrict__ xes, const int* __restrict__ p_order, const T* __restrict__ node_box,
         const T* __restrict__ child_box, const int2* __restrict__ children, const T* __restrict__ leaf_rec,
         T* __restrict__ out, const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes,
         int L, int M, int N, int Bx, int Lx, int chunks, int xes_shared) {
     constexpr int RS = LeafRec<D>::kStride;
     constexpr int NR = BvhSums<D>::k;
-    __shared__ int stack_mem[kBlock / kWave][kStackDepth];
+    constexpr int LS = 2 * D + RS;          // scalars per staged leaf: own box, evaluation record
+    constexpr int kWaves = kTravWaves;
+    __shared__ int stack[kStackCap + 128];
+    __shared__ int leaves[kLeafCap];
+    __shared__ int shared_state[2];         // [0] candidates gathered, [1] nodes left on the stack
+    __shared__ __attribute__((aligned(16))) T staged_mem[kWaves][kStageBatch * LS];
     const int bl = blockIdx.x / chunks;
     const int chunk = blockIdx.x - bl * chunks;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const size_t xseg = size_t(xb) * Lx + xl;
-    const int wave = threadIdx.x >> 6;
-    int* stack = stack_mem[wave];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    T* staged = staged_mem[wave];
+    const unsigned long long below = (1ull << lane) - 1ull;
 
-    const int lane = threadIdx.x & 63;
-    const int j = (chunk * (kBlock / kWave) + wave) * W + lane;
-    const bool valid = lane < W && j < N;
+    // every wavefront holds the same 64 points, one per lane
+    const int j = chunk * kWave + lane;
+    const bool valid = j < N;
     const int pid = valid ? p_order[xseg * N + j] : 0;
     T x[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) x[d] = xes[(xseg * N + pid) * D + d];
     T g = T(0);
     if (MODE == 1) g = valid ? grad_out[size_t(bl) * N + pid] : T(0);
+    T glo[D], ghi[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        glo[d] = wave_min(valid ? x[d] : T(INFINITY));
+        ghi[d] = wave_max(valid ? x[d] : T(-INFINITY));
+    }
 
     const T* boxes = node_box + size_t(bl) * (2 * size_t(M) - 1) * 2 * D;
     const T* cboxes = child_box + size_t(bl) * (M - 1) * 4 * D;
@@ -661,8 +710,16 @@ __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
 #pragma unroll
     for (int d = 0; d < D; ++d) gx[d] = T(0);
 
-    auto visit_leaf = [&](int leaf, bool in) {
-        const T* r = recs + size_t(leaf) * RS;
+    // `lf` points to a staged leaf in LDS: own box first, evaluation record behind it (read only on a hit)
+    auto visit_leaf = [&](const T* lf) {
+        T bx[2 * D];
+#pragma unroll
+        for (int k = 0; k < 2 * D; ++k) bx[k] = lf[k];
+        const bool in = valid & inside_box<T, D>(x, bx);
+        if (__ballot(in) == 0ull) return;
+        T r[RS];
+#pragma unroll
+        for (int k = 0; k < RS; ++k) r[k] = lf[2 * D + k];
         T t[D], u[D];
         const T e = leaf_terms<T, D>(r, x, t, u);
         const T amp = r[D + D * (D + 1) / 2];
@@ -685,11 +742,9 @@ __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
                 for (int a = 0; a < D; ++a)
 #pragma unroll
                     for (int c = a; c < D; ++c) rs[k++] = rs[1 + a] * t[c];
-                // lanes W..63 hold zeros; with W == 16 all points sit in the first DPP row
-                constexpr int kLast = W == 16 ? 15 : 63;
 #pragma unroll
-                for (int i = 0; i < NR; ++i) rs[i] = W == 16 ? row_sum_to_lane15(rs[i]) : wave_sum_to_lane63(rs[i]);
-                if ((threadIdx.x & 63) == kLast) {
+                for (int i = 0; i < NR; ++i) rs[i] = wave_sum_to_lane63(rs[i]);
+                if (lane == 63) {
                     const int comp = reinterpret_cast<const int*>(r + D + D * (D + 1) / 2 + 1)[0];
                     T* dst = sums + (size_t(bl) * M + comp) * NR;
 #pragma unroll
@@ -698,49 +753,106 @@ __global__ __launch_bounds__(kBlock) void bvh_traverse_kernel(
             }
         }
     };
+    // phase 2: this wavefront's share of the candidates [0, n)
+    auto evaluate_share = [&](int n) {
+        const int per = (n + kWaves - 1) / kWaves;
+        const int begin = wave * per, end = begin + per < n ? begin + per : n;
+        for (int base = begin; base < end; base += kStageBatch) {
+            const int cnt = end - base < kStageBatch ? end - base : kStageBatch;
+            if (lane < cnt) {
+                const int leaf = leaves[base + lane];
+                T* dst = staged + lane * LS;
+#pragma unroll
+                for (int i = 0; i < 2 * D; ++i) dst[i] = boxes[(size_t(M - 1) + leaf) * 2 * D + i];
+#pragma unroll
+                for (int i = 0; i < RS; ++i) dst[2 * D + i] = recs[size_t(leaf) * RS + i];
+            }
+            wave_lds_fence();
+            for (int i = 0; i < cnt; ++i) visit_leaf(staged + i * LS);
+            wave_lds_fence();
+        }
+    };
 
     if (M == 1) {
-        T bx[2 * D];
-#pragma unroll
-        for (int i = 0; i < 2 * D; ++i) bx[i] = boxes[i];
-        const bool in = valid & inside_box<T, D>(x, bx);
-        if (__ballot(in) != 0ull) visit_leaf(0, in);
+        if (threadIdx.x == 0) leaves[0] = 0;
+        __syncthreads();
+        evaluate_share(1);
     } else {
-        int sp = 0;
-        stack[sp++] = 0;
-        // every iteration pops one node; a binary tree with M-1 internal nodes bounds the loop
-        for (int iter = 0; sp > 0 && iter < M; ++iter) {
-            const int node = __builtin_amdgcn_readfirstlane(stack[--sp]);
-            const int2 ch = kids[node];
-            // both child boxes in one go: 4 D wave-uniform scalars, independent of the link load above
-            T cb[4 * D];
+        if (threadIdx.x == 0) { stack[0] = 0; shared_state[0] = 0; shared_state[1] = 1; }
+        __syncthreads();
+        // every round retires at least one of the M-1 internal nodes, each of which is pushed at most once
+        for (int round = 0; round < M; ++round) {
+            if (wave == 0) {
+                int sp = shared_state[1], n_leaf = 0;
+                for (int iter = 0; sp > 0 && n_leaf < kLeafFlush && iter < M; ++iter) {
+                    wave_lds_fence();
+                    // wide pops only while the stack has room for 64 more entries; a narrow pop is a depth-first
+                    // step, which adds at most one entry per tree level
+                    const int k = sp <= kStackCap - 128 ? (sp < 64 ? sp : 64) : 1;
+                    const bool active = lane < k;
+                    const int node = active ? stack[sp - 1 - lane] : 0;
+                    sp -= k;
+                    const int2 ch = kids[node];
+                    T cb[4 * D];
 #pragma unroll
-            for (int i = 0; i < 4 * D; ++i) cb[i] = cboxes[size_t(node) * 4 * D + i];
-            const int c0 = __builtin_amdgcn_readfirstlane(ch.x), c1 = __builtin_amdgcn_readfirstlane(ch.y);
-            const bool in0 = valid & inside_box<T, D>(x, cb), in1 = valid & inside_box<T, D>(x, cb + 2 * D);
+                    for (int i = 0; i < 4 * D; ++i) cb[i] = cboxes[size_t(node) * 4 * D + i];
+                    bool push[2], hit[2];
 #pragma unroll
-            for (int side = 0; side < 2; ++side) {
-                const int c = side == 0 ? c0 : c1;
-                if (c >= M - 1 || ~c >= M) continue;                 // not a node of this tree
-                const bool in = side == 0 ? in0 : in1;
-                if (__ballot(in) != 0ull) {
-                    if (c < 0) visit_leaf(~c, in);
-                    else if (sp < kStackDepth) stack[sp++] = c;
+                    for (int side = 0; side < 2; ++side) {
+                        const int c = side == 0 ? ch.x : ch.y;
+                        bool ov = active & (c < M - 1) & (~c < M);          // a node of this tree
+#pragma unroll
+                        for (int d = 0; d < D; ++d)
+                            ov = ov & (cb[side * 2 * D + d] <= ghi[d]) & (cb[side * 2 * D + D + d] >= glo[d]);
+                        push[side] = ov & (c >= 0);
+                        hit[side] = ov & (c < 0);
+                    }
+                    wave_lds_fence();
+#pragma unroll
+                    for (int side = 0; side < 2; ++side) {
+                        const int c = side == 0 ? ch.x : ch.y;
+                        const unsigned long long mp = __ballot(push[side]), mh = __ballot(hit[side]);
+                        const int at = sp + __popcll(mp & below);
+                        if (push[side] && at < kStackCap + 128) stack[at] = c;     // always in range, see the pop rule
+                        sp += __popcll(mp);
+                        if (hit[side]) leaves[n_leaf + __popcll(mh & below)] = ~c;
+                        n_leaf += __popcll(mh);
+                    }
                 }
+                if (lane == 0) { shared_state[0] = n_leaf; shared_state[1] = sp; }
             }
+            __syncthreads();
+            const int n_leaf = shared_state[0], left_on_stack = shared_state[1];
+            evaluate_share(n_leaf);
+            __syncthreads();
+            if (left_on_stack == 0) break;
         }
     }
 
-    if (MODE == 0) {
-        if (valid) out[size_t(bl) * N + pid] = acc;
-    } else if (NEED_GX) {
-        if (valid) {
-            T* dst = grad_xes + (xseg * N + pid) * D;
+    // add the wavefronts' partial results per point (the staging area is free now)
+    __syncthreads();
+    T* red = &staged_mem[0][0];
+    constexpr int kVals = MODE == 0 ? 1 : D;
+    if (MODE == 0 || NEED_GX) {
 #pragma unroll
-            for (int d = 0; d < D; ++d) {
-                const T v = -g * gx[d];
-                if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
-            }
+        for (int d = 0; d < kVals; ++d) red[(wave * kVals + d) * kWave + lane] = MODE == 0 ? acc : gx[d];
+    }
+    __syncthreads();
+    if (wave != 0 || !valid) return;
+    if (MODE == 0) {
+        T v = T(0);
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) v += red[w * kWave + lane];
+        out[size_t(bl) * N + pid] = v;
+    } else if (NEED_GX) {
+        T* dst = grad_xes + (xseg * N + pid) * D;
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            T v = T(0);
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) v += red[(w * D + d) * kWave + lane];
+            v = -g * v;
+            if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
         }
     }
 }
@@ -913,14 +1025,6 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
-// points per wavefront of the traversal: keep at least ~8 wavefronts per SIMD (256 CUs x 4 SIMDs) in flight
-static int points_per_wave(size_t n_mixtures, int n_points) {
-    const size_t pts = n_mixtures * size_t(n_points);
-    if (pts >= size_t(64) * 8192) return 64;
-    if (pts >= size_t(32) * 8192) return 32;
-    return 16;
-}
-
 template <typename T, int D>
 static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, hipStream_t st) {
     const BvhLayout lay = bvh_layout(s);
@@ -931,15 +1035,11 @@ static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, 
         fill_zero_kernel<T><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(out, n);
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    const int W = points_per_wave(BL, s.N);
-    const int chunks = (s.N + 4 * W - 1) / (4 * W);
-    const dim3 grid(unsigned(BL * chunks));
-#define GMC_TRAV(WW) bvh_traverse_kernel<T, D, 0, false, false, WW><<<grid, dim3(kBlock), 0, st>>>( \
-        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const T*)(bvh + lay.child_box), \
-        (const int2*)(bvh + lay.children), (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N, \
-        s.Bx, s.Lx, chunks, 0)
-    if (W == 64) GMC_TRAV(64); else if (W == 32) GMC_TRAV(32); else GMC_TRAV(16);
-#undef GMC_TRAV
+    const int chunks = (s.N + kWave - 1) / kWave;
+    bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kTravBlock), 0, st>>>(
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const T*)(bvh + lay.child_box),
+        (const int2*)(bvh + lay.children), (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N,
+        s.Bx, s.Lx, chunks, 0);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
@@ -963,18 +1063,15 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, const ch
     }
     if (gm) zero(sums, n_g * NR);
     if (gx && xes_shared) zero(grad_xes, n_x);
-    const int W = points_per_wave(BL, s.N);
-    const int chunks = (s.N + 4 * W - 1) / (4 * W);
+    const int chunks = (s.N + kWave - 1) / kWave;
     const dim3 grid(unsigned(BL * chunks));
-#define GMC_TRAV(GM, GX, WW) bvh_traverse_kernel<T, D, 1, GM, GX, WW><<<grid, dim3(kBlock), 0, st>>>( \
+#define GMC_TRAV(GM, GX) bvh_traverse_kernel<T, D, 1, GM, GX><<<grid, dim3(kTravBlock), 0, st>>>( \
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const T*)(bvh + lay.child_box), \
         (const int2*)(bvh + lay.children), (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, s.L, s.M, s.N, \
         s.Bx, s.Lx, chunks, xes_shared)
-#define GMC_TRAV_W(GM, GX) do { if (W == 64) GMC_TRAV(GM, GX, 64); else if (W == 32) GMC_TRAV(GM, GX, 32); else GMC_TRAV(GM, GX, 16); } while (0)
-    if (gm && gx) GMC_TRAV_W(true, true);
-    else if (gm) GMC_TRAV_W(true, false);
-    else if (gx) GMC_TRAV_W(false, true);
-#undef GMC_TRAV_W
+    if (gm && gx) GMC_TRAV(true, true);
+    else if (gm) GMC_TRAV(true, false);
+    else if (gx) GMC_TRAV(false, true);
 #undef GMC_TRAV
     if (gm) bvh_bwd_epilogue_kernel<T, D><<<dim3(grid_for(n_g)), dim3(kBlock), 0, st>>>(mixture, sums, grad_mixture, n_g);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
