@@ -83,6 +83,12 @@ def bench_bvh(args):
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     t0 = time.perf_counter()
     for k in range(args.steps):

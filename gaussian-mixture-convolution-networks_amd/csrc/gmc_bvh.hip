@@ -47,8 +47,8 @@ struct BvhLayout {
     size_t total;
 };
 
-constexpr int kSortItems = 8;                       // items per lane and radix block
-constexpr int kSortChunk = kBlock * kSortItems;     // 2048
+constexpr int kSortItems = 2;                       // items per lane and radix block
+constexpr int kSortChunk = kBlock * kSortItems;     // 512: small chunks, many workgroups (the passes are latency-bound)
 constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the first bounds pass
 
 template <int D> struct LeafRec { static constexpr int kStride = (D == 2) ? 8 : 12; };
@@ -437,7 +437,7 @@ template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, const T* __restrict__ box_lo,
                                                            const T* __restrict__ box_hi, const uint32_t* __restrict__ order,
                                                            T* __restrict__ node_box, T* __restrict__ leaf_rec,
-                                                           int* __restrict__ leaf_comp, long long* __restrict__ enc_box,
+                                                           long long* __restrict__ enc_box,
                                                            int* __restrict__ parent, int M, size_t total) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
@@ -453,7 +453,6 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         node_box[node * 2 * D + d] = box_lo[gi * D + d];
         node_box[node * 2 * D + D + d] = box_hi[gi * D + d];
     }
-    leaf_comp[i] = comp;
     if (leaf < M - 1) {
         // empty box of internal node `leaf`: lower = +inf, upper = -inf in the ordered-integer encoding
         long long* e = enc_box + (bl * (M - 1) + leaf) * 2 * D;
@@ -944,22 +943,23 @@ __global__ void iota_segments_kernel(int* __restrict__ dst, int count, size_t to
 static unsigned grid_for(size_t n) { return unsigned((n + kBlock - 1) / kBlock); }
 
 // sorts `segments` segments of `count` (key, value) pairs held in (ka, va) on the key bits
-// [first_bit, first_bit + 8 * passes); returns 0 if the result is in the a buffers, 1 if in the b buffers
-static int radix_sort(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* hist, uint32_t* totals,
-                      int segments, int count, int first_bit, int passes, hipStream_t st) {
+// [first_bit, first_bit + 8 * passes), ping-ponging with (kb, vb); the last pass writes to (keys_out, vals_out)
+static void radix_sort(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* keys_out, uint32_t* vals_out,
+                       uint32_t* hist, uint32_t* totals, int segments, int count, int first_bit, int passes,
+                       hipStream_t st) {
     const int bps = (count + kSortChunk - 1) / kSortChunk;
     const dim3 grid(unsigned(size_t(segments) * bps));
     int cur = 0;
     for (int p = 0; p < passes; ++p) {
         uint32_t* kin = cur ? kb : ka; uint32_t* vin = cur ? vb : va;
         uint32_t* kout = cur ? ka : kb; uint32_t* vout = cur ? va : vb;
+        if (p == passes - 1) { kout = keys_out; vout = vals_out; }
         const int shift = first_bit + 8 * p;
         radix_hist_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, count, bps, shift, hist);
         radix_scan_kernel<<<dim3(unsigned(segments) * 256), dim3(kWave), 0, st>>>(hist, totals, bps);
         radix_scatter_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, vin, kout, vout, count, bps, shift, hist, totals);
         cur ^= 1;
     }
-    return cur;
 }
 
 template <typename T, int D>
@@ -995,11 +995,11 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         T* gb = (T*)(bvh + lay.g_bounds);
         launch_bounds_of<T, D>(mixture, G, 1, M, BL, parts, gb, st);
         morton_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, G, 1, M, gb, ka, va, n);
-        const int where = radix_sort(ka, va, kb, vb, hist, totals, int(BL), M, 0, 4, st);
         uint32_t* g_keys = (uint32_t*)(bvh + lay.g_keys);
-        copy_kernel<uint32_t><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(where ? kb : ka, g_keys, n);
-        bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, where ? vb : va, node_box,
-                                                                           leaf_rec, leaf_comp, enc_box, parent, M, n);
+        uint32_t* g_order = (uint32_t*)leaf_comp;            // the sorted payload IS the component id of every leaf
+        radix_sort(ka, va, kb, vb, g_keys, g_order, hist, totals, int(BL), M, 0, 4, st);
+        bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, node_box,
+                                                                           leaf_rec, enc_box, parent, M, n);
         if (M > 1) {
             const size_t ni = BL * (M - 1);
             bvh_tree_kernel<<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(g_keys, children, parent, M, ni);
@@ -1015,9 +1015,8 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
             launch_bounds_of<T, D>(xes, D, 0, N, XL, parts, pb, st);
             morton_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(xes, D, 0, N, pb, ka, va, n);
             // 16 Morton bits (65536 cells) are enough to make 64 consecutive points neighbours
-            const int where = radix_sort(ka, va, kb, vb, hist, totals, int(XL), N, 14, 2, st);
-            copy_kernel<uint32_t><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(
-                where ? vb : va, (uint32_t*)p_order, n);
+            // the sorted keys are not needed afterwards: they land in the spare key buffer
+            radix_sort(ka, va, kb, vb, ka, (uint32_t*)p_order, hist, totals, int(XL), N, 14, 2, st);
         } else {
             iota_segments_kernel<<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(p_order, N, n);
         }
