@@ -123,13 +123,13 @@ def bench_bvh(args):
 
 def cpu_baseline_bvh(mode: str):
     """CPU comparison for the culled path: the C restatement of the reference CPU loops with the per-pair box
-    test in front of each evaluation (the reference has no CPU BVH evaluator to restate), on the first 2000
-    query points of C5 with the boxes of the oracle's rule."""
+    test in front of each evaluation (the reference has no CPU BVH evaluator to restate), on 20000 query
+    points of the C5 distribution with the boxes of the oracle's rule."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import cpu_ref
     import gm_oracle
     from gmc import synthetic
-    wl, mix, xes, gout = synthetic.make_workload("C5", N=2000)
+    wl, mix, xes, gout = synthetic.make_workload("C5", N=20000)
     m, x, g = mix.numpy(), xes.numpy(), gout.numpy()
     lo, up = gm_oracle.gaussian_aabbs(m, mode=mode)
     threads, cores = 128, len(os.sched_getaffinity(0))
@@ -141,7 +141,7 @@ def cpu_baseline_bvh(mode: str):
     t_bwd = time.perf_counter() - t0
     return {"value": wl.pairs / (t_fwd + t_bwd), "unit": "dense-equivalent pairs/s (fwd+bwd)", "cores": cores,
             "threads": threads, "kind": "port",
-            "sample": f"C5 slice N=2000 of 100000 points, M=16384 ({wl.pairs:.3g} dense-equivalent pairs), brute-force "
+            "sample": f"C5 slice N=20000 of 100000 points, M=16384 ({wl.pairs:.3g} dense-equivalent pairs), brute-force "
                       f"box test per pair, fwd {t_fwd:.2f} s + bwd {t_bwd:.2f} s"}
 
 
