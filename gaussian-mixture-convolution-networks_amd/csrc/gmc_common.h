@@ -284,4 +284,36 @@ __global__ void fill_zero_kernel(T* p, size_t n) {
     for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = T(0);
 }
 
+// Workgroups are dealt round-robin to the 8 XCDs.  With at least kXcdAffineMin mixtures all point chunks of one
+// mixture go to one XCD, so that its L2 serves the repeated reads of the Gaussians (the grid then has
+// ceil(n_mixtures / 8) * 8 * chunks workgroups, surplus ones exit); with fewer mixtures chunks are dealt
+// plainly, otherwise a single mixture would occupy one XCD only.
+constexpr int kXcdAffineMin = 64;
+
+__device__ __forceinline__ void map_workgroup(int id, int chunks, int n_mixtures, int& bl, int& chunk) {
+    if (n_mixtures >= kXcdAffineMin) {
+        const int xcd = id & 7, slot = id >> 3;
+        bl = (slot / chunks) * 8 + xcd;
+        chunk = slot % chunks;
+    } else {
+        bl = id / chunks;
+        chunk = id - bl * chunks;
+    }
+}
+
+inline size_t grid_mixtures(size_t n_mixtures) {
+    return n_mixtures >= size_t(kXcdAffineMin) ? (n_mixtures + 7) / 8 * 8 : n_mixtures;
+}
+
+// Per-Gaussian partial sums of the backward pass, in the transformed coordinates y = u (x - b):
+//   R0 = sum_n e g,  R1_i = sum_n e g y_i,  R2_ij = sum_n e g y_i y_j (i <= j)     with e = exp2(-|y|^2)
+template <int D> struct Sums { static constexpr int k = 1 + D + D * (D + 1) / 2; };   // 6 / 10
+
+template <typename T>
+inline void zero_async(T* p, size_t n, hipStream_t stream) {
+    if (n == 0) return;
+    const size_t blocks = (n + 255) / 256;
+    fill_zero_kernel<T><<<dim3(unsigned(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream>>>(p, n);
+}
+
 }  // namespace gmc

@@ -124,13 +124,6 @@ void launch_bwd_epilogue(const void* mixture, const void* sums, void* grad_mixtu
                          bool covariance_form, hipStream_t stream);
 size_t dense_backward_workspace_bytes(const gmc_shape& s);
 
-template <typename T>
-static void zero_async(T* p, size_t n, hipStream_t stream) {
-    if (n == 0) return;
-    const size_t blocks = (n + 255) / 256;
-    fill_zero_kernel<T><<<dim3(unsigned(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream>>>(p, n);
-}
-
 template <typename T, int D>
 static int cw_forward(const T* mixture, const T* xes, T* out, const gmc_shape& s, bool cov, hipStream_t st) {
     const size_t BL = size_t(s.B) * s.L;

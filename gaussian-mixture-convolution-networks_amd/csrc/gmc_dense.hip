@@ -14,30 +14,15 @@
 //     into (dw, db, dC).
 #include "gmc_common.h"
 
+#include <type_traits>
+
 namespace gmc {
 
+// float32 forward pair kernel with y = u x - u b on the matrix cores (gmc_dense_mfma.hip)
+int dense_forward_f32(const float* mixture, const float* xes, float* out, const gmc_shape& s, bool covariance_form,
+                      hipStream_t stream);
+
 constexpr int kTile = 256;   // Gaussians staged per LDS tile (one per lane)
-
-// Workgroups are dealt round-robin to the 8 XCDs.  With at least kXcdAffineMin mixtures all point chunks of one
-// mixture go to one XCD, so that its L2 serves the repeated reads of the Gaussians (the grid then has
-// ceil(n_mixtures / 8) * 8 * chunks workgroups, surplus ones exit); with fewer mixtures chunks are dealt
-// plainly, otherwise a single mixture would occupy one XCD only.
-constexpr int kXcdAffineMin = 64;
-
-__device__ __forceinline__ void map_workgroup(int id, int chunks, int n_mixtures, int& bl, int& chunk) {
-    if (n_mixtures >= kXcdAffineMin) {
-        const int xcd = id & 7, slot = id >> 3;
-        bl = (slot / chunks) * 8 + xcd;
-        chunk = slot % chunks;
-    } else {
-        bl = id / chunks;
-        chunk = id - bl * chunks;
-    }
-}
-
-static size_t grid_mixtures(size_t n_mixtures) {
-    return n_mixtures >= size_t(kXcdAffineMin) ? (n_mixtures + 7) / 8 * 8 : n_mixtures;
-}
 
 template <typename T, int D, int P, bool CENTRED>
 __device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, int begin, int end, const T (&x)[P][D], T (&acc)[P]) {
@@ -98,10 +83,6 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
         if (n < N) out[size_t(bl) * N + n] = acc[p];
     }
 }
-
-// Per-Gaussian partial sums of the backward pass, in the transformed coordinates y = u (x - b):
-//   R0 = sum_n e g,  R1_i = sum_n e g y_i,  R2_ij = sum_n e g y_i y_j (i <= j)     with e = exp2(-|y|^2)
-template <int D> struct Sums { static constexpr int k = 1 + D + D * (D + 1) / 2; };   // 6 / 10
 
 // Backward pair kernel, "4 x 16" wavefront layout.  The 64 lanes of a wavefront form 4 DPP rows of 16 lanes:
 // row r works on Gaussian 4k + r of the tile in step k, column c on the points {c, c + 16, ..., c + 16 (P-1)} of
@@ -403,18 +384,12 @@ static int pick_points_per_lane(int N, int BL) {
     return best;
 }
 
-template <typename T>
-static void zero_async(T* p, size_t n, hipStream_t stream) {
-    if (n == 0) return;
-    const size_t blocks = (n + 255) / 256;
-    fill_zero_kernel<T><<<dim3(unsigned(blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream>>>(p, n);
-}
-
 template <typename T, int D>
 static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s, bool cov, hipStream_t stream) {
     const size_t BL = size_t(s.B) * s.L;
     if (BL == 0 || s.N == 0) return GMC_OK;
     if (s.M == 0) { zero_async(out, BL * s.N, stream); return GMC_OK; }
+    if constexpr (std::is_same<T, float>::value) return dense_forward_f32(mixture, xes, out, s, cov, stream);
     const int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
     const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
     const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
