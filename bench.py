@@ -225,7 +225,7 @@ def main():
                                "the time, are inside the event pair)",
                      "bound": "valu", "achieved": bwd_tf, "peak": peak, "unit": "TFLOP/s", "frac": bwd_tf / peak,
                      "traffic": traffic, "launch_ms": bwd_ms, "flop_per_pair": FLOP_BWD[D]},
-        "roofline_fwd": {"kernel": "eval_fwd_kernel", "bound": "valu", "achieved": fwd_tf, "peak": peak,
+        "roofline_fwd": {"kernel": "eval_fwd_mfma_kernel" if dt == "f32" else "eval_fwd_kernel", "bound": "valu", "achieved": fwd_tf, "peak": peak,
                          "unit": "TFLOP/s", "frac": fwd_tf / peak, "launch_ms": fwd_ms, "flop_per_pair": FLOP_FWD[D]},
     }
     if not args.no_cpu_baseline:
