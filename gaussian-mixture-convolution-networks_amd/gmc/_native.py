@@ -16,11 +16,15 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class Shape(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int) for n in ("B", "L", "M", "N", "D", "Bx", "Lx", "dtype")]
+
+
+class ConvShape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int) for n in ("B", "Cin", "Cout", "Nd", "Nk", "D", "dtype")]
 
 
 class BvhConfigC(ctypes.Structure):
@@ -61,6 +65,9 @@ def lib() -> ctypes.CDLL:
     l.gmc_eval_cov_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
     l.gmc_eval_componentwise_fwd.argtypes = [vp, vp, vp, shp, ci, vp]
     l.gmc_eval_componentwise_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, ci, vp]
+    cshp = ctypes.POINTER(ConvShape)
+    l.gmc_convolution_fwd.argtypes = [vp, vp, vp, cshp, vp]
+    l.gmc_convolution_bwd.argtypes = [vp, vp, vp, vp, vp, cshp, ci, ci, vp]
     if hasattr(l, "gmc_bvh_bytes"):
         l.gmc_bvh_bytes.restype = sz
         l.gmc_bvh_bytes.argtypes = [shp]
@@ -279,3 +286,56 @@ def eval_bvh_bwd(grad_output, mixture, xes, bvh: Bvh, need_mixture: bool, need_x
                                      _p(ws), ws_bytes, ctypes.byref(shape), int(need_mixture), int(need_xes),
                                      _stream(dev)))
     return grad_mixture, grad_xes
+
+
+def check_convolution_input(data: torch.Tensor, kernels: torch.Tensor) -> ConvShape:
+    """Rules and messages of convolution::forward_impl_t (src/gmc/cpp/extensions/convolution/implementation_forward.h:35-43);
+    its n_batch x n_layers < 65535 grid limit does not apply here."""
+    if data.dim() != 4 or kernels.dim() != 4:
+        raise RuntimeError("data and kernels must have 4 dimensions")
+    d = n_dimensions(data)
+    if data.shape[2] < 1 or kernels.shape[2] < 1:
+        raise RuntimeError("number of components must be greater 1 for this implementation")
+    if data.shape[1] != kernels.shape[1]:
+        raise RuntimeError("number of input feature maps must agree with the second kernel dimension")
+    if n_dimensions(kernels) != d:
+        raise RuntimeError("number of dimensions of data and kernel must agree")
+    if data.dtype != kernels.dtype:
+        raise RuntimeError("kernel and data dtypes must agree")
+    if data.dtype not in (torch.float32, torch.float64):
+        raise RuntimeError("unsupported datatype: the convolution is implemented for float32 and float64")
+    if data.device != kernels.device:
+        raise RuntimeError("data and kernel devices must agree")
+    if not data.is_contiguous() or not kernels.is_contiguous():
+        raise RuntimeError("data and kernels must be contiguous")
+    if not data.is_cuda:
+        raise RuntimeError("gmc_hip convolves on an AMD GPU only: data and kernels must be HIP ('cuda') tensors; "
+                           "this build has no CPU implementation")
+    return ConvShape(data.shape[0], data.shape[1], kernels.shape[0], data.shape[2], kernels.shape[2], d,
+                     GMC_F32 if data.dtype == torch.float32 else GMC_F64)
+
+
+def convolution_fwd(data: torch.Tensor, kernels: torch.Tensor) -> torch.Tensor:
+    shape = check_convolution_input(data, kernels)
+    out = torch.empty((shape.B, shape.Cout, shape.Nd * shape.Cin * shape.Nk, data.shape[-1]), dtype=data.dtype,
+                      device=data.device)
+    with torch.cuda.device(data.device):
+        check(lib().gmc_convolution_fwd(_p(data), _p(kernels), _p(out), ctypes.byref(shape), _stream(data.device)))
+    return out
+
+
+def convolution_bwd(grad_out: torch.Tensor, data: torch.Tensor, kernels: torch.Tensor, need_data: bool = True,
+                    need_kernels: bool = True):
+    """-> (grad_data, grad_kernels); a gradient that is not asked for comes back as zeros, like the reference's"""
+    shape = check_convolution_input(data, kernels)
+    expected = (shape.B, shape.Cout, shape.Nd * shape.Cin * shape.Nk, data.shape[-1])
+    if tuple(grad_out.shape) != expected or grad_out.dtype != data.dtype or grad_out.device != data.device:
+        raise RuntimeError("grad_output must have the shape, dtype and device of the convolution result")
+    if not grad_out.is_contiguous():
+        raise RuntimeError("grad_output must be contiguous")
+    grad_data = torch.empty_like(data) if need_data else torch.zeros_like(data)
+    grad_kernels = torch.empty_like(kernels) if need_kernels else torch.zeros_like(kernels)
+    with torch.cuda.device(data.device):
+        check(lib().gmc_convolution_bwd(_p(grad_out), _p(data), _p(kernels), _p(grad_data), _p(grad_kernels),
+                                        ctypes.byref(shape), int(need_data), int(need_kernels), _stream(data.device)))
+    return grad_data, grad_kernels

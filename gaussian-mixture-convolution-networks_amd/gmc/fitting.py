@@ -1,0 +1,59 @@
+"""ReLU transfer fitting on top of the evaluation path: the part of the reference's src/gmc/fitting.py that calls
+gm.evaluate with the mixture's own centres as query points (initial_approx_to_relu :279-284,
+fixed_point_iteration_to_relu :287-312, generate_random_sampling :315-322).  The evaluations run through the HIP
+kernels (covariance-form entry points); the element-wise updates around them are torch operations on the
+[batch, layers, components] weight tensors.  The tree-based reduction fitters of that file are not part of this
+package."""
+import typing
+
+import torch
+from torch import Tensor
+
+from . import mixture as gm
+
+
+def _relu(t: Tensor) -> Tensor:
+    return torch.clamp(t, min=0)
+
+
+def initial_approx_to_relu(mixture: Tensor, constant: Tensor) -> Tensor:
+    """components whose weight does not lift the constant above zero are replaced by -relu(constant)"""
+    w = gm.weights(mixture)
+    c = constant.unsqueeze(-1)
+    new_w = torch.where(w + c > 0, w, -_relu(c).expand_as(w))
+    return gm.pack_mixture(new_w, gm.positions(mixture), gm.covariances(mixture))
+
+
+def fixed_point_iteration_to_relu(target_mixture: Tensor, target_constant: Tensor, fitting_mixture: Tensor,
+                                  n_iter: int = 1) -> typing.Tuple[Tensor, Tensor]:
+    """Weights for `fitting_mixture` (positions and covariances stay) such that it matches
+    relu(target_mixture + target_constant) - relu(target_constant) at its own centres, by the multiplicative
+    update x <- |x| (b + 0.05) / (fit(centres) + 0.05).  Returns (mixture, relu(target_constant))."""
+    assert gm.is_valid_mixture_and_constant(target_mixture, target_constant)
+    assert gm.is_valid_mixture(fitting_mixture)
+    assert gm.n_batch(target_mixture) == gm.n_batch(fitting_mixture)
+    assert gm.n_layers(target_mixture) == gm.n_layers(fitting_mixture)
+    assert gm.n_dimensions(target_mixture) == gm.n_dimensions(fitting_mixture)
+    assert target_mixture.device == fitting_mixture.device
+
+    centres = gm.positions(fitting_mixture).contiguous()
+    covariances = gm.covariances(fitting_mixture)
+    out_constant = _relu(target_constant)
+    goal = _relu(gm.evaluate(target_mixture, centres) + target_constant.unsqueeze(-1)) - out_constant.unsqueeze(-1)
+
+    x = gm.weights(fitting_mixture).abs() + 0.1
+    for _ in range(n_iter):
+        x = x.abs()
+        current = gm.evaluate(gm.pack_mixture(x, centres, covariances), centres)
+        x = x * (goal + 0.05) / (current + 0.05)
+    return gm.pack_mixture(x, centres, covariances), out_constant
+
+
+def generate_random_sampling(m: Tensor, n: int) -> Tensor:
+    """n uniform positions per (batch, layer) inside the box of the centres widened by one standard deviation"""
+    md = m.detach()
+    sd = torch.sqrt(torch.diagonal(gm.covariances(md), dim1=-2, dim2=-1))
+    hi = torch.max(gm.positions(md) + sd, dim=2, keepdim=True)[0]
+    lo = torch.min(gm.positions(md) - sd, dim=2, keepdim=True)[0]
+    u = torch.rand(gm.n_batch(m), gm.n_layers(m), n, gm.n_dimensions(m), device=m.device, dtype=m.dtype)
+    return u * (hi - lo) + lo

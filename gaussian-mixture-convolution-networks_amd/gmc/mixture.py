@@ -72,6 +72,16 @@ def is_valid_mixture(mixture: Tensor) -> bool:
     return True
 
 
+def is_valid_mixture_and_constant(mixture: Tensor, constant: Tensor) -> bool:
+    """a per-(batch or 1, layer) constant that is added to the mixture's values (src/gmc/mixture.py:188-204)"""
+    assert is_valid_mixture(mixture)
+    assert constant.dim() == 2
+    assert constant.shape[0] in (1, mixture.shape[0])
+    assert constant.shape[1] == mixture.shape[1]
+    assert constant.device == mixture.device
+    return True
+
+
 def integrate(mixture: Tensor) -> Tensor:
     return weights(mixture).sum(dim=-1)
 

@@ -87,6 +87,22 @@ int gmc_eval_componentwise_bwd(const void* grad_out, const void* mixture, const 
                                void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
                                int need_grad_mixture, int need_grad_xes, int covariance_form, void* stream);
 
+/* ---- closed-form convolution of Gaussian mixtures ----------------------------------------------------
+ * Replaces convolution::forward_impl / backward_impl (src/gmc/cpp/extensions/convolution/implementation_forward.h:27-103,
+ * implementation_backward.h:27-128, bound to Python at convolution/binding.py:21-43), the step that produces the
+ * mixtures the evaluation consumes (src/gmc/modules.py:163):
+ *   data [B][Cin][Nd][1+D+D*D], kernels [Cout][Cin][Nk][1+D+D*D] (covariance form)
+ *   out  [B][Cout][Nd*Cin*Nk][1+D+D*D],  out[b][co][cd + Nd*(ci + Cin*k)] = (w_d*w_k, b_d + b_k, S_d + S_k)
+ * Backward: grad_data and grad_kernels are fully written (no pre-zeroing needed); a flag of 0 leaves its output
+ * untouched.  No workspace.
+ */
+typedef struct gmc_conv_shape {
+    int B, Cin, Cout, Nd, Nk, D, dtype;
+} gmc_conv_shape;
+int gmc_convolution_fwd(const void* data, const void* kernels, void* out, const gmc_conv_shape* shape, void* stream);
+int gmc_convolution_bwd(const void* grad_out, const void* data, const void* kernels, void* grad_data, void* grad_kernels,
+                        const gmc_conv_shape* shape, int need_grad_data, int need_grad_kernels, void* stream);
+
 /* ---- LBVH-culled evaluation ------------------------------------------------------------------------
  * Replaces lbvh::Bvh<D,T> (src/gmc/cpp/extensions/lbvh/bvh.h:97-148, bvh.cu:24-144: per-Gaussian boxes from
  * the contribution cutoff, Morton codes, sort, Karras node build, bottom-up box merge) and the point query

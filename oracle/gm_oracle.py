@@ -14,6 +14,10 @@ src/gmc/cpp/extensions/ unless they start with src/):
   inside_mask / evaluate_*_bvh   lbvh/aabb.h:39-47, lbvh/query.h:13-66 (culled sum = sum over leaves whose own
                                  box contains the point; internal boxes are exact unions, lbvh/bvh.cu:501-506)
   morton30                       lbvh/morton_code.h:77-85,145-168
+  convolution_forward/backward   convolution/implementation_forward.h:27-103, implementation_backward.h:27-128,
+                                 index order util/helper.h:11-24
+  fixed_point_iteration_to_relu  src/gmc/fitting.py:287-312
+  batch_norm_forward             src/gmc/modules.py:374-425 (sampling positions are an argument here)
 
 Pinning status (what checks each function independently of its own formula; see tests/test_oracle.py):
   evaluate_inversed            known answer 1/pi (src/gmc/test_cpp_eval.py:25-28), scipy multivariate_normal,
@@ -24,6 +28,15 @@ Pinning status (what checks each function independently of its own formula; see 
   gaussian_aabbs (tight)       closed form: box of the ellipsoid {t : t^T C t <= s^2}, checked by sampling it
   gaussian_aabbs (reference)   PARITY UNPINNED: no reference test or fixture covers compute_aabbs; restated by
                                reading the code (glm is column-major); in 2-D it must equal the tight box (pinned)
+  convolution_forward          closed form (sum of independent Gaussians) checked as the reference's own test does:
+                               scipy.signal.fftconvolve of the sampled operands (src/gmc/test_mixture.py:108-136)
+  convolution_backward         central differences of convolution_forward (the reference uses gradcheck,
+                               src/gmc/test_mixture.py:138-152)
+  fixed_point_iteration_to_relu, batch_norm_forward
+                               literal restatements on top of evaluate(); checked through their fixed points and
+                               invariants (a mixture that already equals relu(target) is reproduced; unit variance
+                               and zero mean of the normalised samples); PARITY UNPINNED beyond that: the
+                               reference holds no test for either
   evaluate_inversed_bvh        PARITY UNPINNED against the reference (its composed BVH evaluator is absent from
                                the snapshot); pinned mathematically as a brute-force masked dense sum
 """
@@ -346,3 +359,72 @@ def morton30(p01: np.ndarray, resolution: int = 1024) -> np.ndarray:
     if p01.shape[-1] == 3:
         code = code + expand_bits3(q[..., 2])
     return code.astype(np.uint32)
+
+
+# ---- closed-form convolution of Gaussian mixtures ------------------------------------------------------------
+
+def convolution_forward(data: np.ndarray, kernels: np.ndarray) -> np.ndarray:
+    """data [B, Cin, Nd, G] (covariance form), kernels [Cout, Cin, Nk, G] -> [B, Cout, Nd*Cin*Nk, G].
+    Output component index = component_in + Nd * (channel_in + Cin * component_kernel)
+    (convolution/implementation_forward.h:84-101, util/helper.h:11-24).  Each output Gaussian is
+    (w_d * w_k, b_d + b_k, S_d + S_k): weights are integrals, so no normalisation factor appears."""
+    B, Cin, Nd, G = data.shape
+    Cout, Cin2, Nk, G2 = kernels.shape
+    if Cin != Cin2 or G != G2:
+        raise RuntimeError("number of input feature maps / dimensions of data and kernel must agree")
+    out = np.empty((B, Cout, Nk, Cin, Nd, G), dtype=data.dtype)
+    d = data[:, None, None, :, :, :]                                   # [B, 1, 1, Cin, Nd, G]
+    k = np.transpose(kernels, (0, 2, 1, 3))[None, :, :, :, None, :]    # [1, Cout, Nk, Cin, 1, G]
+    out[..., 0] = d[..., 0] * k[..., 0]
+    out[..., 1:] = d[..., 1:] + k[..., 1:]
+    return out.reshape(B, Cout, Nk * Cin * Nd, G)
+
+
+def convolution_backward(grad_out: np.ndarray, data: np.ndarray, kernels: np.ndarray):
+    """-> (grad_data like data, grad_kernels like kernels), convolution/implementation_backward.h:107-121"""
+    B, Cin, Nd, G = data.shape
+    Cout, _, Nk, _ = kernels.shape
+    g = grad_out.reshape(B, Cout, Nk, Cin, Nd, G)
+    k = np.transpose(kernels, (0, 2, 1, 3))[None, :, :, :, None, :]
+    d = data[:, None, None, :, :, :]
+    gd = np.empty((B, Cin, Nd, G), dtype=data.dtype)
+    gd[..., 0] = (g[..., 0] * k[..., 0]).sum(axis=(1, 2))
+    gd[..., 1:] = g[..., 1:].sum(axis=(1, 2))
+    gk = np.empty((Cout, Nk, Cin, G), dtype=data.dtype)
+    gk[..., 0] = (g[..., 0] * d[..., 0]).sum(axis=(0, 4))
+    gk[..., 1:] = g[..., 1:].sum(axis=(0, 4))
+    return gd, np.transpose(gk, (0, 2, 1, 3)).copy()
+
+
+# ---- consumers of evaluate(): ReLU transfer fitting and batch normalisation ---------------------------------
+
+def pack(weights: np.ndarray, positions: np.ndarray, covariances: np.ndarray) -> np.ndarray:
+    return np.concatenate((weights[..., None], positions, covariances.reshape(*positions.shape[:-1], -1)), axis=-1)
+
+
+def fixed_point_iteration_to_relu(target_mixture, target_constant, fitting_mixture, n_iter: int = 1):
+    """src/gmc/fitting.py:287-312: weights of `fitting_mixture` such that it approximates relu(target + constant)
+    at its own centres.  Mixtures hold covariances.  -> (mixture, relu(constant))"""
+    w, pos, cov = split(fitting_mixture)
+    ret_const = np.where(target_constant > 0, target_constant, 0.0)
+    b = evaluate(target_mixture, pos) + target_constant[..., None]
+    b = np.where(b > 0, b, 0.0) - ret_const[..., None]
+    x = np.abs(w) + 0.1
+    for _ in range(n_iter):
+        x = np.abs(x)
+        x = x * (b + 0.05) / (evaluate(pack(x, pos, cov), pos) + 0.05)
+    return pack(x, pos, cov), ret_const
+
+
+def batch_norm_forward(mixture, constant, sampling_positions, learnable_scaling=None):
+    """src/gmc/modules.py:374-425 in its per-sample mode (batch_norm == False): the mixture is sampled at
+    `sampling_positions` [B, L, S, D], every channel is scaled by 1 / max(std, 0.001) (unbiased std over the
+    samples) and its mean is taken off the constant.  -> (mixture, constant)"""
+    w, pos, cov = split(mixture)
+    values = evaluate(mixture, sampling_positions) + constant[..., None]
+    sd = values.std(axis=2, ddof=1)
+    mean = values.mean(axis=2)
+    scaling = 1.0 / np.maximum(sd, 0.001)
+    if learnable_scaling is not None:
+        scaling = scaling * learnable_scaling
+    return pack(w * scaling[..., None], pos, cov), constant - mean

@@ -1,0 +1,136 @@
+"""Parity of the closed-form convolution (HIP kernels behind gmc_convolution_fwd / gmc_convolution_bwd) and of the
+evaluate() consumers (ReLU fixed-point fitting, BatchNorm) against the CPU oracle.
+Tolerances: the convolution forward is one rounding per scalar and must be bit-exact; sums (convolution backward)
+and everything built on evaluate(): relative L2 <= 1e-5 (float32) / 1e-12 (float64)."""
+import numpy as np
+import pytest
+import torch
+
+import gm_oracle as o
+from conftest import rel_l2
+from gmc import fitting, modules
+from gmc import mixture as gm
+from gmc.cpp.extensions.convolution import binding as cpp_convolution
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL = {torch.float32: 1e-5, torch.float64: 1e-12}
+
+
+def _cov_mixture(rng, B, L, M, D, cov=0.5):
+    w = rng.uniform(-1, 1, (B, L, M))
+    p = rng.uniform(-1, 1, (B, L, M, D))
+    a = rng.normal(size=(B, L, M, D, D))
+    c = (a @ np.swapaxes(a, -1, -2) + 0.3 * np.eye(D)) * cov
+    return o.pack(w, p, c)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("dims", [(3, 5, 7, 2, 4, 2), (2, 3, 1, 4, 1, 3), (1, 1, 300, 1, 5, 3), (5, 8, 33, 16, 5, 2),
+                                  (70, 2, 9, 3, 2, 3)])
+def test_convolution_forward_backward(dims, dtype):
+    B, Cin, Nd, Cout, Nk, D = dims
+    rng = np.random.default_rng(sum(dims))
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    d = _cov_mixture(rng, B, Cin, Nd, D).astype(npdt)
+    k = _cov_mixture(rng, Cout, Cin, Nk, D).astype(npdt)
+    dt = torch.tensor(d, device=DEV, requires_grad=True)
+    kt = torch.tensor(k, device=DEV, requires_grad=True)
+    out = cpp_convolution.apply(dt, kt)
+    ref = o.convolution_forward(d, k)
+    assert out.shape == ref.shape
+    assert np.array_equal(out.detach().cpu().numpy(), ref)          # bit-exact
+    g = rng.normal(size=ref.shape).astype(npdt)
+    out.backward(torch.tensor(g, device=DEV))
+    gd, gk = o.convolution_backward(g.astype(np.float64), d.astype(np.float64), k.astype(np.float64))
+    assert rel_l2(dt.grad.cpu().numpy(), gd) <= TOL[dtype]
+    assert rel_l2(kt.grad.cpu().numpy(), gk) <= TOL[dtype]
+    # one-sided requests and the raw binding (zeros for a gradient that is not asked for)
+    dt2 = torch.tensor(d, device=DEV, requires_grad=True)
+    cpp_convolution.apply(dt2, torch.tensor(k, device=DEV)).backward(torch.tensor(g, device=DEV))
+    assert rel_l2(dt2.grad.cpu().numpy(), gd) <= TOL[dtype]
+    raw_d, raw_k = cpp_convolution.cpp_binding.backward(torch.tensor(g, device=DEV), dt.detach(), kt.detach())
+    assert rel_l2(raw_k.cpu().numpy(), gk) <= TOL[dtype] and rel_l2(raw_d.cpu().numpy(), gd) <= TOL[dtype]
+
+
+def test_convolution_gradcheck_like_the_reference():
+    """src/gmc/test_mixture.py:138-152"""
+    for D in (2, 3):
+        a = gm.generate_random_mixtures(3, 5, 7, n_dims=D, pos_radius=1, cov_radius=0.5).to(torch.double).to(DEV)
+        b = gm.generate_random_mixtures(2, 5, 4, n_dims=D, pos_radius=1, cov_radius=0.5).to(torch.double).to(DEV)
+        a.requires_grad = True
+        b.requires_grad = True
+        assert torch.autograd.gradcheck(cpp_convolution.apply, (a, b))
+
+
+def test_convolution_input_checks():
+    a = gm.generate_random_mixtures(2, 3, 4, n_dims=2).to(DEV)
+    with pytest.raises(RuntimeError, match="input feature maps"):
+        cpp_convolution.apply(a, gm.generate_random_mixtures(2, 4, 4, n_dims=2).to(DEV))
+    with pytest.raises(RuntimeError, match="dimensions of data and kernel"):
+        cpp_convolution.apply(a, gm.generate_random_mixtures(2, 3, 4, n_dims=3).to(DEV))
+    with pytest.raises(RuntimeError, match="dtypes"):
+        cpp_convolution.apply(a, gm.generate_random_mixtures(2, 3, 4, n_dims=2).double().to(DEV))
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        cpp_convolution.apply(a.cpu(), a.cpu())
+
+
+def test_convolved_mixture_evaluates_like_the_oracle():
+    """convolution -> evaluate, the order in which the network uses the two (src/gmc/modules.py:163)"""
+    rng = np.random.default_rng(3)
+    d = _cov_mixture(rng, 2, 3, 6, 2, cov=0.2).astype(np.float32)
+    k = _cov_mixture(rng, 4, 3, 5, 2, cov=0.2).astype(np.float32)
+    xes = rng.uniform(-3, 3, (1, 1, 500, 2)).astype(np.float32)
+    out = gm.evaluate(modules.convolve(torch.tensor(d, device=DEV), torch.tensor(k, device=DEV)), torch.tensor(xes, device=DEV))
+    ref = o.evaluate(o.convolution_forward(d, k).astype(np.float64), xes.astype(np.float64))
+    assert rel_l2(out.cpu().numpy(), ref) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_relu_fixed_point_iteration(D, dtype):
+    rng = np.random.default_rng(20 + D)
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    target = _cov_mixture(rng, 3, 4, 40, D, cov=0.1).astype(npdt)
+    const = rng.normal(size=(3, 4)).astype(npdt) * 0.3
+    fit = _cov_mixture(rng, 3, 4, 24, D, cov=0.1).astype(npdt)
+    for n_iter in (1, 3):
+        got, got_c = fitting.fixed_point_iteration_to_relu(torch.tensor(target, device=DEV), torch.tensor(const, device=DEV),
+                                                           torch.tensor(fit, device=DEV), n_iter)
+        ref, ref_c = o.fixed_point_iteration_to_relu(target.astype(np.float64), const.astype(np.float64),
+                                                     fit.astype(np.float64), n_iter)
+        assert rel_l2(got.cpu().numpy(), ref) <= 10 * TOL[dtype]      # n_iter chained evaluations and divisions
+        assert np.array_equal(got_c.cpu().numpy(), np.maximum(const, 0))
+    relu0 = fitting.initial_approx_to_relu(torch.tensor(target, device=DEV), torch.tensor(const, device=DEV)).cpu().numpy()
+    w = target[..., 0]
+    assert np.array_equal(relu0[..., 0], np.where(w + const[..., None] > 0, w, -np.maximum(const, 0)[..., None]))
+
+
+@pytest.mark.parametrize("batch_norm", [False, True])
+def test_batch_norm(batch_norm):
+    rng = np.random.default_rng(31)
+    m = _cov_mixture(rng, 4, 3, 30, 2, cov=0.1).astype(np.float32)
+    const = rng.normal(size=(4, 3)).astype(np.float32)
+    layer = modules.BatchNorm(3, batch_norm=batch_norm, learn_scaling=True).to(DEV)
+    mt = torch.tensor(m, device=DEV, requires_grad=True)
+    xes = layer.sampling_positions(mt)
+    assert xes.shape == (4, 3, 2500 if batch_norm else 1000, 2)
+    scaled, new_const = layer((mt, torch.tensor(const, device=DEV)), sampling_positions=xes)
+    xn = xes.cpu().numpy().astype(np.float64)
+    if not batch_norm:
+        ref, ref_c = o.batch_norm_forward(m.astype(np.float64), const.astype(np.float64), xn)
+    else:
+        values = o.evaluate(m.astype(np.float64), xn) + const.astype(np.float64)[..., None]
+        vt = np.transpose(values, (1, 0, 2)).reshape(3, -1)
+        alpha = min(4 / 1000, 0.1)
+        sd = (1 - alpha) * 1.0 + alpha * vt.std(axis=1, ddof=1)
+        mean = (1 - alpha) * 1.0 + alpha * vt.mean(axis=1)
+        ref = m.astype(np.float64).copy()
+        ref[..., 0] /= np.maximum(sd, 0.001)[None, :, None]
+        ref_c = const - mean[None, :]
+    assert rel_l2(scaled.detach().cpu().numpy(), ref) <= 1e-5
+    assert rel_l2(new_const.cpu().numpy(), ref_c) <= 1e-5
+    # the gradient reaches the weights through the scaling only
+    scaled[..., 0].sum().backward()
+    assert torch.all(mt.grad[..., 1:] == 0) and torch.all(mt.grad[..., 0] != 0)

@@ -415,3 +415,102 @@ def test_workloads_are_seeded_and_valid():
         assert (torch.linalg.eigvalsh(c) > 0).all()
     wl, mix, xes, g = synthetic.make_workload("C1")
     assert xes[0, 0, 29].tolist() == [1.0, 1.0] and g.eq(1).all()
+
+
+# ---- convolution and the consumers of evaluate() ---------------------------------------------------------------
+
+def _rand_cov_mixture(rng, B, L, M, D, pos=1.0, cov=0.5):
+    w = rng.uniform(-1, 1, (B, L, M))
+    p = rng.uniform(-pos, pos, (B, L, M, D))
+    a = rng.normal(size=(B, L, M, D, D))
+    c = (a @ np.swapaxes(a, -1, -2) + 0.3 * np.eye(D)) * cov
+    return o.pack(w, p, c)
+
+
+def test_convolution_equals_numeric_convolution_of_the_sampled_operands():
+    """protocol of src/gmc/test_mixture.py:108-136: the closed form against scipy.signal.fftconvolve on a grid"""
+    import scipy.signal
+    rng = np.random.default_rng(5)
+    gm1 = _rand_cov_mixture(rng, 2, 1, 3, 2, cov=0.15)
+    gm2 = _rand_cov_mixture(rng, 1, 1, 4, 2, cov=0.15)
+    conv = o.convolution_forward(gm1, gm2)
+    assert conv.shape == (2, 1, 12, 7)
+    per_unit = 25
+    axis = np.arange(-6, 6, 1 / per_unit)
+    xv, yv = np.meshgrid(axis, axis, indexing="ij")
+    xes = np.stack((xv.ravel(), yv.ravel()), axis=1).reshape(1, 1, -1, 2)
+    size = axis.size
+    s1 = o.evaluate(gm1, xes).reshape(2, size, size)
+    s2 = o.evaluate(gm2, xes).reshape(size, size)
+    sc = o.evaluate(conv, xes).reshape(2, size, size)
+    for i in range(2):
+        ref = scipy.signal.fftconvolve(s1[i], s2, "same") / (per_unit * per_unit)
+        assert np.max((ref[1:, 1:] - sc[i][:-1, :-1]) ** 2) < 1e-7
+    # an independent statement of the index order (convolution/implementation_forward.h:84-101)
+    d = _rand_cov_mixture(rng, 2, 3, 4, 3)
+    k = _rand_cov_mixture(rng, 5, 3, 2, 3)
+    out = o.convolution_forward(d, k)
+    for (b, co, cd, ci, kk) in [(0, 0, 0, 0, 0), (1, 4, 3, 2, 1), (1, 2, 1, 0, 1), (0, 3, 2, 1, 0)]:
+        idx = cd + 4 * (ci + 3 * kk)
+        assert out[b, co, idx, 0] == d[b, ci, cd, 0] * k[co, ci, kk, 0]
+        assert np.array_equal(out[b, co, idx, 1:], d[b, ci, cd, 1:] + k[co, ci, kk, 1:])
+
+
+@pytest.mark.parametrize("D", [2, 3])
+def test_convolution_backward_matches_central_differences(D):
+    rng = np.random.default_rng(6 + D)
+    d = _rand_cov_mixture(rng, 2, 3, 4, D)
+    k = _rand_cov_mixture(rng, 2, 3, 3, D)
+    g = rng.normal(size=o.convolution_forward(d, k).shape)
+    gd, gk = o.convolution_backward(g, d, k)
+    eps = 1e-6
+    for arr, grad, which in ((d, gd, 0), (k, gk, 1)):
+        for _ in range(12):
+            i = tuple(rng.integers(0, s) for s in arr.shape)
+            hi, lo = arr.copy(), arr.copy()
+            hi[i] += eps
+            lo[i] -= eps
+            f = (lambda a: o.convolution_forward(a, k)) if which == 0 else (lambda a: o.convolution_forward(d, a))
+            num = ((f(hi) - f(lo)) * g).sum() / (2 * eps)
+            assert abs(num - grad[i]) <= 1e-7 * max(1.0, abs(num))
+
+
+def test_relu_fixed_point_iteration_restatement():
+    rng = np.random.default_rng(9)
+    target = _rand_cov_mixture(rng, 2, 2, 6, 2)
+    target[..., 0] = np.abs(target[..., 0]) + 0.2          # positive target with constant 0: relu changes nothing
+    const = np.zeros((2, 2))
+    fitted, ret_const = o.fixed_point_iteration_to_relu(target, const, target, n_iter=0)
+    assert np.array_equal(ret_const, const)
+    assert np.allclose(fitted[..., 0], target[..., 0] + 0.1) and np.array_equal(fitted[..., 1:], target[..., 1:])
+    # one update by hand at a single centre
+    fitted1, _ = o.fixed_point_iteration_to_relu(target, const, target, n_iter=1)
+    w, pos, cov = o.split(target)
+    x0 = np.abs(w) + 0.1
+    goal = np.maximum(o.evaluate(target, pos), 0.0)
+    cur = o.evaluate(o.pack(x0, pos, cov), pos)
+    assert np.allclose(fitted1[..., 0], x0 * (goal + 0.05) / (cur + 0.05), rtol=1e-13)
+    # the exact weights are a fixed point of the update: start from them (minus the 0.1 of the start value)
+    start = target.copy()
+    start[..., 0] -= 0.1
+    again, _ = o.fixed_point_iteration_to_relu(target, const, start, n_iter=3)
+    assert np.allclose(again[..., 0], target[..., 0], rtol=1e-12)
+    # a negative constant below every value gives the zero function: the goal is 0 and the weights shrink
+    low = np.full((2, 2), -1e3)
+    shrunk, rc = o.fixed_point_iteration_to_relu(target, low, target, n_iter=1)
+    assert np.all(rc == 0) and np.all(shrunk[..., 0] < x0)
+
+
+def test_batch_norm_restatement_normalises_the_samples():
+    rng = np.random.default_rng(10)
+    m = _rand_cov_mixture(rng, 3, 2, 5, 3)
+    const = rng.normal(size=(3, 2))
+    xes = rng.uniform(-1.5, 1.5, (3, 2, 400, 3))
+    scaled, new_const = o.batch_norm_forward(m, const, xes)
+    before = o.evaluate(m, xes) + const[..., None]
+    after = o.evaluate(scaled, xes)
+    # scaling the weights scales the mixture's values (not the constant): unit spread of the mixture part
+    assert np.allclose(after.std(axis=2, ddof=1) * before.std(axis=2, ddof=1),
+                       (before - const[..., None]).std(axis=2, ddof=1), rtol=1e-12)
+    assert np.allclose(new_const, const - before.mean(axis=2), rtol=1e-13)
+    assert np.array_equal(scaled[..., 1:], m[..., 1:])
