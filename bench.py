@@ -145,13 +145,96 @@ def cpu_baseline_bvh(mode: str):
                       f"box test per pair, fwd {t_fwd:.2f} s + bwd {t_bwd:.2f} s"}
 
 
+def bench_convolution(args):
+    """Closed-form convolution on a layer-sized problem (2-D, float32, batch 100, 8 -> 16 channels, 128 data and 5
+    kernel components per channel: 8.2e6 output Gaussians, 229 MB).  A step is forward plus backward (both
+    gradients).  The path is streaming: the unit is output Gaussians per second and the roofline is HBM with the
+    compulsory bytes (forward: operands in, result out; backward: grad_out is read once per gradient)."""
+    import torch
+    from gmc import _native
+    from gmc import mixture as gm
+    B, Cin, Cout, Nd, Nk, D = 100, 8, 16, 128, 5, 2
+    G = 1 + D + D * D
+    gen = torch.Generator().manual_seed(20246)
+    data = gm.generate_random_mixtures(B, Cin, Nd, n_dims=D, pos_radius=1, cov_radius=0.5)
+    kernels = gm.generate_random_mixtures(Cout, Cin, Nk, n_dims=D, pos_radius=1, cov_radius=0.5)
+    dev = torch.device("cuda:0")
+    data, kernels = data.to(dev), kernels.to(dev)
+    n_out = B * Cout * Nd * Cin * Nk
+    gout = torch.randn((B, Cout, Nd * Cin * Nk, G), generator=gen).to(dev)
+    torch.cuda.synchronize()
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        out = _native.convolution_fwd(data, kernels)
+        if ev:
+            ev[1].record()
+        g = _native.convolution_bwd(gout, data, kernels, True, True)
+        if ev:
+            ev[2].record()
+        return out, g
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(events[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_step = wall * 1e3 / args.steps
+    fwd_ms, bwd_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(2))
+    small = (data.numel() + kernels.numel()) * 4
+    bytes_fwd = n_out * G * 4 + small
+    bytes_bwd = 2 * n_out * G * 4 + 3 * small
+    line = {
+        "metric": "closed-form mixture convolution, output Gaussians per second (forward + backward step)",
+        "value": n_out / (ms_step * 1e-3), "unit": "output Gaussians/s (forward + backward step)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"conv: D={D} f32 data [{B},{Cin},{Nd}] * kernels [{Cout},{Cin},{Nk}] -> "
+                               f"[{B},{Cout},{Nd * Cin * Nk}], {n_out:.4g} output Gaussians per step"},
+        "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "roofline": {"kernel": "conv_bwd_data_kernel + conv_bwd_kernels_kernel (one event pair)", "bound": "hbm",
+                     "achieved": bytes_bwd / (bwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
+                     "frac": bytes_bwd / (bwd_ms * 1e-3) / 8e12, "traffic": None, "launch_ms": bwd_ms,
+                     "algorithmic_bytes": bytes_bwd},
+        "roofline_fwd": {"kernel": "conv_fwd_kernel", "bound": "hbm", "achieved": bytes_fwd / (fwd_ms * 1e-3) / 1e9,
+                         "peak": 8000.0, "unit": "GB/s", "frac": bytes_fwd / (fwd_ms * 1e-3) / 8e12,
+                         "launch_ms": fwd_ms, "algorithmic_bytes": bytes_fwd},
+    }
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import gm_oracle
+        d, k, g = data.cpu().numpy(), kernels.cpu().numpy(), gout.cpu().numpy()
+        t0 = time.perf_counter()
+        gm_oracle.convolution_forward(d, k)
+        t_fwd = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        gm_oracle.convolution_backward(g, d, k)
+        t_bwd = time.perf_counter() - t0
+        line["cpu_baseline"] = {"value": n_out / (t_fwd + t_bwd), "unit": "output Gaussians/s (fwd+bwd)", "cores": 1,
+                                "kind": "port", "sample": f"the whole step once in numpy float32 (the oracle's "
+                                f"restatement), fwd {t_fwd:.2f} s + bwd {t_bwd:.2f} s"}
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5"],
-                    help="C1..C4: dense all-pairs path; C5: LBVH-culled path (build + forward + backward per step)")
+    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5", "conv"],
+                    help="C1..C4: dense all-pairs path; C5: LBVH-culled path (build + forward + backward per step); "
+                         "conv: closed-form convolution (forward + backward per step)")
     ap.add_argument("--aabb-mode", default="reference", choices=["reference", "tight"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -168,6 +251,8 @@ def main():
 
     if args.workload == "C5":
         return bench_bvh(args)
+    if args.workload == "conv":
+        return bench_convolution(args)
     wl, mix, xes, gout = synthetic.make_workload(args.workload)
     dev = torch.device("cuda:0")
     mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)

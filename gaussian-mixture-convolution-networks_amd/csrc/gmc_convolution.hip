@@ -5,7 +5,7 @@
 // (weights are integrals, so the product needs no normalisation; index order of util/helper.h:11-24).
 // The work is pure streaming (HBM-bound: the output is Nk Cout / 1 times larger than the data), so the kernels are
 // laid out for coalescing and for single passes over the big tensor:
-//   forward   one lane per output scalar, stores fully coalesced, operands from cache;
+//   forward   one lane per scalar of the data: one load, then Cout Nk coalesced stores;
 //   backward  grad_data: one lane per scalar of grad_data gathers its Cout Nk terms, every read of grad_out is
 //             coalesced and no atomics are needed (the reference adds every term atomically);
 //             grad_kernels: one workgroup per (co, ci, k) and slice of the batch sums B Nd terms per scalar with
@@ -16,48 +16,72 @@ namespace gmc {
 
 struct ConvDims { int B, Cin, Cout, Nd, Nk; };
 
+// One lane per scalar of data[b] (Cin * Nd * G of them): it loads its operand once and stores the Nk outputs of
+// each output channel co in [co_begin, co_end) that are built from it.  Every store instruction of a wavefront
+// covers contiguous memory (the run of Nd * G scalars of one (b, co, ci, k)), and the per-lane index arithmetic
+// is paid once for Nk * (co_end - co_begin) stores.  grid.x = B * chunks, grid.y = splits of the output channels.
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void conv_fwd_kernel(const T* __restrict__ data, const T* __restrict__ kernels,
-                                                          T* __restrict__ out, ConvDims n, size_t total) {
+                                                          T* __restrict__ out, ConvDims n, unsigned chunks,
+                                                          unsigned co_per_split) {
     constexpr int G = 1 + D + D * D;
-    const size_t e = size_t(blockIdx.x) * kBlock + threadIdx.x;
-    if (e >= total) return;
-    const size_t gauss = e / G;
-    const int el = int(e - gauss * G);
-    const size_t n_out = size_t(n.Nd) * n.Cin * n.Nk;
-    const size_t bc = gauss / n_out;                  // b * Cout + co
-    const size_t idx = gauss - bc * n_out;
-    const int b = int(bc / n.Cout), co = int(bc - size_t(b) * n.Cout);
-    const int cd = int(idx % n.Nd);
-    const size_t rest = idx / n.Nd;
-    const int ci = int(rest % n.Cin), k = int(rest / n.Cin);
-    const T dv = data[((size_t(b) * n.Cin + ci) * n.Nd + cd) * G + el];
-    const T kv = kernels[((size_t(co) * n.Cin + ci) * n.Nk + k) * G + el];
-    out[e] = el == 0 ? dv * kv : dv + kv;
-}
-
-template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void conv_bwd_data_kernel(const T* __restrict__ grad_out, const T* __restrict__ kernels,
-                                                               T* __restrict__ grad_data, ConvDims n, size_t total) {
-    constexpr int G = 1 + D + D * D;
-    const size_t e = size_t(blockIdx.x) * kBlock + threadIdx.x;   // scalar of grad_data [B][Cin][Nd][G]
-    if (e >= total) return;
-    const size_t gauss = e / G;
-    const int el = int(e - gauss * G);
-    const int cd = int(gauss % n.Nd);
-    const size_t rest = gauss / n.Nd;
-    const int ci = int(rest % n.Cin), b = int(rest / n.Cin);
-    const size_t n_out = size_t(n.Nd) * n.Cin * n.Nk;
-    T acc = T(0);
-    for (int co = 0; co < n.Cout; ++co) {
-        const T* __restrict__ g_bc = grad_out + (size_t(b) * n.Cout + co) * n_out * G;
-        const T* __restrict__ k_cc = kernels + (size_t(co) * n.Cin + ci) * n.Nk * G;
+    const unsigned run = unsigned(n.Nd) * G;
+    const unsigned per_b = run * unsigned(n.Cin);
+    const unsigned b = blockIdx.x / chunks;
+    const unsigned e = (blockIdx.x - b * chunks) * kBlock + threadIdx.x;
+    if (e >= per_b) return;
+    const unsigned ci = e / run, t = e - ci * run;
+    const unsigned el = t % G;
+    const T dv = data[size_t(b) * per_b + e];
+    const unsigned co_begin = blockIdx.y * co_per_split;
+    const unsigned co_end = co_begin + co_per_split < unsigned(n.Cout) ? co_begin + co_per_split : unsigned(n.Cout);
+    const size_t slab = size_t(per_b) * n.Nk;                       // scalars of one (b, co)
+    for (unsigned co = co_begin; co < co_end; ++co) {
+        const T* __restrict__ kv = kernels + (size_t(co) * n.Cin + ci) * n.Nk * G + el;
+        T* __restrict__ o = out + (size_t(b) * n.Cout + co) * slab + size_t(ci) * run + t;
         for (int k = 0; k < n.Nk; ++k) {
-            const T g = g_bc[(size_t(cd) + size_t(n.Nd) * (ci + size_t(n.Cin) * k)) * G + el];
-            acc += el == 0 ? g * k_cc[size_t(k) * G] : g;
+            const T w = kv[size_t(k) * G];
+            o[size_t(k) * per_b] = el == 0 ? dv * w : dv + w;
         }
     }
-    grad_data[e] = acc;
+}
+
+// Mirror image of the forward kernel: one lane per scalar of grad_data[b] gathers its Cout Nk terms; every load
+// instruction of a wavefront reads contiguous memory.  grid.x = B * chunks.
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void conv_bwd_data_kernel(const T* __restrict__ grad_out, const T* __restrict__ kernels,
+                                                               T* __restrict__ grad_data, ConvDims n, unsigned chunks) {
+    constexpr int G = 1 + D + D * D;
+    const unsigned run = unsigned(n.Nd) * G;
+    const unsigned per_b = run * unsigned(n.Cin);
+    const unsigned b = blockIdx.x / chunks;
+    const unsigned e = (blockIdx.x - b * chunks) * kBlock + threadIdx.x;
+    if (e >= per_b) return;
+    const unsigned ci = e / run, t = e - ci * run;
+    const unsigned el = t % G;
+    const size_t slab = size_t(per_b) * n.Nk;
+    const T* __restrict__ g = grad_out + size_t(b) * n.Cout * slab + size_t(ci) * run + t;
+    const T* __restrict__ kv = kernels + size_t(ci) * n.Nk * G;
+    const size_t kv_stride = size_t(n.Cin) * n.Nk * G;
+    // eight loads in flight per lane: the terms are walked in their flattened (co, k) order
+    const int terms = n.Cout * n.Nk;
+    T acc0 = T(0), acc1 = T(0);
+    for (int i0 = 0; i0 < terms; i0 += 8) {
+        T gv[8], wv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u < terms ? i0 + u : terms - 1;
+            const int co = i / n.Nk, k = i - co * n.Nk;
+            gv[u] = g[size_t(co) * slab + size_t(k) * per_b];
+            wv[u] = el == 0 ? kv[size_t(co) * kv_stride + size_t(k) * G] : T(1);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const T term = i0 + u < terms ? gv[u] * wv[u] : T(0);
+            if (u & 1) acc1 += term; else acc0 += term;
+        }
+    }
+    grad_data[size_t(b) * per_b + e] = acc0 + acc1;
 }
 
 // grid: (Cout * Cin * Nk) x slices workgroups; workgroup (c, s) sums the batches b = s, s + slices, ...
@@ -99,7 +123,16 @@ static int conv_forward_t(const T* data, const T* kernels, T* out, const ConvDim
     constexpr int G = 1 + D + D * D;
     const size_t total = size_t(n.B) * n.Cout * n.Nd * n.Cin * n.Nk * G;
     if (total == 0) return GMC_OK;
-    conv_fwd_kernel<T, D><<<dim3(unsigned((total + kBlock - 1) / kBlock)), dim3(kBlock), 0, st>>>(data, kernels, out, n, total);
+    const size_t per_b = size_t(n.Nd) * G * n.Cin;                  // < 2^31 by the shape check
+    const unsigned chunks = unsigned((per_b + kBlock - 1) / kBlock);
+    if (size_t(n.B) * chunks > 0x7fffffffull) return GMC_E_SHAPE;
+    // split the output channels over grid.y until there are a few thousand workgroups
+    unsigned splits = 1;
+    while (size_t(n.B) * chunks * splits < 4096 && splits < unsigned(n.Cout)) splits *= 2;
+    if (splits > unsigned(n.Cout)) splits = unsigned(n.Cout);
+    const unsigned co_per_split = (unsigned(n.Cout) + splits - 1) / splits;
+    splits = (unsigned(n.Cout) + co_per_split - 1) / co_per_split;
+    conv_fwd_kernel<T, D><<<dim3(unsigned(n.B) * chunks, splits), dim3(kBlock), 0, st>>>(data, kernels, out, n, chunks, co_per_split);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
@@ -111,7 +144,10 @@ static int conv_backward_t(const T* grad_out, const T* data, const T* kernels, T
     const bool empty_sum = n.Cout == 0 || n.Nk == 0 || n.B == 0 || n.Nd == 0 || n.Cin == 0;
     if (need_data && n_data > 0) {
         if (empty_sum) zero_async(grad_data, n_data, st);
-        else conv_bwd_data_kernel<T, D><<<dim3(unsigned((n_data + kBlock - 1) / kBlock)), dim3(kBlock), 0, st>>>(grad_out, kernels, grad_data, n, n_data);
+        else {
+            const unsigned chunks = unsigned((size_t(n.Nd) * G * n.Cin + kBlock - 1) / kBlock);
+            conv_bwd_data_kernel<T, D><<<dim3(unsigned(n.B) * chunks), dim3(kBlock), 0, st>>>(grad_out, kernels, grad_data, n, chunks);
+        }
     }
     if (need_kernels && n_kern > 0) {
         if (empty_sum) {
@@ -138,6 +174,7 @@ static int check_conv_shape(const gmc_conv_shape* s) {
     if (s->B < 0 || s->Cin < 0 || s->Cout < 0 || s->Nd < 0 || s->Nk < 0) return GMC_E_SHAPE;
     // the cell index Cout * Cin * Nk and the per-(b, co) component index are 32-bit inside the kernels
     if (size_t(s->Cout) * s->Cin * s->Nk > 0x3fffffffull || size_t(s->Nd) * s->Cin * s->Nk > 0x7fffffffull / 13) return GMC_E_SHAPE;
+    if (size_t(s->B) * s->Cout * s->Cin * s->Nk > 0x7fffffffull) return GMC_E_SHAPE;
     return GMC_OK;
 }
 
