@@ -94,6 +94,26 @@ def test_tile_and_chunk_boundaries(dtype, D):
 
 
 @pytest.mark.parametrize("D", [2, 3])
+def test_matrix_core_forward_shapes(D):
+    """float32 shapes that take the wide matrix-core forward kernel (more than 128 components and either many
+    mixtures or many points): several 512-component tiles with a ragged last one, point counts that are no multiple
+    of the 16-point groups, almost empty point blocks, and components far from the origin in units of their width
+    (those are evaluated with an explicit x - b next to the matrix-core ones)."""
+    dtype = torch.float32
+    mix, xes, gout = _case(1, 1, 700, 8200, D, 900 + D, False)
+    _check(mix, xes, gout, dtype, tag=f"wide M700 N8200 D{D}")
+    far = mix.copy()
+    far[:, :, ::3, 1:1 + D] *= 9.0           # every third component: |u b| well above the shifted-form limit
+    xes_far = xes.copy()
+    xes_far[:, :, ::2] *= 9.0
+    _check(far, xes_far, gout, dtype, tag=f"wide far components D{D}")
+    mix, xes, gout = _case(40, 16, 130, 100, D, 910 + D, False)
+    _check(mix, xes, gout, dtype, tag=f"wide many mixtures few points D{D}")
+    mix, xes, gout = _case(2, 1, 1030, 8192 + 17, D, 920 + D, True)
+    _check(mix, xes, gout, dtype, tag=f"wide broadcast three tiles D{D}")
+
+
+@pytest.mark.parametrize("D", [2, 3])
 def test_reference_literal_collections(golden_dir, D):
     """the literal Gaussians / points of unittests/support.h:68-183 (weights 0, identity and skewed matrices)"""
     data = json.load(open(os.path.join(golden_dir, "support_collections.json")))
