@@ -19,8 +19,8 @@
 namespace gmc {
 
 // float32 forward pair kernel with y = u x - u b on the matrix cores (gmc_dense_mfma.hip)
-int dense_forward_f32(const float* mixture, const float* xes, float* out, const gmc_shape& s, bool covariance_form,
-                      hipStream_t stream);
+bool dense_forward_f32(const float* mixture, const float* xes, float* out, const gmc_shape& s, bool covariance_form,
+                       hipStream_t stream);
 
 constexpr int kTile = 256;   // Gaussians staged per LDS tile (one per lane)
 
@@ -389,7 +389,9 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
     const size_t BL = size_t(s.B) * s.L;
     if (BL == 0 || s.N == 0) return GMC_OK;
     if (s.M == 0) { zero_async(out, BL * s.N, stream); return GMC_OK; }
-    if constexpr (std::is_same<T, float>::value) return dense_forward_f32(mixture, xes, out, s, cov, stream);
+    if constexpr (std::is_same<T, float>::value) {
+        if (dense_forward_f32(mixture, xes, out, s, cov, stream)) return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+    }
     const int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
     const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
     const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
