@@ -28,7 +28,7 @@ def _cov_mixture(rng, B, L, M, D, cov=0.5):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("dims", [(3, 5, 7, 2, 4, 2), (2, 3, 1, 4, 1, 3), (1, 1, 300, 1, 5, 3), (5, 8, 33, 16, 5, 2),
-                                  (70, 2, 9, 3, 2, 3)])
+                                  (70, 2, 9, 3, 2, 3), (700, 1, 2, 100, 1, 2)])
 def test_convolution_forward_backward(dims, dtype):
     B, Cin, Nd, Cout, Nk, D = dims
     rng = np.random.default_rng(sum(dims))

@@ -149,6 +149,14 @@ def test_need_flags_and_zero_grads():
     assert gx_.shape == x.shape and not gx_.any().item() and rel_l2(gm_.cpu().numpy(), rgm) < 1e-12
 
 
+def test_more_than_65535_mixtures():
+    """the reference refuses batch x layers >= 65535 (parallel_implementation.cu:68); here the grid is flat"""
+    mix, xes, gout = _case(70000, 1, 3, 5, 2, 77, False)
+    _check(mix, xes, gout, torch.float32, tag="B70000")
+    mix, xes, gout = _case(300, 250, 2, 4, 3, 78, True)
+    _check(mix, xes, gout, torch.float64, tag="B300 L250 broadcast")
+
+
 def test_empty_inputs():
     for M, N in ((0, 5), (4, 0), (0, 0)):
         mix = torch.zeros(2, 3, M, 13, device=DEV, requires_grad=True)
