@@ -21,6 +21,9 @@ sys.path.insert(0, os.path.join(ROOT, "gaussian-mixture-convolution-networks_amd
 
 FLOP_FWD = {2: 12, 3: 20}
 FLOP_BWD = {2: 30, 3: 52}
+# forward flops per pair of the reference's literal arithmetic (determinant, square root and exp per pair,
+# util/gaussian.h:82-95); reported for transparency only, never as the headline
+FLOP_FWD_LITERAL = {2: 15, 3: 27}
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}     # MI355X vector peaks
 # HBM bytes per launch of the backward pair kernel, from rocprofv3 counter runs of this script (summary under
 # profiles/): FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0, factors from a 1 GiB copy kernel in the same runs.
@@ -102,6 +105,12 @@ def bench_bvh(args):
     wall = time.perf_counter() - t0
     ms_step = wall * 1e3 / args.steps
     build_ms, fwd_ms, bwd_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(3))
+    # pairs actually evaluated: points inside the cutoff box of a Gaussian (counted outside the timed region)
+    lo, up = _native.Bvh(mix, xes, 0.001, args.aabb_mode).boxes()
+    hits = 0
+    for n0 in range(0, wl.N, 2048):
+        x = xes[0, 0, n0:n0 + 2048].unsqueeze(1)                       # [n, 1, D]
+        hits += int(((x >= lo[0, 0].unsqueeze(0)) & (x <= up[0, 0].unsqueeze(0))).all(dim=-1).sum().item())
     s, M, N, D = 8, wl.M, wl.N, 3
     bytes_fwd = M * 13 * s + (2 * M - 1) * (2 * D * s + 8) + N * (D + 1) * s
     bytes_bwd = bytes_fwd + N * s + M * 13 * s + N * D * s
@@ -113,6 +122,8 @@ def bench_bvh(args):
         "config": {"workload": f"C5: D=3 f64 B=1 L=1 M={M} N={N}, LBVH-culled (aabb_mode={args.aabb_mode}, "
                                f"threshold 0.001), {wl.pairs:.4g} dense-equivalent pairs per step"},
         "build_ms": build_ms, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "evaluated_pairs": hits, "evaluated_pairs_per_s": hits / (ms_step * 1e-3),
+        "evaluated_fraction_of_dense": hits / wl.pairs,
         "roofline": {"kernel": "bvh_traverse_kernel (backward mode; event pair also holds its zero-fill and epilogue)",
                      "bound": "hbm", "achieved": bytes_bwd / (bwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
                      "frac": bytes_bwd / (bwd_ms * 1e-3) / 8e12, "traffic": None, "launch_ms": bwd_ms,
@@ -308,7 +319,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
         "config": {"workload": f"{wl.name}: D={D} {dt} B={wl.B} L={wl.L} M={wl.M} N={wl.N}, dense all-pairs, "
                                f"{wl.pairs:.4g} pairs per step, forward + backward (grad mixture and grad xes)"},
-        "fwd": {"ms": fwd_ms, "pairs_per_s": wl.pairs / (fwd_ms * 1e-3), "tflops": fwd_tf, "frac_of_peak": fwd_tf / peak},
+        "fwd": {"ms": fwd_ms, "pairs_per_s": wl.pairs / (fwd_ms * 1e-3), "tflops": fwd_tf, "frac_of_peak": fwd_tf / peak,
+                "tflops_by_reference_literal_count": FLOP_FWD_LITERAL[D] * wl.pairs / (fwd_ms * 1e-3) / 1e12},
         "fwd_bwd": {"ms": ms_step, "pairs_per_s": wl.pairs / (ms_step * 1e-3), "tflops": step_tf,
                     "frac_of_peak": step_tf / peak},
         "roofline": {"kernel": "eval_bwd_rc_kernel (backward pair kernel; its zero-fill and epilogue launches, <1% of "
