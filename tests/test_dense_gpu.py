@@ -111,6 +111,15 @@ def test_matrix_core_forward_shapes(D):
     _check(mix, xes, gout, dtype, tag=f"wide many mixtures few points D{D}")
     mix, xes, gout = _case(2, 1, 1030, 8192 + 17, D, 920 + D, True)
     _check(mix, xes, gout, dtype, tag=f"wide broadcast three tiles D{D}")
+    # covariance form on the same kernel: gm.evaluate inverts inside the staging
+    mix, xes, gout = _case(1, 2, 300, 8200, D, 930 + D, False)
+    B, L, M = mix.shape[:3]
+    cov = np.linalg.inv(mix[..., 1 + D:].reshape(B, L, M, D, D))
+    cov = 0.5 * (cov + np.swapaxes(cov, -1, -2))
+    mc = np.concatenate((mix[..., :1 + D], cov.reshape(B, L, M, D * D)), axis=-1).astype(np.float32)
+    out = gm.evaluate(torch.tensor(mc, device=DEV), torch.tensor(xes.astype(np.float32), device=DEV))
+    ref = o.evaluate(mc.astype(np.float64), xes.astype(np.float32).astype(np.float64))
+    assert rel_l2(out.cpu().numpy(), ref, FLOOR[dtype]) <= TOL[dtype]
 
 
 @pytest.mark.parametrize("D", [2, 3])
