@@ -122,6 +122,33 @@ def test_matrix_core_forward_shapes(D):
     assert rel_l2(out.cpu().numpy(), ref, FLOOR[dtype]) <= TOL[dtype]
 
 
+def test_matrix_core_forward_random_shapes():
+    """differential run of the wide float32 forward kernel over random shapes, position scales (mix of shifted- and
+    centred-form components) and widths, against the C restatement of the reference in float64"""
+    rng = np.random.default_rng(4242)
+    worst = 0.0
+    for case in range(24):
+        D = 2 + case % 2
+        if case % 3 == 0:
+            B, L, M, N = int(rng.integers(20, 40)), int(rng.integers(16, 30)), int(rng.integers(129, 400)), int(rng.integers(1, 2100))
+        else:
+            B, L, M, N = 1, int(rng.integers(1, 3)), int(rng.integers(129, 1300)), int(rng.integers(8192, 9300))
+        g = torch.Generator().manual_seed(5000 + case)
+        pos_radius = float(rng.choice([0.5, 2.0, 10.0, 40.0]))
+        cov_radius = float(rng.choice([0.05, 0.5, 3.0]))
+        mix = synthetic.random_inversed_mixture(B, L, M, D, g, pos_radius=pos_radius, cov_radius=cov_radius, dtype=torch.float64)
+        broadcast = case % 4 == 1
+        shape = (1, 1, N, D) if broadcast else (B, L, N, D)
+        xes = (torch.rand(shape, generator=g, dtype=torch.float64) * 2 - 1) * pos_radius * 1.2
+        m32, x32 = mix.float(), xes.float()
+        out = gm.evaluate_inversed(m32.to(DEV), x32.to(DEV)).cpu().numpy()
+        ref = cpu_ref.forward(m32.numpy().astype(np.float64), x32.numpy().astype(np.float64), n_threads=16)
+        err = rel_l2(out, ref, FLOOR[torch.float32])
+        worst = max(worst, err)
+        assert err <= TOL[torch.float32], f"case {case}: B{B} L{L} M{M} N{N} D{D} pos {pos_radius} cov {cov_radius}: {err}"
+    print("worst relative L2", worst, flush=True)
+
+
 @pytest.mark.parametrize("D", [2, 3])
 def test_reference_literal_collections(golden_dir, D):
     """the literal Gaussians / points of unittests/support.h:68-183 (weights 0, identity and skewed matrices)"""
