@@ -134,3 +134,38 @@ def test_batch_norm(batch_norm):
     # the gradient reaches the weights through the scaling only
     scaled[..., 0].sum().backward()
     assert torch.all(mt.grad[..., 1:] == 0) and torch.all(mt.grad[..., 0] != 0)
+
+
+def test_layer_pipeline_against_the_oracle_composition():
+    """convolution -> batch norm (per sample) -> ReLU fixed-point fitting -> evaluation on a grid, the order in which
+    a network layer of the reference chains these pieces (src/gmc/modules.py:163, :374-425, src/gmc/fitting.py:287-312),
+    against the same chain of oracle functions in float64; gradients flow back to the data and the kernels."""
+    rng = np.random.default_rng(77)
+    D = 2
+    data = _cov_mixture(rng, 3, 4, 12, D, cov=0.15).astype(np.float32)
+    kernels = _cov_mixture(rng, 5, 4, 3, D, cov=0.15).astype(np.float32)
+    samples = rng.uniform(-2.5, 2.5, (3, 5, 600, D)).astype(np.float32)
+    grid = rng.uniform(-3, 3, (1, 1, 900, D)).astype(np.float32)
+
+    dt = torch.tensor(data, device=DEV, requires_grad=True)
+    kt = torch.tensor(kernels, device=DEV, requires_grad=True)
+    conv = modules.convolve(dt, kt)
+    norm = modules.BatchNorm(5, batch_norm=False, learn_scaling=False).to(DEV)
+    normed, const = norm((conv, None), sampling_positions=torch.tensor(samples, device=DEV))
+    fitted, fitted_const = fitting.fixed_point_iteration_to_relu(normed.detach(), const.detach(), normed.detach()[:, :, ::4].contiguous(), 2)
+    values = gm.evaluate(fitted, torch.tensor(grid, device=DEV)) + fitted_const.unsqueeze(-1)
+    pre = gm.evaluate(normed, torch.tensor(grid, device=DEV))          # differentiable branch
+    pre.sum().backward()
+
+    d64, k64 = data.astype(np.float64), kernels.astype(np.float64)
+    oconv = o.convolution_forward(d64, k64)
+    onormed, oconst = o.batch_norm_forward(oconv, np.zeros((3, 5)), samples.astype(np.float64))
+    ofitted, ofc = o.fixed_point_iteration_to_relu(onormed, oconst, onormed[:, :, ::4], 2)
+    ovalues = o.evaluate(ofitted, grid.astype(np.float64)) + ofc[..., None]
+    assert rel_l2(conv.detach().cpu().numpy(), oconv) <= 1e-6
+    assert rel_l2(normed.detach().cpu().numpy(), onormed) <= 1e-5
+    assert rel_l2(const.cpu().numpy(), oconst) <= 1e-5
+    assert rel_l2(values.cpu().numpy(), ovalues) <= 5e-5          # two chained multiplicative updates
+    assert rel_l2(pre.detach().cpu().numpy(), o.evaluate(onormed, grid.astype(np.float64))) <= 1e-5
+    assert torch.isfinite(dt.grad).all() and torch.isfinite(kt.grad).all()
+    assert dt.grad.abs().sum() > 0 and kt.grad.abs().sum() > 0
