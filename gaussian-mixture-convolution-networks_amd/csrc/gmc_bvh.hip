@@ -13,9 +13,10 @@
 //   -> bottom-up union of boxes with integer atomic min/max on order-preserving encodings.
 // Query points are Morton-sorted the same way so that a wavefront owns 64 neighbouring points.
 //
-// Traversal: one wavefront per 64 sorted points with ONE node stack per wavefront (LDS); lanes work on tree nodes
-// while the tree is descended and on points while the gathered leaves are evaluated (see bvh_traverse_kernel).
-// Backward reduces the per-Gaussian sums over the wavefront and issues one atomic per scalar, leaf and wavefront.
+// Traversal: 64 sorted points form a group with ONE node stack (LDS); lanes work on tree nodes while the tree is
+// descended and on points while the gathered leaves are evaluated; a workgroup serves up to four groups, whose
+// descents overlap (see bvh_traverse_kernel).  Backward collects the per-Gaussian sums of a batch of leaves in LDS
+// and issues one global atomic per non-zero scalar, leaf and wavefront.
 #include "gmc_common.h"
 
 namespace gmc {
@@ -51,8 +52,8 @@ constexpr int kSortItems = 2;                       // items per lane and radix 
 constexpr int kSortChunk = kBlock * kSortItems;     // 512: small chunks, many workgroups (the passes are latency-bound)
 constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the first bounds pass
 
-template <int D> struct LeafRec { static constexpr int kStride = (D == 2) ? 8 : 12; };
-// D=3: b0 b1 b2 c00 c01 c02 c11 c12 c22 amp comp -   D=2: b0 b1 c00 c01 c11 amp comp -
+template <int D> struct LeafRec { static constexpr int kStride = (D == 2) ? 12 : 18; };
+// own box (lower[D], upper[D]), then  D=3: b0 b1 b2 c00 c01 c02 c11 c12 c22 amp comp -   D=2: b0 b1 c00 c01 c11 amp comp -
 
 static size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
 
@@ -461,6 +462,8 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
     if (M == 1) parent[node] = -1;                  // a single leaf is its own root
     const T* g = mixture + gi * G;
     T* r = leaf_rec + i * RS;
+    for (int d = 0; d < D; ++d) { r[d] = box_lo[gi * D + d]; r[D + d] = box_hi[gi * D + d]; }
+    r += 2 * D;
     const T* c = g + 1 + D;
     for (int d = 0; d < D; ++d) r[d] = g[1 + d];
     if constexpr (D == 2) {
@@ -619,12 +622,14 @@ __device__ __forceinline__ T leaf_terms(const T* __restrict__ r, const T (&x)[D]
 
 template <int D> struct BvhSums { static constexpr int k = 1 + D + D * (D + 1) / 2; };
 
-constexpr int kStackCap = 512;          // soft capacity of the node stack (the array has 128 more)
+constexpr int kStackCap = 512;          // soft capacity of a node stack (the array has 128 more)
 constexpr int kLeafFlush = 512;         // candidate leaves are evaluated whenever this many have gathered
 constexpr int kLeafCap = kLeafFlush + 128;
-constexpr int kTravWaves = 8;           // wavefronts per workgroup of the traversal (one workgroup per 64 points)
+constexpr int kTravWaves = 8;           // wavefronts per workgroup of the traversal
 constexpr int kTravBlock = kTravWaves * kWave;
-constexpr int kStageBatch = 32;         // candidate leaves a wavefront stages in LDS at a time
+constexpr int kGroupsMax = 4;           // 64-point groups per workgroup (each descends the tree with its own wavefront)
+constexpr int kStageBatch = 20;         // candidate leaves a wavefront stages in LDS at a time
+constexpr int kTravSlots = 2 * 256;     // workgroups resident at once: two per compute unit
 
 template <typename T>
 __device__ __forceinline__ T wave_min(T v) {
@@ -646,211 +651,343 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Traversal of one tree for 64 Morton-neighbouring points by one workgroup of 8 wavefronts, in two alternating
-// phases.
-//   Phase 1 (wavefront 0, lanes = tree nodes): ONE stack of internal nodes in LDS; up to 64 of them are popped at
-//   a time, each lane fetches the two child boxes of its node and tests them against the bounding box of the 64
-//   points (a node that contains any of the points overlaps that box).  Overlapping internal children go back on
-//   the stack, overlapping leaves into a candidate list (ballot + prefix-popcount compaction).
-//   Phase 2 (all wavefronts, lanes = points): the candidates are dealt to the wavefronts; each stages 32 of its
-//   candidates (own box + evaluation record) in LDS with one memory round trip, then tests every staged leaf
-//   against each point with the leaf's OWN box (closed interval, lbvh/aabb.h:39-47) and evaluates it where it
-//   contains the point.  The per-point partial results of the wavefronts are added at the end.
-// Phase 1 only filters, phase 2 applies the per-point rule, so the result is the sum over the Gaussians whose own
-// box contains the point.  Dependent memory round trips: about one per tree level plus one per 64 visited nodes,
-// instead of one per visited node; the candidate lists vary a lot between point groups (dense regions), which
-// is why one group gets a whole workgroup.
-// MODE 0: forward.  MODE 1: backward (grad_out given; accumulates per-Gaussian sums and dL/dx).
+// Traversal of one tree by a workgroup of 8 wavefronts for up to kGroupsMax groups of 64 Morton-neighbouring
+// points, in two alternating phases.
+//   Phase 1 (wavefront i descends for group i, lanes = tree nodes): one stack of internal nodes per group in LDS;
+//   up to 64 of them are popped at a time, each lane fetches the two child boxes of its node and tests them against
+//   the bounding box of the group's points (a node that contains any of the points overlaps that box).
+//   Overlapping internal children go back on the stack, overlapping leaves into the group's candidate list (ballot
+//   + prefix-popcount compaction).  The descents of the groups are independent chains of memory round trips (about
+//   one per tree level) and run side by side.
+//   Phase 2 (all wavefronts, group after group, lanes = points): the candidates of a group are dealt to the
+//   wavefronts; each stages kStageBatch of its candidates (own box + evaluation record, one contiguous leaf
+//   record) in LDS, the records of the next batch being fetched while the current one is worked on, tests every
+//   lane's point against all staged boxes (closed interval, lbvh/aabb.h:39-47; the lane keeps a bit mask of the
+//   leaves that contain its point) and then evaluates, lane by lane, only the leaves of its own mask: the loop
+//   runs as often as the busiest lane has hits, not once per leaf.  The per-point partial results of the
+//   wavefronts are added in wavefront order (deterministic).
+// Phase 1 only filters, phase 2 applies the per-point rule of lbvh/query.h:13-66, so the result is the sum over the
+// Gaussians whose own box contains the point.
+// MODE 0: forward.  MODE 1: backward (grad_out given): dL/dx stays in the lanes' registers.  The per-Gaussian sums
+// of a batch are collected in a per-wavefront LDS copy and flushed with one global atomic per non-zero scalar:
+// a leaf that contains many of the points is evaluated by all lanes at once and its sums are reduced over the
+// wavefront (DPP); the remaining hits go through the lane-by-lane loop and are added with LDS atomics (a few
+// cycles per instruction when the lanes of an instruction address different leaves, hence the lanes start at
+// different leaves of the batch).
 template <typename T, int D, int MODE, bool NEED_GM, bool NEED_GX>
-__global__ __launch_bounds__(kTravBlock) void bvh_traverse_kernel(
-        const T* __restrict__ xes, const int* __restrict__ p_order, const T* __restrict__ node_box,
-        const T* __restrict__ child_box, const int2* __restrict__ children, const T* __restrict__ leaf_rec,
-        T* __restrict__ out, const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes,
-        int L, int M, int N, int Bx, int Lx, int chunks, int xes_shared) {
-    constexpr int RS = LeafRec<D>::kStride;
+__global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4))) void bvh_traverse_kernel(
+        const T* __restrict__ xes, const int* __restrict__ p_order, const T* __restrict__ child_box,
+        const int2* __restrict__ children, const T* __restrict__ leaf_rec, T* __restrict__ out,
+        const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes, int L, int M, int N, int Bx,
+        int Lx, int chunks, int groups, int xes_shared) {
+    constexpr int LS = LeafRec<D>::kStride;
     constexpr int NR = BvhSums<D>::k;
-    constexpr int LS = 2 * D + RS;          // scalars per staged leaf: own box, evaluation record
-    constexpr int kWaves = kTravWaves;
-    __shared__ int stack[kStackCap + 128];
-    __shared__ int leaves[kLeafCap];
-    __shared__ int shared_state[2];         // [0] candidates gathered, [1] nodes left on the stack
-    __shared__ __attribute__((aligned(16))) T staged_mem[kWaves][kStageBatch * LS];
+    constexpr int kVals = MODE == 0 ? 1 : D;
+    constexpr int kAmp = 2 * D + D + D * (D + 1) / 2;       // position of the amplitude inside a leaf record
+    __shared__ int stack[kGroupsMax][kStackCap + 128];
+    __shared__ int leaves[kGroupsMax][kLeafCap];
+    __shared__ int state[kGroupsMax][2];                    // [0] candidates gathered, [1] nodes left on the stack
+    __shared__ int pids[kGroupsMax][kWave];                 // index of every point, -1 beyond the end
+    __shared__ T pts[kGroupsMax][D + 1][kWave];             // coordinates and upstream gradient of every point
+    __shared__ T gbox[kGroupsMax][2 * D];                   // bounding box of every group's points
+    __shared__ T result[kGroupsMax][kVals][kWave];
+    // per wavefront: the staged leaf records of a batch; between two groups its partial results per point
+    static_assert(kStageBatch * LS >= kVals * kWave, "staging area too small for the partial results");
+    __shared__ __attribute__((aligned(16))) T staged_mem[kTravWaves][kStageBatch * LS];
+    // double in both precisions: LDS atomic adds of doubles on distinct addresses cost a few cycles per
+    // instruction, those of floats are serialised lane by lane
+    __shared__ double rsum_mem[kTravWaves][NEED_GM ? kStageBatch * NR : 1];
     const int bl = blockIdx.x / chunks;
     const int chunk = blockIdx.x - bl * chunks;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const size_t xseg = size_t(xb) * Lx + xl;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     T* staged = staged_mem[wave];
+    double* rsum = rsum_mem[wave];
     const unsigned long long below = (1ull << lane) - 1ull;
 
-    // every wavefront holds the same 64 points, one per lane
-    const int j = chunk * kWave + lane;
-    const bool valid = j < N;
-    const int pid = valid ? p_order[xseg * N + j] : 0;
-    T x[D];
+    // wavefront i loads the points of group i and their bounding box
+    int sp = 0;                                             // nodes on this wavefront's stack (wave-uniform)
+    if (wave < groups) {
+        // The groups of a workgroup lie far apart in Morton order, one in every quarter of the range and at
+        // different places within the quarters: point groups with long candidate lists come in clusters (dense
+        // regions), often at matching places of a symmetric point set.
+        const int group = wave * chunks + (chunk + wave * (chunks / (groups + 1))) % chunks;
+        const int j = group * kWave + lane;
+        const bool valid = j < N;
+        const int pid = valid ? p_order[xseg * N + j] : 0;
+        T x[D];
 #pragma unroll
-    for (int d = 0; d < D; ++d) x[d] = xes[(xseg * N + pid) * D + d];
-    T g = T(0);
-    if (MODE == 1) g = valid ? grad_out[size_t(bl) * N + pid] : T(0);
-    T glo[D], ghi[D];
+        for (int d = 0; d < D; ++d) x[d] = xes[(xseg * N + pid) * D + d];
+        T g = T(0);
+        if (MODE == 1) g = valid ? grad_out[size_t(bl) * N + pid] : T(0);
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-        glo[d] = wave_min(valid ? x[d] : T(INFINITY));
-        ghi[d] = wave_max(valid ? x[d] : T(-INFINITY));
+        for (int d = 0; d < D; ++d) {
+            pts[wave][d][lane] = x[d];
+            const T lo = wave_min(valid ? x[d] : T(INFINITY)), hi = wave_max(valid ? x[d] : T(-INFINITY));
+            if (lane == 0) { gbox[wave][d] = lo; gbox[wave][D + d] = hi; }
+        }
+        pts[wave][D][lane] = g;
+        pids[wave][lane] = valid ? pid : -1;
+        const bool any = group * kWave < N;
+        if (lane == 0) {
+            // a single Gaussian is a tree without internal nodes: its leaf is the only candidate
+            stack[wave][0] = 0;
+            leaves[wave][0] = 0;
+            state[wave][0] = (any && M == 1) ? 1 : 0;
+            state[wave][1] = 0;
+        }
+        sp = (any && M > 1) ? 1 : 0;
     }
+    for (int i = threadIdx.x; i < kGroupsMax * kVals * kWave; i += kTravBlock) (&result[0][0][0])[i] = T(0);
 
-    const T* boxes = node_box + size_t(bl) * (2 * size_t(M) - 1) * 2 * D;
     const T* cboxes = child_box + size_t(bl) * (M - 1) * 4 * D;
     const int2* kids = children + size_t(bl) * (M - 1);
-    const T* recs = leaf_rec + size_t(bl) * M * RS;
-    T acc = T(0);
-    T gx[D];
-#pragma unroll
-    for (int d = 0; d < D; ++d) gx[d] = T(0);
+    const T* recs = leaf_rec + size_t(bl) * M * LS;
 
-    // `lf` points to a staged leaf in LDS: own box first, evaluation record behind it (read only on a hit)
-    auto visit_leaf = [&](const T* lf) {
-        T bx[2 * D];
+    // Phase 2 walks this wavefront's batches of the round, group after group, with a wave-uniform cursor; the
+    // leaf records of the NEXT batch (possibly of the next group) are fetched into registers before the current
+    // batch is tested and evaluated, so their memory round trip overlaps that work and the group's barriers.
+    constexpr int kPre = (kStageBatch * LS + kWave - 1) / kWave;
+    constexpr int kDenseHits = sizeof(T) == 8 ? 32 : 12;    // lanes per leaf from which the reduction is cheaper
+    int cur_group = -1, cur_base = 0, cur_end = 0;
+    T pre[kPre];
+    auto next_batch = [&]() {
+        cur_base += kStageBatch;
+        while (cur_base >= cur_end && cur_group < groups) {
+            ++cur_group;
+            if (cur_group >= groups) break;
+            const int n = __builtin_amdgcn_readfirstlane(state[cur_group][0]);
+            const int per = (n + kTravWaves - 1) / kTravWaves;
+            cur_base = wave * per;
+            cur_end = cur_base + per < n ? cur_base + per : n;
+        }
+    };
+    auto prefetch = [&]() {
+        if (cur_group >= groups) return;
+        const int cnt = cur_end - cur_base < kStageBatch ? cur_end - cur_base : kStageBatch;
 #pragma unroll
-        for (int k = 0; k < 2 * D; ++k) bx[k] = lf[k];
-        const bool in = valid & inside_box<T, D>(x, bx);
-        if (__ballot(in) == 0ull) return;
-        T r[RS];
+        for (int r = 0; r < kPre; ++r) {
+            const int s = lane + r * kWave;
+            if (s < cnt * LS) {
+                const int c = s / LS, k = s - c * LS;
+                pre[r] = recs[size_t(leaves[cur_group][cur_base + c]) * LS + k];
+            }
+        }
+    };
+    // all batches of group gi that belong to this wavefront; the cursor stands on the first of them (or beyond)
+    auto evaluate_share = [&](int gi) {
+        T x[D];
 #pragma unroll
-        for (int k = 0; k < RS; ++k) r[k] = lf[2 * D + k];
-        T t[D], u[D];
-        const T e = leaf_terms<T, D>(r, x, t, u);
-        const T amp = r[D + D * (D + 1) / 2];
-        if (MODE == 0) {
-            acc += in ? amp * e : T(0);
-        } else {
-            const T eg = in ? e * g : T(0);
-            if (NEED_GX) {
-                const T s = in ? amp * e : T(0);
+        for (int d = 0; d < D; ++d) x[d] = pts[gi][d][lane];
+        const T g = pts[gi][D][lane];
+        const bool valid = pids[gi][lane] >= 0;
+        T acc = T(0);
+        T gx[D];
 #pragma unroll
-                for (int d = 0; d < D; ++d) gx[d] = fma_(s, u[d], gx[d]);
+        for (int d = 0; d < D; ++d) gx[d] = T(0);
+        // lanes start at different leaves of a batch, so that LDS atomics of one instruction spread over the leaves
+        const int rot = NEED_GM ? lane % kStageBatch : 0;
+        while (cur_group == gi) {
+            const int cnt = cur_end - cur_base < kStageBatch ? cur_end - cur_base : kStageBatch;
+#pragma unroll
+            for (int r = 0; r < kPre; ++r) {
+                const int s = lane + r * kWave;
+                if (s < cnt * LS) staged[s] = pre[r];
+            }
+            if (NEED_GM)
+                for (int s = lane; s < cnt * NR; s += kWave) rsum[s] = 0.0;
+            wave_lds_fence();
+            next_batch();
+            prefetch();
+            unsigned mask = 0u;
+#pragma unroll 1
+            for (int i0 = 0; i0 < cnt; i0 += 2) {
+                T box[2][2 * D];
+#pragma unroll
+                for (int q = 0; q < 2; ++q)
+#pragma unroll
+                    for (int k = 0; k < 2 * D; ++k) box[q][k] = staged[(i0 + q) * LS + k];
+#pragma unroll
+                for (int q = 0; q < 2; ++q) mask |= (valid & inside_box<T, D>(x, box[q])) ? (1u << (i0 + q)) : 0u;
+            }
+            mask &= (1u << cnt) - 1u;                   // slots beyond the batch hold stale records
+            if (NEED_GM) {
+                // Leaves that contain many of the points: every lane evaluates the same leaf, the sums are
+                // reduced over the wavefront and lane 63 alone adds them to the LDS copy.  (LDS atomics serialise
+                // the lanes that add to the same address; a reduction costs the same however many lanes hit.)
+                for (int i = 0; i < cnt; ++i) {
+                    const bool has = (mask >> i) & 1u;
+                    if (__popcll(__ballot(has)) < kDenseHits) continue;
+                    mask &= ~(1u << i);
+                    const T* lf = staged + i * LS + 2 * D;
+                    T r[kAmp - 2 * D + 1];
+#pragma unroll
+                    for (int k = 0; k < kAmp - 2 * D + 1; ++k) r[k] = lf[k];
+                    T t[D], u[D];
+                    const T e = leaf_terms<T, D>(r, x, t, u);
+                    if (NEED_GX) {
+                        const T s = has ? r[kAmp - 2 * D] * e : T(0);
+#pragma unroll
+                        for (int d = 0; d < D; ++d) gx[d] = fma_(s, u[d], gx[d]);
+                    }
+                    T rs[NR];
+                    rs[0] = has ? e * g : T(0);
+#pragma unroll
+                    for (int d = 0; d < D; ++d) rs[1 + d] = rs[0] * t[d];
+                    int k = 1 + D;
+#pragma unroll
+                    for (int a = 0; a < D; ++a)
+#pragma unroll
+                        for (int c = a; c < D; ++c) rs[k++] = rs[1 + a] * t[c];
+#pragma unroll
+                    for (int q = 0; q < NR; ++q) rs[q] = wave_sum_to_lane63(rs[q]);
+                    if (lane == 63) {
+#pragma unroll
+                        for (int q = 0; q < NR; ++q) rsum[i * NR + q] += double(rs[q]);
+                    }
+                }
+                mask = ((mask >> rot) | (mask << (kStageBatch - rot))) & ((1u << kStageBatch) - 1u);
+            }
+            while (__ballot(mask != 0u) != 0ull) {
+                const bool has = mask != 0u;
+                int i = has ? __builtin_ctz(mask) + rot : 0;
+                i = i >= kStageBatch ? i - kStageBatch : i;
+                mask &= mask - 1u;
+                const T* lf = staged + i * LS + 2 * D;
+                T r[kAmp - 2 * D + 1];
+#pragma unroll
+                for (int k = 0; k < kAmp - 2 * D + 1; ++k) r[k] = lf[k];
+                T t[D], u[D];
+                const T e = leaf_terms<T, D>(r, x, t, u);
+                const T amp = r[kAmp - 2 * D];
+                if (MODE == 0) {
+                    acc += has ? amp * e : T(0);
+                } else {
+                    if (NEED_GX) {
+                        const T s = has ? amp * e : T(0);
+#pragma unroll
+                        for (int d = 0; d < D; ++d) gx[d] = fma_(s, u[d], gx[d]);
+                    }
+                    if (NEED_GM && has) {
+                        double* rs = rsum + i * NR;
+                        const T eg = e * g;
+                        atomic_add(&rs[0], double(eg));
+                        T rt[D];
+#pragma unroll
+                        for (int d = 0; d < D; ++d) { rt[d] = eg * t[d]; atomic_add(&rs[1 + d], double(rt[d])); }
+                        int k = 1 + D;
+#pragma unroll
+                        for (int a = 0; a < D; ++a)
+#pragma unroll
+                            for (int c = a; c < D; ++c) atomic_add(&rs[k++], double(rt[a] * t[c]));
+                    }
+                }
             }
             if (NEED_GM) {
-                T rs[NR];
-                rs[0] = eg;
-#pragma unroll
-                for (int d = 0; d < D; ++d) rs[1 + d] = eg * t[d];
-                int k = 1 + D;
-#pragma unroll
-                for (int a = 0; a < D; ++a)
-#pragma unroll
-                    for (int c = a; c < D; ++c) rs[k++] = rs[1 + a] * t[c];
-#pragma unroll
-                for (int i = 0; i < NR; ++i) rs[i] = wave_sum_to_lane63(rs[i]);
-                if (lane == 63) {
-                    const int comp = reinterpret_cast<const int*>(r + D + D * (D + 1) / 2 + 1)[0];
-                    T* dst = sums + (size_t(bl) * M + comp) * NR;
-#pragma unroll
-                    for (int i = 0; i < NR; ++i) atomic_add(&dst[i], rs[i]);
+                wave_lds_fence();
+                for (int s = lane; s < cnt * NR; s += kWave) {
+                    const int c = s / NR, k = s - c * NR;
+                    const T v = T(rsum[s]);
+                    if (v != T(0)) {
+                        const int comp = reinterpret_cast<const int*>(staged + c * LS + kAmp + 1)[0];
+                        atomic_add(&sums[(size_t(bl) * M + comp) * NR + k], v);
+                    }
                 }
             }
+            wave_lds_fence();
         }
-    };
-    // phase 2: this wavefront's share of the candidates [0, n)
-    auto evaluate_share = [&](int n) {
-        const int per = (n + kWaves - 1) / kWaves;
-        const int begin = wave * per, end = begin + per < n ? begin + per : n;
-        for (int base = begin; base < end; base += kStageBatch) {
-            const int cnt = end - base < kStageBatch ? end - base : kStageBatch;
-            if (lane < cnt) {
-                const int leaf = leaves[base + lane];
-                T* dst = staged + lane * LS;
+        if (MODE == 0 || NEED_GX) {
 #pragma unroll
-                for (int i = 0; i < 2 * D; ++i) dst[i] = boxes[(size_t(M - 1) + leaf) * 2 * D + i];
-#pragma unroll
-                for (int i = 0; i < RS; ++i) dst[2 * D + i] = recs[size_t(leaf) * RS + i];
-            }
-            wave_lds_fence();
-            for (int i = 0; i < cnt; ++i) visit_leaf(staged + i * LS);
-            wave_lds_fence();
+            for (int d = 0; d < kVals; ++d) staged[d * kWave + lane] = MODE == 0 ? acc : gx[d];   // staging area is idle now
         }
     };
 
-    if (M == 1) {
-        if (threadIdx.x == 0) leaves[0] = 0;
-        __syncthreads();
-        evaluate_share(1);
-    } else {
-        if (threadIdx.x == 0) { stack[0] = 0; shared_state[0] = 0; shared_state[1] = 1; }
-        __syncthreads();
-        // every round retires at least one of the M-1 internal nodes, each of which is pushed at most once
-        for (int round = 0; round < M; ++round) {
-            if (wave == 0) {
-                int sp = shared_state[1], n_leaf = 0;
-                for (int iter = 0; sp > 0 && n_leaf < kLeafFlush && iter < M; ++iter) {
-                    wave_lds_fence();
-                    // wide pops only while the stack has room for 64 more entries; a narrow pop is a depth-first
-                    // step, which adds at most one entry per tree level
-                    const int k = sp <= kStackCap - 128 ? (sp < 64 ? sp : 64) : 1;
-                    const bool active = lane < k;
-                    const int node = active ? stack[sp - 1 - lane] : 0;
-                    sp -= k;
-                    const int2 ch = kids[node];
-                    T cb[4 * D];
+    __syncthreads();
+    // every descent step retires at least one of the M-1 internal nodes, each of which is pushed at most once
+    for (int round = 0; round < M; ++round) {
+        if (sp > 0) {
+            int n_leaf = 0;
+            int* stk = stack[wave];
+            int* cand = leaves[wave];
+            T glo[D], ghi[D];
 #pragma unroll
-                    for (int i = 0; i < 4 * D; ++i) cb[i] = cboxes[size_t(node) * 4 * D + i];
-                    bool push[2], hit[2];
+            for (int d = 0; d < D; ++d) { glo[d] = gbox[wave][d]; ghi[d] = gbox[wave][D + d]; }
+            for (int iter = 0; sp > 0 && n_leaf < kLeafFlush && iter < M; ++iter) {
+                wave_lds_fence();
+                // wide pops only while the stack has room for 128 more entries; a narrow pop is a depth-first
+                // step, which adds at most one entry per tree level
+                const int k = sp <= kStackCap - 128 ? (sp < 64 ? sp : 64) : 1;
+                const bool active = lane < k;
+                const int node = active ? stk[sp - 1 - lane] : 0;
+                sp -= k;
+                const int2 ch = kids[node];
+                T cb[4 * D];
 #pragma unroll
-                    for (int side = 0; side < 2; ++side) {
-                        const int c = side == 0 ? ch.x : ch.y;
-                        bool ov = active & (c < M - 1) & (~c < M);          // a node of this tree
+                for (int i = 0; i < 4 * D; ++i) cb[i] = cboxes[size_t(node) * 4 * D + i];
+                bool push[2], hit[2];
 #pragma unroll
-                        for (int d = 0; d < D; ++d)
-                            ov = ov & (cb[side * 2 * D + d] <= ghi[d]) & (cb[side * 2 * D + D + d] >= glo[d]);
-                        push[side] = ov & (c >= 0);
-                        hit[side] = ov & (c < 0);
-                    }
-                    wave_lds_fence();
+                for (int side = 0; side < 2; ++side) {
+                    const int c = side == 0 ? ch.x : ch.y;
+                    bool ov = active & (c < M - 1) & (~c < M);          // a node of this tree
 #pragma unroll
-                    for (int side = 0; side < 2; ++side) {
-                        const int c = side == 0 ? ch.x : ch.y;
-                        const unsigned long long mp = __ballot(push[side]), mh = __ballot(hit[side]);
-                        const int at = sp + __popcll(mp & below);
-                        if (push[side] && at < kStackCap + 128) stack[at] = c;     // always in range, see the pop rule
-                        sp += __popcll(mp);
-                        if (hit[side]) leaves[n_leaf + __popcll(mh & below)] = ~c;
-                        n_leaf += __popcll(mh);
-                    }
+                    for (int d = 0; d < D; ++d)
+                        ov = ov & (cb[side * 2 * D + d] <= ghi[d]) & (cb[side * 2 * D + D + d] >= glo[d]);
+                    push[side] = ov & (c >= 0);
+                    hit[side] = ov & (c < 0);
                 }
-                if (lane == 0) { shared_state[0] = n_leaf; shared_state[1] = sp; }
+                wave_lds_fence();
+#pragma unroll
+                for (int side = 0; side < 2; ++side) {
+                    const int c = side == 0 ? ch.x : ch.y;
+                    const unsigned long long mp = __ballot(push[side]), mh = __ballot(hit[side]);
+                    const int at = sp + __popcll(mp & below);
+                    if (push[side] && at < kStackCap + 128) stk[at] = c;       // always in range, see the pop rule
+                    sp += __popcll(mp);
+                    if (hit[side]) cand[n_leaf + __popcll(mh & below)] = ~c;
+                    n_leaf += __popcll(mh);
+                }
+            }
+            if (lane == 0) { state[wave][0] = n_leaf; state[wave][1] = sp; }
+        }
+        __syncthreads();
+        bool left_on_stack = false;
+        cur_group = -1; cur_base = 0; cur_end = 0;
+        next_batch();
+        prefetch();
+        for (int gi = 0; gi < groups; ++gi) {
+            const int n_leaf = state[gi][0];
+            left_on_stack |= state[gi][1] > 0;
+            if (n_leaf == 0) continue;                                  // uniform over the workgroup
+            evaluate_share(gi);
+            __syncthreads();
+            if ((MODE == 0 || NEED_GX) && wave < kVals) {
+                T v = T(0);
+#pragma unroll
+                for (int w = 0; w < kTravWaves; ++w) v += staged_mem[w][wave * kWave + lane];
+                result[gi][wave][lane] += v;
             }
             __syncthreads();
-            const int n_leaf = shared_state[0], left_on_stack = shared_state[1];
-            evaluate_share(n_leaf);
-            __syncthreads();
-            if (left_on_stack == 0) break;
         }
+        if (!left_on_stack) break;
+        __syncthreads();                                                // every wavefront has read this round's state
+        // a group without nodes left gathers nothing in later rounds
+        if (wave < groups && sp == 0 && lane == 0) state[wave][0] = 0;
     }
 
-    // add the wavefronts' partial results per point (the staging area is free now)
     __syncthreads();
-    T* red = &staged_mem[0][0];
-    constexpr int kVals = MODE == 0 ? 1 : D;
-    if (MODE == 0 || NEED_GX) {
-#pragma unroll
-        for (int d = 0; d < kVals; ++d) red[(wave * kVals + d) * kWave + lane] = MODE == 0 ? acc : gx[d];
-    }
-    __syncthreads();
-    if (wave != 0 || !valid) return;
+    if (wave >= groups) return;
+    const int pid = pids[wave][lane];
+    if (pid < 0) return;
     if (MODE == 0) {
-        T v = T(0);
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) v += red[w * kWave + lane];
-        out[size_t(bl) * N + pid] = v;
+        out[size_t(bl) * N + pid] = result[wave][0][lane];
     } else if (NEED_GX) {
+        const T g = pts[wave][D][lane];
         T* dst = grad_xes + (xseg * N + pid) * D;
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-            T v = T(0);
-#pragma unroll
-            for (int w = 0; w < kWaves; ++w) v += red[(w * D + d) * kWave + lane];
-            v = -g * v;
+            const T v = -g * result[wave][d][lane];
             if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
         }
     }
@@ -1024,6 +1161,16 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
+// 64-point groups per traversal workgroup: one while every workgroup of the launch is resident at once anyway,
+// more (their descents then overlap inside the workgroup) when the launch would otherwise need several rounds
+static int traversal_groups(size_t BL, int N) {
+    const size_t per_mixture = (size_t(N) + kWave - 1) / kWave;
+    const size_t want = (BL * per_mixture + kTravSlots - 1) / kTravSlots;
+    size_t g = want < size_t(kGroupsMax) ? want : size_t(kGroupsMax);
+    if (g > per_mixture) g = per_mixture;
+    return g < 1 ? 1 : int(g);
+}
+
 template <typename T, int D>
 static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, hipStream_t st) {
     const BvhLayout lay = bvh_layout(s);
@@ -1034,11 +1181,11 @@ static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, 
         fill_zero_kernel<T><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(out, n);
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    const int chunks = (s.N + kWave - 1) / kWave;
+    const int groups = traversal_groups(BL, s.N);
+    const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kTravBlock), 0, st>>>(
-        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const T*)(bvh + lay.child_box),
-        (const int2*)(bvh + lay.children), (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N,
-        s.Bx, s.Lx, chunks, 0);
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children),
+        (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, 0);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
@@ -1062,12 +1209,13 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, const ch
     }
     if (gm) zero(sums, n_g * NR);
     if (gx && xes_shared) zero(grad_xes, n_x);
-    const int chunks = (s.N + kWave - 1) / kWave;
+    const int groups = traversal_groups(BL, s.N);
+    const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     const dim3 grid(unsigned(BL * chunks));
 #define GMC_TRAV(GM, GX) bvh_traverse_kernel<T, D, 1, GM, GX><<<grid, dim3(kTravBlock), 0, st>>>( \
-        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.node_box), (const T*)(bvh + lay.child_box), \
-        (const int2*)(bvh + lay.children), (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, s.L, s.M, s.N, \
-        s.Bx, s.Lx, chunks, xes_shared)
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children), \
+        (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, \
+        xes_shared)
     if (gm && gx) GMC_TRAV(true, true);
     else if (gm) GMC_TRAV(true, false);
     else if (gx) GMC_TRAV(false, true);

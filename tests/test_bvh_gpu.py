@@ -138,6 +138,24 @@ def test_culled_matches_masked_dense_sum(dtype, D, mode):
         assert rel_l2(out, dense) < 0.05
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_several_point_groups_per_workgroup(dtype):
+    """Launches with more 64-point groups than resident workgroups give every workgroup two to four groups (their
+    descents overlap); the last groups are ragged or empty.  Narrow Gaussians exercise the lane-by-lane evaluation
+    with LDS atomics, wide ones the wavefront reduction and candidate lists that are evaluated in several rounds."""
+    seed = 350
+    for B, L, M, N, D, cov in ((4, 4, 50, 2577, 3, 0.3), (4, 4, 40, 5000, 2, 0.3), (2, 8, 30, 8200, 3, 0.05),
+                               (1, 9, 20, 64 * 57 + 1, 3, 0.3)):
+        seed += 1
+        mix, xes, gout = _case(B, L, M, N, D, seed, cov_radius=cov)
+        _check_culled(mix, xes, gout, dtype, "tight", tag=f"B{B} L{L} M{M} N{N} D{D} cov{cov}")
+    # every box contains nearly every point: more candidates per group than one round gathers
+    mix, xes, gout = _case(1, 2, 700, 300, 3, seed + 1, spread=1.0, cov_radius=3.0)
+    _check_culled(mix, xes, gout, dtype, "tight", tag="wide")
+    mix, xes, gout = _case(9, 1, 600, 64 * 60, 2, seed + 2, spread=1.0, cov_radius=3.0)
+    _check_culled(mix, xes, gout, dtype, "tight", tag="wide, several groups")
+
+
 def test_points_outside_every_box_and_need_flags():
     mix, xes, gout = _case(1, 2, 40, 64, 3, seed=400)
     far = xes + 1000.0
