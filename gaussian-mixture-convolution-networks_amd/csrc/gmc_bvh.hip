@@ -37,20 +37,28 @@ struct BvhLayout {
     size_t parent;              // int [BL][2M-1]
     size_t leaf_comp;           // int [BL][M]             component id of each leaf
     size_t enc_box;             // int64 [BL][M-1][2D]     boxes of the internal nodes as order-preserving integers
-    size_t g_bounds;            // T [BL][2D]              bounds of the centres
-    size_t p_bounds;            // T [BxLx][2D]            bounds of the query points
-    size_t part_bounds;         // T [segments][blocks][2D] per-block partial bounds
+    size_t part_bounds;         // T [segments][blocks][2D] per-block partial bounds of the centres / query points
     size_t keys_a, keys_b, vals_a, vals_b;   // uint32 [max(BL*M, BxLx*N)] radix ping-pong
-    size_t hist;                // uint32 [segments][256][blocks] block histograms, then [segments][256] digit totals
-    size_t hist_totals;         // offset of the digit totals inside the histogram area
+    size_t hist;                // uint32 [segments][blocks][256] block histograms of one radix pass
     size_t p_order;             // int [BxLx][N]           Morton order of the query points
     size_t g_keys;              // uint32 [BL][M]          sorted Morton codes of the leaves
     size_t total;
 };
 
-constexpr int kSortItems = 2;                       // items per lane and radix block
-constexpr int kSortChunk = kBlock * kSortItems;     // 512: small chunks, many workgroups (the passes are latency-bound)
-constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the first bounds pass
+constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
+constexpr int kSortBlocksMax = 256;                 // radix blocks per segment (more items per lane beyond that)
+constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the partial bounds of the query points
+
+// items per lane of a radix block for segments of `count` keys
+static int sort_items(size_t count) {
+    size_t items = kSortItems;
+    while ((count + kBlock * items - 1) / (kBlock * items) > size_t(kSortBlocksMax)) items *= 2;
+    return int(items);
+}
+static size_t sort_blocks(size_t count) {
+    const size_t chunk = size_t(kBlock) * sort_items(count);
+    return (count + chunk - 1) / chunk;
+}
 
 template <int D> struct LeafRec { static constexpr int kStride = (D == 2) ? 12 : 18; };
 // own box (lower[D], upper[D]), then  D=3: b0 b1 b2 c00 c01 c02 c11 c12 c22 amp comp -   D=2: b0 b1 c00 c01 c11 amp comp -
@@ -75,10 +83,8 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.parent = take(BL * nodes * 4);
     l.leaf_comp = take(BL * M * 4);
     l.enc_box = take(BL * (M > 0 ? M - 1 : 0) * 2 * D * 8);
-    l.g_bounds = take(BL * 2 * D * e);
-    l.p_bounds = take(XL * 2 * D * e);
     {
-        const size_t pg = BL * ((M + kBoundsChunk - 1) / kBoundsChunk), pp = XL * ((N + kBoundsChunk - 1) / kBoundsChunk);
+        const size_t pg = BL * ((M + kBlock - 1) / kBlock), pp = XL * ((N + kBoundsChunk - 1) / kBoundsChunk);
         l.part_bounds = take((pg > pp ? pg : pp) * 2 * D * e);
     }
     const size_t items = BL * M > XL * N ? BL * M : XL * N;
@@ -86,9 +92,8 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.keys_b = take(items * 4);
     l.vals_a = take(items * 4);
     l.vals_b = take(items * 4);
-    const size_t bg = BL * ((M + kSortChunk - 1) / kSortChunk), bp = XL * ((N + kSortChunk - 1) / kSortChunk);
+    const size_t bg = BL * sort_blocks(M), bp = XL * sort_blocks(N);
     l.hist = take((bg > bp ? bg : bp) * 256 * 4);
-    l.hist_totals = take((BL > XL ? BL : XL) * 256 * 4);
     l.p_order = take(XL * N * 4);
     l.g_keys = take(BL * M * 4);
     l.total = o;
@@ -236,44 +241,10 @@ __device__ inline void box_half_extent(const T* __restrict__ g, double threshold
     for (int k = 0; k < D; ++k) delta[k] = s * (literal ? lit[k] : tight[k]);
 }
 
+// minimum / maximum over the workgroup of every lane's (lo, hi); thread t < 2D returns component t of
+// (min_0..min_D-1, max_0..max_D-1), the other threads return garbage
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
-                                                          T* __restrict__ box_hi, size_t n, double threshold, int mode) {
-    constexpr int G = 1 + D + D * D;
-    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
-    if (i >= n) return;
-    const T* g = mixture + i * G;
-    double delta[D];
-    box_half_extent<T, D>(g, threshold, mode, delta);
-    for (int k = 0; k < D; ++k) {
-        box_lo[i * D + k] = T(double(g[1 + k]) - delta[k]);
-        box_hi[i * D + k] = T(double(g[1 + k]) + delta[k]);
-    }
-}
-
-// ---------------------------------------------------------------------------------------------------------------
-// bounds of a point set, Morton keys
-// ---------------------------------------------------------------------------------------------------------------
-
-// Bounds of `count` points per segment in two passes.  Pass 1: workgroup (blk, seg) reduces kBoundsChunk points
-// to parts[seg][blk] = (min_0..min_D-1, max_0..max_D-1); pass 2 runs the same kernel over the partial results
-// (`hi_off` = D: maxima are taken from the second half of every partial record).
-template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bounds_kernel(const T* __restrict__ pts, int stride, int offset, int hi_off,
-                                                       int count, int chunk, int blocks_per_seg, T* __restrict__ out) {
-    __shared__ T red[2 * D][kBlock];
-    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
-    const T* p = pts + size_t(seg) * count * stride + offset;
-    const int begin = blk * chunk;
-    const int end = begin + chunk < count ? begin + chunk : count;
-    T lo[D], hi[D];
-    for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
-    for (int i = begin + threadIdx.x; i < end; i += kBlock)
-        for (int d = 0; d < D; ++d) {
-            const T a = p[size_t(i) * stride + d], b = p[size_t(i) * stride + hi_off + d];
-            lo[d] = a < lo[d] ? a : lo[d];
-            hi[d] = b > hi[d] ? b : hi[d];
-        }
+__device__ __forceinline__ T block_bounds(const T (&lo)[D], const T (&hi)[D], T (*red)[kBlock]) {
     for (int d = 0; d < D; ++d) { red[d][threadIdx.x] = lo[d]; red[D + d][threadIdx.x] = hi[d]; }
     __syncthreads();
     for (int s = kBlock / 2; s > 0; s >>= 1) {
@@ -285,7 +256,60 @@ __global__ __launch_bounds__(kBlock) void bounds_kernel(const T* __restrict__ pt
             }
         __syncthreads();
     }
-    if (threadIdx.x < 2 * D) out[size_t(blockIdx.x) * 2 * D + threadIdx.x] = red[threadIdx.x][0];
+    return red[threadIdx.x < 2 * D ? threadIdx.x : 0][0];
+}
+
+// cutoff box of every Gaussian; workgroup (blk, seg) also leaves the bounds of its 256 centres in parts[seg][blk]
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
+                                                          T* __restrict__ box_hi, int M, int blocks_per_seg,
+                                                          double threshold, int mode, T* __restrict__ parts) {
+    constexpr int G = 1 + D + D * D;
+    __shared__ T red[2 * D][kBlock];
+    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    const int m = blk * kBlock + threadIdx.x;
+    T lo[D], hi[D];
+    for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
+    if (m < M) {
+        const size_t i = size_t(seg) * M + m;
+        const T* g = mixture + i * G;
+        double delta[D];
+        box_half_extent<T, D>(g, threshold, mode, delta);
+        for (int k = 0; k < D; ++k) {
+            box_lo[i * D + k] = T(double(g[1 + k]) - delta[k]);
+            box_hi[i * D + k] = T(double(g[1 + k]) + delta[k]);
+            lo[k] = g[1 + k] < lo[k] ? g[1 + k] : lo[k];          // comparisons as in bounds_kernel: NaN is skipped
+            hi[k] = g[1 + k] > hi[k] ? g[1 + k] : hi[k];
+        }
+    }
+    const T v = block_bounds<T, D>(lo, hi, red);
+    if (threadIdx.x < 2 * D) parts[size_t(blockIdx.x) * 2 * D + threadIdx.x] = v;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// bounds of a point set, Morton keys
+// ---------------------------------------------------------------------------------------------------------------
+
+// Partial bounds of `count` points per segment: workgroup (blk, seg) reduces `chunk` points to
+// parts[seg][blk] = (min_0..min_D-1, max_0..max_D-1); the Morton kernel combines the partial records.
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bounds_kernel(const T* __restrict__ pts, int stride, int offset, int count,
+                                                       int chunk, int blocks_per_seg, T* __restrict__ out) {
+    __shared__ T red[2 * D][kBlock];
+    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    const T* p = pts + size_t(seg) * count * stride + offset;
+    const int begin = blk * chunk;
+    const int end = begin + chunk < count ? begin + chunk : count;
+    T lo[D], hi[D];
+    for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
+    for (int i = begin + threadIdx.x; i < end; i += kBlock)
+        for (int d = 0; d < D; ++d) {
+            const T a = p[size_t(i) * stride + d];
+            lo[d] = a < lo[d] ? a : lo[d];
+            hi[d] = a > hi[d] ? a : hi[d];
+        }
+    const T v = block_bounds<T, D>(lo, hi, red);
+    if (threadIdx.x < 2 * D) out[size_t(blockIdx.x) * 2 * D + threadIdx.x] = v;
 }
 
 __device__ __forceinline__ uint32_t expand_bits3(uint32_t v) {
@@ -311,68 +335,80 @@ __device__ __forceinline__ uint32_t morton30(const T* __restrict__ p, const T* _
     return code;
 }
 
+// Morton keys of the points of segment `seg` (workgroup (blk, seg), 256 points); every workgroup first combines
+// the segment's `n_parts` partial bounds
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void morton_kernel(const T* __restrict__ pts, int stride, int offset, int count,
-                                                       const T* __restrict__ bounds, uint32_t* __restrict__ keys,
-                                                       uint32_t* __restrict__ vals, size_t total) {
-    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
-    if (i >= total) return;
-    const size_t seg = i / count;
-    keys[i] = morton30<T, D>(pts + i * stride + offset, bounds + seg * 2 * D);
-    vals[i] = uint32_t(i - seg * count);
+                                                       int blocks_per_seg, const T* __restrict__ parts, int n_parts,
+                                                       uint32_t* __restrict__ keys, uint32_t* __restrict__ vals) {
+    __shared__ T red[2 * D][kBlock];
+    __shared__ T bounds[2 * D];
+    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    T lo[D], hi[D];
+    for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
+    for (int i = threadIdx.x; i < n_parts; i += kBlock) {
+        const T* q = parts + (size_t(seg) * n_parts + i) * 2 * D;
+        for (int d = 0; d < D; ++d) {
+            lo[d] = q[d] < lo[d] ? q[d] : lo[d];
+            hi[d] = q[D + d] > hi[d] ? q[D + d] : hi[d];
+        }
+    }
+    const T v = block_bounds<T, D>(lo, hi, red);
+    if (threadIdx.x < 2 * D) bounds[threadIdx.x] = v;
+    __syncthreads();
+    const int i = blk * kBlock + threadIdx.x;
+    if (i >= count) return;
+    const size_t at = size_t(seg) * count + i;
+    keys[at] = morton30<T, D>(pts + at * stride + offset, bounds);
+    vals[at] = uint32_t(i);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
 // segmented LSD radix sort, 8 bits per pass, stable; segments of equal length `count`
 // ---------------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void radix_hist_kernel(const uint32_t* __restrict__ keys, int count, int blocks_per_seg,
-                                                           int shift, uint32_t* __restrict__ hist) {
+__global__ __launch_bounds__(kBlock) void radix_hist_kernel(const uint32_t* __restrict__ keys, int count, int chunk,
+                                                           int blocks_per_seg, int shift, uint32_t* __restrict__ hist) {
     __shared__ uint32_t h[256];
     const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
     h[threadIdx.x] = 0;
     __syncthreads();
     const uint32_t* k = keys + size_t(seg) * count;
-    const int begin = blk * kSortChunk;
-    const int end = begin + kSortChunk < count ? begin + kSortChunk : count;
+    const int begin = blk * chunk;
+    const int end = begin + chunk < count ? begin + chunk : count;
     for (int i = begin + threadIdx.x; i < end; i += kBlock) atomicAdd(&h[(k[i] >> shift) & 255u], 1u);
     __syncthreads();
-    // digit-major layout so that one exclusive scan over (digit, block) yields the scatter offsets
-    hist[(size_t(seg) * 256 + threadIdx.x) * blocks_per_seg + blk] = h[threadIdx.x];
-}
-
-// one wavefront per (segment, digit): exclusive scan of that digit's block counts, digit total to `totals`
-__global__ __launch_bounds__(kWave) void radix_scan_kernel(uint32_t* __restrict__ hist, uint32_t* __restrict__ totals,
-                                                          int blocks_per_seg) {
-    uint32_t* h = hist + size_t(blockIdx.x) * blocks_per_seg;
-    const int lane = threadIdx.x;
-    uint32_t carry = 0;
-    for (int base = 0; base < blocks_per_seg; base += kWave) {
-        const int b = base + lane;
-        const uint32_t c = b < blocks_per_seg ? h[b] : 0u;
-        uint32_t incl = c;
-#pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
-            const uint32_t o = __shfl_up(incl, off, kWave);
-            if (lane >= off) incl += o;
-        }
-        if (b < blocks_per_seg) h[b] = carry + incl - c;
-        carry += __shfl(incl, kWave - 1, kWave);
-    }
-    if (lane == 0) totals[blockIdx.x] = carry;
+    hist[(size_t(seg) * blocks_per_seg + blk) * 256 + threadIdx.x] = h[threadIdx.x];
 }
 
 __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const uint32_t* __restrict__ keys_in,
                                                               const uint32_t* __restrict__ vals_in,
                                                               uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
-                                                              int count, int blocks_per_seg, int shift,
-                                                              const uint32_t* __restrict__ hist,
-                                                              const uint32_t* __restrict__ totals) {
+                                                              int count, int items, int blocks_per_seg, int shift,
+                                                              const uint32_t* __restrict__ hist) {
     __shared__ uint32_t running[256];        // next output slot of every digit for this block
     __shared__ uint32_t wave_count[4][256];
     const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // thread d: keys of digit d in the whole segment and in the blocks before this one (at most kSortBlocksMax
+    // counts per digit, so no separate scan pass is needed)
+    uint32_t mine = 0, earlier = 0;
+    {
+        const uint32_t* col = hist + size_t(seg) * blocks_per_seg * 256 + threadIdx.x;
+        int b = 0;
+        for (; b + 8 <= blocks_per_seg; b += 8) {           // eight independent loads in flight
+            uint32_t c[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) c[q] = col[size_t(b + q) * 256];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) { mine += c[q]; earlier += b + q < blk ? c[q] : 0u; }
+        }
+        for (; b < blocks_per_seg; ++b) {
+            const uint32_t c = col[size_t(b) * 256];
+            mine += c;
+            earlier += b < blk ? c : 0u;
+        }
+    }
     // exclusive scan of the segment's digit totals (Hillis-Steele on LDS) = first slot of every digit
-    const uint32_t mine = totals[size_t(seg) * 256 + threadIdx.x];
     running[threadIdx.x] = mine;
 #pragma unroll
     for (int w = 0; w < 4; ++w) wave_count[w][threadIdx.x] = 0;
@@ -383,13 +419,13 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const uint32_t* _
         running[threadIdx.x] += add;
         __syncthreads();
     }
-    running[threadIdx.x] += hist[(size_t(seg) * 256 + threadIdx.x) * blocks_per_seg + blk] - mine;
+    running[threadIdx.x] += earlier - mine;
     __syncthreads();
     const size_t seg_off = size_t(seg) * count;
-    const int begin = blk * kSortChunk;
-    for (int round = 0; round < kSortItems; ++round) {
+    const int begin = blk * items * kBlock;
+    for (int round = 0; round < items; ++round) {
         const int i = begin + round * kBlock + threadIdx.x;
-        const bool valid = i < count && i < begin + kSortChunk;
+        const bool valid = i < count;
         uint32_t key = 0, val = 0, digit = 0;
         if (valid) { key = keys_in[seg_off + i]; val = vals_in[seg_off + i]; digit = (key >> shift) & 255u; }
         // lanes of this wavefront holding the same digit
@@ -434,12 +470,59 @@ __device__ __forceinline__ double from_ordered_bits(long long k) {
     return __builtin_bit_cast(double, k ^ ((k >> 63) & 0x7fffffffffffffffll));
 }
 
+// number of leading bits shared by the unique keys (morton[i] << 32 | i) and (morton[j] << 32 | j); -1 outside
+__device__ __forceinline__ int common_prefix(const uint32_t* __restrict__ keys, int n, int i, int j) {
+    if (j < 0 || j >= n) return -1;
+    const uint32_t a = keys[i], b = keys[j];
+    if (a != b) return __clz(a ^ b);
+    return 32 + __clz(uint32_t(i) ^ uint32_t(j));
+}
+
+// internal node i of the radix tree of mixture bl (Karras 2012; lbvh/building.h:11-103)
+__device__ __forceinline__ void build_internal_node(const uint32_t* __restrict__ keys, int2* __restrict__ children,
+                                                    int* __restrict__ parent, int M, size_t bl, int i) {
+    const size_t t = bl * (M - 1) + i;
+    const uint32_t* k = keys + bl * M;
+    // range of keys covered by internal node i
+    int first, last;
+    if (i == 0) { first = 0; last = M - 1; }
+    else {
+        const int dl = common_prefix(k, M, i, i - 1), dr = common_prefix(k, M, i, i + 1);
+        const int dir = dr > dl ? 1 : -1;
+        const int dmin = dr > dl ? dl : dr;
+        int lmax = 2;
+        while (common_prefix(k, M, i, i + lmax * dir) > dmin) lmax <<= 1;
+        int len = 0;
+        for (int step = lmax >> 1; step > 0; step >>= 1)
+            if (common_prefix(k, M, i, i + (len + step) * dir) > dmin) len += step;
+        const int j = i + len * dir;
+        first = i < j ? i : j;
+        last = i < j ? j : i;
+    }
+    // split: the highest key that shares more than the node's prefix with the first key
+    const int dnode = common_prefix(k, M, first, last);
+    int split = first, stride = last - first;
+    do {
+        stride = (stride + 1) >> 1;
+        const int mid = split + stride;
+        if (mid < last && common_prefix(k, M, first, mid) > dnode) split = mid;
+    } while (stride > 1);
+    const int left = (split == first) ? ~split : split;               // leaf `split` or internal node `split`
+    const int right = (split + 1 == last) ? ~(split + 1) : split + 1;
+    children[t] = make_int2(left, right);
+    int* par = parent + bl * (2 * size_t(M) - 1);
+    par[left >= 0 ? left : (M - 1) + ~left] = i;
+    par[right >= 0 ? right : (M - 1) + ~right] = i;
+    if (i == 0) par[0] = -1;
+}
+
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, const T* __restrict__ box_lo,
                                                            const T* __restrict__ box_hi, const uint32_t* __restrict__ order,
-                                                           T* __restrict__ node_box, T* __restrict__ leaf_rec,
-                                                           long long* __restrict__ enc_box,
-                                                           int* __restrict__ parent, int M, size_t total) {
+                                                           const uint32_t* __restrict__ keys, T* __restrict__ node_box,
+                                                           T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
+                                                           int2* __restrict__ children, int* __restrict__ parent, int M,
+                                                           size_t total) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
     const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
@@ -479,55 +562,8 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         r[9] = T(double(g[0]) * Kappa<3>::v * sqrt(det));
         reinterpret_cast<int*>(r + 10)[0] = comp;
     }
-}
-
-// number of leading bits shared by the unique keys (morton[i] << 32 | i) and (morton[j] << 32 | j); -1 outside
-__device__ __forceinline__ int common_prefix(const uint32_t* __restrict__ keys, int n, int i, int j) {
-    if (j < 0 || j >= n) return -1;
-    const uint32_t a = keys[i], b = keys[j];
-    if (a != b) return __clz(a ^ b);
-    return 32 + __clz(uint32_t(i) ^ uint32_t(j));
-}
-
-__global__ __launch_bounds__(kBlock) void bvh_tree_kernel(const uint32_t* __restrict__ keys, int2* __restrict__ children,
-                                                         int* __restrict__ parent, int M, size_t total) {
-    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
-    if (t >= total) return;
-    const int n_int = M - 1;
-    const size_t bl = t / n_int;
-    const int i = int(t - bl * n_int);
-    const uint32_t* k = keys + bl * M;
-    // range of keys covered by internal node i
-    int first, last;
-    if (i == 0) { first = 0; last = M - 1; }
-    else {
-        const int dl = common_prefix(k, M, i, i - 1), dr = common_prefix(k, M, i, i + 1);
-        const int dir = dr > dl ? 1 : -1;
-        const int dmin = dr > dl ? dl : dr;
-        int lmax = 2;
-        while (common_prefix(k, M, i, i + lmax * dir) > dmin) lmax <<= 1;
-        int len = 0;
-        for (int step = lmax >> 1; step > 0; step >>= 1)
-            if (common_prefix(k, M, i, i + (len + step) * dir) > dmin) len += step;
-        const int j = i + len * dir;
-        first = i < j ? i : j;
-        last = i < j ? j : i;
-    }
-    // split: the highest key that shares more than the node's prefix with the first key
-    const int dnode = common_prefix(k, M, first, last);
-    int split = first, stride = last - first;
-    do {
-        stride = (stride + 1) >> 1;
-        const int mid = split + stride;
-        if (mid < last && common_prefix(k, M, first, mid) > dnode) split = mid;
-    } while (stride > 1);
-    const int left = (split == first) ? ~split : split;               // leaf `split` or internal node `split`
-    const int right = (split + 1 == last) ? ~(split + 1) : split + 1;
-    children[t] = make_int2(left, right);
-    int* par = parent + bl * (2 * size_t(M) - 1);
-    par[left >= 0 ? left : (M - 1) + ~left] = i;
-    par[right >= 0 ? right : (M - 1) + ~right] = i;
-    if (i == 0) par[0] = -1;
+    // the same lane builds internal node `leaf` of the tree (there are M-1 of them); nothing above depends on it
+    if (leaf < M - 1) build_internal_node(keys, children, parent, M, bl, leaf);
 }
 
 // Bottom-up boxes without inter-lane ordering: one lane per leaf walks towards the root and merges ITS OWN leaf
@@ -1082,9 +1118,9 @@ static unsigned grid_for(size_t n) { return unsigned((n + kBlock - 1) / kBlock);
 // sorts `segments` segments of `count` (key, value) pairs held in (ka, va) on the key bits
 // [first_bit, first_bit + 8 * passes), ping-ponging with (kb, vb); the last pass writes to (keys_out, vals_out)
 static void radix_sort(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* keys_out, uint32_t* vals_out,
-                       uint32_t* hist, uint32_t* totals, int segments, int count, int first_bit, int passes,
-                       hipStream_t st) {
-    const int bps = (count + kSortChunk - 1) / kSortChunk;
+                       uint32_t* hist, int segments, int count, int first_bit, int passes, hipStream_t st) {
+    const int items = sort_items(size_t(count));
+    const int bps = int(sort_blocks(size_t(count)));
     const dim3 grid(unsigned(size_t(segments) * bps));
     int cur = 0;
     for (int p = 0; p < passes; ++p) {
@@ -1092,20 +1128,10 @@ static void radix_sort(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, u
         uint32_t* kout = cur ? ka : kb; uint32_t* vout = cur ? va : vb;
         if (p == passes - 1) { kout = keys_out; vout = vals_out; }
         const int shift = first_bit + 8 * p;
-        radix_hist_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, count, bps, shift, hist);
-        radix_scan_kernel<<<dim3(unsigned(segments) * 256), dim3(kWave), 0, st>>>(hist, totals, bps);
-        radix_scatter_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, vin, kout, vout, count, bps, shift, hist, totals);
+        radix_hist_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, count, items * kBlock, bps, shift, hist);
+        radix_scatter_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, vin, kout, vout, count, items, bps, shift, hist);
         cur ^= 1;
     }
-}
-
-template <typename T, int D>
-static void launch_bounds_of(const T* pts, int stride, int offset, int count, size_t segments, T* parts, T* out,
-                             hipStream_t st) {
-    const int nb = (count + kBoundsChunk - 1) / kBoundsChunk;
-    bounds_kernel<T, D><<<dim3(unsigned(segments * nb)), dim3(kBlock), 0, st>>>(pts, stride, offset, 0, count, kBoundsChunk,
-                                                                              nb, parts);
-    bounds_kernel<T, D><<<dim3(unsigned(segments)), dim3(kBlock), 0, st>>>(parts, 2 * D, 0, D, nb, nb, 1, out);
 }
 
 template <typename T, int D>
@@ -1122,24 +1148,21 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     uint32_t* ka = (uint32_t*)(bvh + lay.keys_a); uint32_t* kb = (uint32_t*)(bvh + lay.keys_b);
     uint32_t* va = (uint32_t*)(bvh + lay.vals_a); uint32_t* vb = (uint32_t*)(bvh + lay.vals_b);
     uint32_t* hist = (uint32_t*)(bvh + lay.hist);
-    uint32_t* totals = (uint32_t*)(bvh + lay.hist_totals);
     T* parts = (T*)(bvh + lay.part_bounds);
     T* child_box = (T*)(bvh + lay.child_box);
     if (BL > 0 && M > 0) {
         const size_t n = BL * M;
-        bvh_boxes_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, n,
-                                                                          double(cfg.aabb_threshold), cfg.aabb_mode);
-        T* gb = (T*)(bvh + lay.g_bounds);
-        launch_bounds_of<T, D>(mixture, G, 1, M, BL, parts, gb, st);
-        morton_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, G, 1, M, gb, ka, va, n);
+        const int bpm = (M + kBlock - 1) / kBlock;          // workgroups per mixture
+        bvh_boxes_kernel<T, D><<<dim3(unsigned(BL * bpm)), dim3(kBlock), 0, st>>>(
+            mixture, box_lo, box_hi, M, bpm, double(cfg.aabb_threshold), cfg.aabb_mode, parts);
+        morton_kernel<T, D><<<dim3(unsigned(BL * bpm)), dim3(kBlock), 0, st>>>(mixture, G, 1, M, bpm, parts, bpm, ka, va);
         uint32_t* g_keys = (uint32_t*)(bvh + lay.g_keys);
         uint32_t* g_order = (uint32_t*)leaf_comp;            // the sorted payload IS the component id of every leaf
-        radix_sort(ka, va, kb, vb, g_keys, g_order, hist, totals, int(BL), M, 0, 4, st);
-        bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, node_box,
-                                                                           leaf_rec, enc_box, parent, M, n);
+        radix_sort(ka, va, kb, vb, g_keys, g_order, hist, int(BL), M, 0, 4, st);
+        bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, g_keys,
+                                                                           node_box, leaf_rec, enc_box, children, parent, M, n);
         if (M > 1) {
             const size_t ni = BL * (M - 1);
-            bvh_tree_kernel<<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(g_keys, children, parent, M, ni);
             bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(parent, node_box, enc_box, M, n);
             bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(children, enc_box, node_box, child_box, M, ni);
         }
@@ -1148,12 +1171,12 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         int* p_order = (int*)(bvh + lay.p_order);
         const size_t n = XL * N;
         if (xes) {
-            T* pb = (T*)(bvh + lay.p_bounds);
-            launch_bounds_of<T, D>(xes, D, 0, N, XL, parts, pb, st);
-            morton_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(xes, D, 0, N, pb, ka, va, n);
+            const int nb = (N + kBoundsChunk - 1) / kBoundsChunk, bpx = (N + kBlock - 1) / kBlock;
+            bounds_kernel<T, D><<<dim3(unsigned(XL * nb)), dim3(kBlock), 0, st>>>(xes, D, 0, N, kBoundsChunk, nb, parts);
+            morton_kernel<T, D><<<dim3(unsigned(XL * bpx)), dim3(kBlock), 0, st>>>(xes, D, 0, N, bpx, parts, nb, ka, va);
             // 16 Morton bits (65536 cells) are enough to make 64 consecutive points neighbours
             // the sorted keys are not needed afterwards: they land in the spare key buffer
-            radix_sort(ka, va, kb, vb, ka, (uint32_t*)p_order, hist, totals, int(XL), N, 14, 2, st);
+            radix_sort(ka, va, kb, vb, ka, (uint32_t*)p_order, hist, int(XL), N, 14, 2, st);
         } else {
             iota_segments_kernel<<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(p_order, N, n);
         }
@@ -1161,12 +1184,13 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
-// 64-point groups per traversal workgroup: one while every workgroup of the launch is resident at once anyway,
-// more (their descents then overlap inside the workgroup) when the launch would otherwise need several rounds
+// 64-point groups per traversal workgroup.  More groups per workgroup overlap more descents and pay off when the
+// launch has many times more groups than resident workgroups; with few groups, smaller workgroups balance better
+// over the compute units (measured: 1563 groups run fastest with 2 per workgroup, 4096 and more with 4).
 static int traversal_groups(size_t BL, int N) {
     const size_t per_mixture = (size_t(N) + kWave - 1) / kWave;
-    const size_t want = (BL * per_mixture + kTravSlots - 1) / kTravSlots;
-    size_t g = want < size_t(kGroupsMax) ? want : size_t(kGroupsMax);
+    const size_t total = BL * per_mixture;
+    size_t g = total <= size_t(kTravSlots) ? 1 : total < 4 * size_t(kTravSlots) ? 2 : total < 8 * size_t(kTravSlots) ? 3 : kGroupsMax;
     if (g > per_mixture) g = per_mixture;
     return g < 1 ? 1 : int(g);
 }

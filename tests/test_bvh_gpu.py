@@ -145,7 +145,7 @@ def test_several_point_groups_per_workgroup(dtype):
     with LDS atomics, wide ones the wavefront reduction and candidate lists that are evaluated in several rounds."""
     seed = 350
     for B, L, M, N, D, cov in ((4, 4, 50, 2577, 3, 0.3), (4, 4, 40, 5000, 2, 0.3), (2, 8, 30, 8200, 3, 0.05),
-                               (1, 9, 20, 64 * 57 + 1, 3, 0.3)):
+                               (1, 9, 20, 64 * 57 + 1, 3, 0.3), (8, 8, 20, 4100, 3, 0.2)):
         seed += 1
         mix, xes, gout = _case(B, L, M, N, D, seed, cov_radius=cov)
         _check_culled(mix, xes, gout, dtype, "tight", tag=f"B{B} L{L} M{M} N{N} D{D} cov{cov}")
