@@ -37,9 +37,10 @@ struct BvhLayout {
     size_t parent;              // int [BL][2M-1]
     size_t leaf_comp;           // int [BL][M]             component id of each leaf
     size_t enc_box;             // int64 [BL][M-1][2D]     boxes of the internal nodes as order-preserving integers
-    size_t part_bounds;         // T [segments][blocks][2D] per-block partial bounds of the centres / query points
-    size_t keys_a, keys_b, vals_a, vals_b;   // uint32 [max(BL*M, BxLx*N)] radix ping-pong
-    size_t hist;                // uint32 [segments][blocks][256] block histograms of one radix pass
+    size_t parts_g, parts_p;    // T [segments][blocks][2D] per-block partial bounds of the centres / the query points
+    size_t keys_a, keys_b, vals_a, vals_b;       // uint32 [BL*M]   radix ping-pong of the leaves
+    size_t pkeys_a, pkeys_b, pvals_a, pvals_b;   // uint32 [BxLx*N] radix ping-pong of the query points
+    size_t hist_g, hist_p;      // uint32 [segments][blocks][256] block histograms of one radix pass
     size_t p_order;             // int [BxLx][N]           Morton order of the query points
     size_t g_keys;              // uint32 [BL][M]          sorted Morton codes of the leaves
     size_t total;
@@ -83,17 +84,18 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.parent = take(BL * nodes * 4);
     l.leaf_comp = take(BL * M * 4);
     l.enc_box = take(BL * (M > 0 ? M - 1 : 0) * 2 * D * 8);
-    {
-        const size_t pg = BL * ((M + kBlock - 1) / kBlock), pp = XL * ((N + kBoundsChunk - 1) / kBoundsChunk);
-        l.part_bounds = take((pg > pp ? pg : pp) * 2 * D * e);
-    }
-    const size_t items = BL * M > XL * N ? BL * M : XL * N;
-    l.keys_a = take(items * 4);
-    l.keys_b = take(items * 4);
-    l.vals_a = take(items * 4);
-    l.vals_b = take(items * 4);
-    const size_t bg = BL * sort_blocks(M), bp = XL * sort_blocks(N);
-    l.hist = take((bg > bp ? bg : bp) * 256 * 4);
+    l.parts_g = take(BL * ((M + kBlock - 1) / kBlock) * 2 * D * e);
+    l.parts_p = take(XL * ((N + kBoundsChunk - 1) / kBoundsChunk) * 2 * D * e);
+    l.keys_a = take(BL * M * 4);
+    l.keys_b = take(BL * M * 4);
+    l.vals_a = take(BL * M * 4);
+    l.vals_b = take(BL * M * 4);
+    l.pkeys_a = take(XL * N * 4);
+    l.pkeys_b = take(XL * N * 4);
+    l.pvals_a = take(XL * N * 4);
+    l.pvals_b = take(XL * N * 4);
+    l.hist_g = take(BL * sort_blocks(M) * 256 * 4);
+    l.hist_p = take(XL * sort_blocks(N) * 256 * 4);
     l.p_order = take(XL * N * 4);
     l.g_keys = take(BL * M * 4);
     l.total = o;
@@ -259,58 +261,58 @@ __device__ __forceinline__ T block_bounds(const T (&lo)[D], const T (&hi)[D], T 
     return red[threadIdx.x < 2 * D ? threadIdx.x : 0][0];
 }
 
-// cutoff box of every Gaussian; workgroup (blk, seg) also leaves the bounds of its 256 centres in parts[seg][blk]
+// One launch for two independent jobs.
+// Workgroups [0, box_blocks): cutoff box of every Gaussian; workgroup (blk, seg) also leaves the bounds of its 256
+// centres in parts_g[seg][blk].
+// Workgroups behind them: partial bounds of the query points; workgroup (blk, seg) reduces kBoundsChunk points to
+// parts_p[seg][blk] = (min_0..min_D-1, max_0..max_D-1).  The Morton kernel combines the partial records.
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
-                                                          T* __restrict__ box_hi, int M, int blocks_per_seg,
-                                                          double threshold, int mode, T* __restrict__ parts) {
+                                                          T* __restrict__ box_hi, int M, int blocks_per_mixture,
+                                                          double threshold, int mode, T* __restrict__ parts_g,
+                                                          unsigned box_blocks, const T* __restrict__ xes, int N,
+                                                          int blocks_per_xseg, T* __restrict__ parts_p) {
     constexpr int G = 1 + D + D * D;
     __shared__ T red[2 * D][kBlock];
-    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
-    const int m = blk * kBlock + threadIdx.x;
     T lo[D], hi[D];
     for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
-    if (m < M) {
-        const size_t i = size_t(seg) * M + m;
-        const T* g = mixture + i * G;
-        double delta[D];
-        box_half_extent<T, D>(g, threshold, mode, delta);
-        for (int k = 0; k < D; ++k) {
-            box_lo[i * D + k] = T(double(g[1 + k]) - delta[k]);
-            box_hi[i * D + k] = T(double(g[1 + k]) + delta[k]);
-            lo[k] = g[1 + k] < lo[k] ? g[1 + k] : lo[k];          // comparisons as in bounds_kernel: NaN is skipped
-            hi[k] = g[1 + k] > hi[k] ? g[1 + k] : hi[k];
+    if (blockIdx.x < box_blocks) {
+        const int seg = blockIdx.x / blocks_per_mixture, blk = blockIdx.x - seg * blocks_per_mixture;
+        const int m = blk * kBlock + threadIdx.x;
+        if (m < M) {
+            const size_t i = size_t(seg) * M + m;
+            const T* g = mixture + i * G;
+            double delta[D];
+            box_half_extent<T, D>(g, threshold, mode, delta);
+            for (int k = 0; k < D; ++k) {
+                box_lo[i * D + k] = T(double(g[1 + k]) - delta[k]);
+                box_hi[i * D + k] = T(double(g[1 + k]) + delta[k]);
+                lo[k] = g[1 + k] < lo[k] ? g[1 + k] : lo[k];       // a NaN coordinate is skipped
+                hi[k] = g[1 + k] > hi[k] ? g[1 + k] : hi[k];
+            }
         }
+        const T v = block_bounds<T, D>(lo, hi, red);
+        if (threadIdx.x < 2 * D) parts_g[size_t(blockIdx.x) * 2 * D + threadIdx.x] = v;
+    } else {
+        const unsigned id = blockIdx.x - box_blocks;
+        const int seg = id / blocks_per_xseg, blk = id - seg * blocks_per_xseg;
+        const T* p = xes + size_t(seg) * N * D;
+        const int begin = blk * kBoundsChunk;
+        const int end = begin + kBoundsChunk < N ? begin + kBoundsChunk : N;
+        for (int i = begin + threadIdx.x; i < end; i += kBlock)
+            for (int d = 0; d < D; ++d) {
+                const T a = p[size_t(i) * D + d];
+                lo[d] = a < lo[d] ? a : lo[d];
+                hi[d] = a > hi[d] ? a : hi[d];
+            }
+        const T v = block_bounds<T, D>(lo, hi, red);
+        if (threadIdx.x < 2 * D) parts_p[size_t(id) * 2 * D + threadIdx.x] = v;
     }
-    const T v = block_bounds<T, D>(lo, hi, red);
-    if (threadIdx.x < 2 * D) parts[size_t(blockIdx.x) * 2 * D + threadIdx.x] = v;
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// bounds of a point set, Morton keys
+// Morton keys
 // ---------------------------------------------------------------------------------------------------------------
-
-// Partial bounds of `count` points per segment: workgroup (blk, seg) reduces `chunk` points to
-// parts[seg][blk] = (min_0..min_D-1, max_0..max_D-1); the Morton kernel combines the partial records.
-template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bounds_kernel(const T* __restrict__ pts, int stride, int offset, int count,
-                                                       int chunk, int blocks_per_seg, T* __restrict__ out) {
-    __shared__ T red[2 * D][kBlock];
-    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
-    const T* p = pts + size_t(seg) * count * stride + offset;
-    const int begin = blk * chunk;
-    const int end = begin + chunk < count ? begin + chunk : count;
-    T lo[D], hi[D];
-    for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
-    for (int i = begin + threadIdx.x; i < end; i += kBlock)
-        for (int d = 0; d < D; ++d) {
-            const T a = p[size_t(i) * stride + d];
-            lo[d] = a < lo[d] ? a : lo[d];
-            hi[d] = a > hi[d] ? a : hi[d];
-        }
-    const T v = block_bounds<T, D>(lo, hi, red);
-    if (threadIdx.x < 2 * D) out[size_t(blockIdx.x) * 2 * D + threadIdx.x] = v;
-}
 
 __device__ __forceinline__ uint32_t expand_bits3(uint32_t v) {
     v = (v * 0x00010001u) & 0xFF0000FFu;
@@ -335,19 +337,28 @@ __device__ __forceinline__ uint32_t morton30(const T* __restrict__ p, const T* _
     return code;
 }
 
-// Morton keys of the points of segment `seg` (workgroup (blk, seg), 256 points); every workgroup first combines
-// the segment's `n_parts` partial bounds
+// a set of points to be Morton-coded: the centres of the mixtures or the query points
+template <typename T> struct MortonJob {
+    const T* pts; int stride, offset, count, blocks_per_seg;      // workgroup (blk, seg) codes 256 points
+    const T* parts; int n_parts;                                   // partial bounds of every segment
+    uint32_t* keys; uint32_t* vals;
+    unsigned blocks;                                               // workgroups of this job in the launch
+};
+
+// Morton keys and index payload for two jobs in one launch (job b behind job a); every workgroup first combines
+// its segment's partial bounds
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void morton_kernel(const T* __restrict__ pts, int stride, int offset, int count,
-                                                       int blocks_per_seg, const T* __restrict__ parts, int n_parts,
-                                                       uint32_t* __restrict__ keys, uint32_t* __restrict__ vals) {
+__global__ __launch_bounds__(kBlock) void morton_kernel(MortonJob<T> a, MortonJob<T> b) {
     __shared__ T red[2 * D][kBlock];
     __shared__ T bounds[2 * D];
-    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    const bool first = blockIdx.x < a.blocks;
+    const MortonJob<T>& j = first ? a : b;
+    const unsigned id = first ? blockIdx.x : blockIdx.x - a.blocks;
+    const int seg = id / j.blocks_per_seg, blk = id - seg * j.blocks_per_seg;
     T lo[D], hi[D];
     for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
-    for (int i = threadIdx.x; i < n_parts; i += kBlock) {
-        const T* q = parts + (size_t(seg) * n_parts + i) * 2 * D;
+    for (int i = threadIdx.x; i < j.n_parts; i += kBlock) {
+        const T* q = j.parts + (size_t(seg) * j.n_parts + i) * 2 * D;
         for (int d = 0; d < D; ++d) {
             lo[d] = q[d] < lo[d] ? q[d] : lo[d];
             hi[d] = q[D + d] > hi[d] ? q[D + d] : hi[d];
@@ -357,55 +368,67 @@ __global__ __launch_bounds__(kBlock) void morton_kernel(const T* __restrict__ pt
     if (threadIdx.x < 2 * D) bounds[threadIdx.x] = v;
     __syncthreads();
     const int i = blk * kBlock + threadIdx.x;
-    if (i >= count) return;
-    const size_t at = size_t(seg) * count + i;
-    keys[at] = morton30<T, D>(pts + at * stride + offset, bounds);
-    vals[at] = uint32_t(i);
+    if (i >= j.count) return;
+    const size_t at = size_t(seg) * j.count + i;
+    j.keys[at] = morton30<T, D>(j.pts + at * j.stride + j.offset, bounds);
+    j.vals[at] = uint32_t(i);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
 // segmented LSD radix sort, 8 bits per pass, stable; segments of equal length `count`
 // ---------------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void radix_hist_kernel(const uint32_t* __restrict__ keys, int count, int chunk,
-                                                           int blocks_per_seg, int shift, uint32_t* __restrict__ hist) {
+// one pass over one set of segments
+struct SortJob {
+    const uint32_t* keys_in; const uint32_t* vals_in; uint32_t* keys_out; uint32_t* vals_out;
+    uint32_t* hist;                      // [segments][blocks_per_seg][256]
+    int count, items, blocks_per_seg, shift;
+    unsigned blocks;                     // workgroups of this job in the launch
+};
+
+// block histograms of the pass's digit, for two jobs in one launch (job b behind job a)
+__global__ __launch_bounds__(kBlock) void radix_hist_kernel(SortJob a, SortJob b) {
     __shared__ uint32_t h[256];
-    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    const bool first = blockIdx.x < a.blocks;
+    const SortJob& j = first ? a : b;
+    const unsigned id = first ? blockIdx.x : blockIdx.x - a.blocks;
+    const int seg = id / j.blocks_per_seg, blk = id - seg * j.blocks_per_seg;
     h[threadIdx.x] = 0;
     __syncthreads();
-    const uint32_t* k = keys + size_t(seg) * count;
+    const uint32_t* k = j.keys_in + size_t(seg) * j.count;
+    const int chunk = j.items * kBlock;
     const int begin = blk * chunk;
-    const int end = begin + chunk < count ? begin + chunk : count;
-    for (int i = begin + threadIdx.x; i < end; i += kBlock) atomicAdd(&h[(k[i] >> shift) & 255u], 1u);
+    const int end = begin + chunk < j.count ? begin + chunk : j.count;
+    for (int i = begin + threadIdx.x; i < end; i += kBlock) atomicAdd(&h[(k[i] >> j.shift) & 255u], 1u);
     __syncthreads();
-    hist[(size_t(seg) * blocks_per_seg + blk) * 256 + threadIdx.x] = h[threadIdx.x];
+    j.hist[size_t(id) * 256 + threadIdx.x] = h[threadIdx.x];
 }
 
-__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const uint32_t* __restrict__ keys_in,
-                                                              const uint32_t* __restrict__ vals_in,
-                                                              uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
-                                                              int count, int items, int blocks_per_seg, int shift,
-                                                              const uint32_t* __restrict__ hist) {
+__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJob b) {
     __shared__ uint32_t running[256];        // next output slot of every digit for this block
     __shared__ uint32_t wave_count[4][256];
-    const int seg = blockIdx.x / blocks_per_seg, blk = blockIdx.x - seg * blocks_per_seg;
+    const bool first = blockIdx.x < a.blocks;
+    const SortJob& j = first ? a : b;
+    const unsigned id = first ? blockIdx.x : blockIdx.x - a.blocks;
+    const int blocks_per_seg = j.blocks_per_seg, count = j.count, shift = j.shift;
+    const int seg = id / blocks_per_seg, blk = id - seg * blocks_per_seg;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     // thread d: keys of digit d in the whole segment and in the blocks before this one (at most kSortBlocksMax
     // counts per digit, so no separate scan pass is needed)
     uint32_t mine = 0, earlier = 0;
     {
-        const uint32_t* col = hist + size_t(seg) * blocks_per_seg * 256 + threadIdx.x;
-        int b = 0;
-        for (; b + 8 <= blocks_per_seg; b += 8) {           // eight independent loads in flight
+        const uint32_t* col = j.hist + size_t(seg) * blocks_per_seg * 256 + threadIdx.x;
+        int q0 = 0;
+        for (; q0 + 8 <= blocks_per_seg; q0 += 8) {         // eight independent loads in flight
             uint32_t c[8];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) c[q] = col[size_t(b + q) * 256];
+            for (int q = 0; q < 8; ++q) c[q] = col[size_t(q0 + q) * 256];
 #pragma unroll
-            for (int q = 0; q < 8; ++q) { mine += c[q]; earlier += b + q < blk ? c[q] : 0u; }
+            for (int q = 0; q < 8; ++q) { mine += c[q]; earlier += q0 + q < blk ? c[q] : 0u; }
         }
-        for (; b < blocks_per_seg; ++b) {
-            const uint32_t c = col[size_t(b) * 256];
+        for (; q0 < blocks_per_seg; ++q0) {
+            const uint32_t c = col[size_t(q0) * 256];
             mine += c;
-            earlier += b < blk ? c : 0u;
+            earlier += q0 < blk ? c : 0u;
         }
     }
     // exclusive scan of the segment's digit totals (Hillis-Steele on LDS) = first slot of every digit
@@ -422,18 +445,18 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const uint32_t* _
     running[threadIdx.x] += earlier - mine;
     __syncthreads();
     const size_t seg_off = size_t(seg) * count;
-    const int begin = blk * items * kBlock;
-    for (int round = 0; round < items; ++round) {
+    const int begin = blk * j.items * kBlock;
+    for (int round = 0; round < j.items; ++round) {
         const int i = begin + round * kBlock + threadIdx.x;
         const bool valid = i < count;
         uint32_t key = 0, val = 0, digit = 0;
-        if (valid) { key = keys_in[seg_off + i]; val = vals_in[seg_off + i]; digit = (key >> shift) & 255u; }
+        if (valid) { key = j.keys_in[seg_off + i]; val = j.vals_in[seg_off + i]; digit = (key >> shift) & 255u; }
         // lanes of this wavefront holding the same digit
         unsigned long long same = __ballot(valid);
 #pragma unroll
         for (int bit = 0; bit < 8; ++bit) {
-            const unsigned long long b = __ballot((digit >> bit) & 1u);
-            same &= ((digit >> bit) & 1u) ? b : ~b;
+            const unsigned long long m = __ballot((digit >> bit) & 1u);
+            same &= ((digit >> bit) & 1u) ? m : ~m;
         }
         const int rank = __popcll(same & ((1ull << lane) - 1ull));
         if (valid && rank == 0) wave_count[wave][digit] = uint32_t(__popcll(same));
@@ -442,8 +465,8 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(const uint32_t* _
             uint32_t slot = running[digit] + rank;
             for (int w = 0; w < wave; ++w) slot += wave_count[w][digit];
             if (slot < uint32_t(count)) {          // always true for a consistent histogram; keeps a bug from writing out of bounds
-                keys_out[seg_off + slot] = key;
-                vals_out[seg_off + slot] = val;
+                j.keys_out[seg_off + slot] = key;
+                j.vals_out[seg_off + slot] = val;
             }
         }
         __syncthreads();
@@ -1115,25 +1138,28 @@ __global__ void iota_segments_kernel(int* __restrict__ dst, int count, size_t to
 // ---------------------------------------------------------------------------------------------------------------
 static unsigned grid_for(size_t n) { return unsigned((n + kBlock - 1) / kBlock); }
 
-// sorts `segments` segments of `count` (key, value) pairs held in (ka, va) on the key bits
-// [first_bit, first_bit + 8 * passes), ping-ponging with (kb, vb); the last pass writes to (keys_out, vals_out)
-static void radix_sort(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* keys_out, uint32_t* vals_out,
-                       uint32_t* hist, int segments, int count, int first_bit, int passes, hipStream_t st) {
-    const int items = sort_items(size_t(count));
-    const int bps = int(sort_blocks(size_t(count)));
-    const dim3 grid(unsigned(size_t(segments) * bps));
-    int cur = 0;
-    for (int p = 0; p < passes; ++p) {
-        uint32_t* kin = cur ? kb : ka; uint32_t* vin = cur ? vb : va;
-        uint32_t* kout = cur ? ka : kb; uint32_t* vout = cur ? va : vb;
-        if (p == passes - 1) { kout = keys_out; vout = vals_out; }
-        const int shift = first_bit + 8 * p;
-        radix_hist_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, count, items * kBlock, bps, shift, hist);
-        radix_scatter_kernel<<<grid, dim3(kBlock), 0, st>>>(kin, vin, kout, vout, count, items, bps, shift, hist);
-        cur ^= 1;
-    }
+// Pass `pass` (8 key bits from `first_bit + 8 * pass` on) of the stable LSD radix sort of `segments` segments of
+// `count` (key, value) pairs: input (ka, va) on even passes and (kb, vb) on odd ones, output the other pair, the
+// last pass writes to (keys_out, vals_out).  A job without workgroups stands for "nothing to do in this pass".
+static SortJob sort_job(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* keys_out, uint32_t* vals_out,
+                        uint32_t* hist, size_t segments, int count, int first_bit, int passes, int pass) {
+    SortJob j = {};
+    if (segments == 0 || count == 0 || pass >= passes) return j;
+    const bool odd = pass & 1;
+    j.keys_in = odd ? kb : ka; j.vals_in = odd ? vb : va;
+    j.keys_out = odd ? ka : kb; j.vals_out = odd ? va : vb;
+    if (pass == passes - 1) { j.keys_out = keys_out; j.vals_out = vals_out; }
+    j.hist = hist;
+    j.count = count;
+    j.items = sort_items(size_t(count));
+    j.blocks_per_seg = int(sort_blocks(size_t(count)));
+    j.shift = first_bit + 8 * pass;
+    j.blocks = unsigned(segments * size_t(j.blocks_per_seg));
+    return j;
 }
 
+// Build of the trees and of the Morton order of the query points.  The two chains (boxes -> keys -> sort of the
+// leaves; bounds -> keys -> sort of the points) do not depend on each other, so each launch serves both.
 template <typename T, int D>
 static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shape& s, const gmc_bvh_config& cfg,
                        hipStream_t st) {
@@ -1147,18 +1173,39 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     int* leaf_comp = (int*)(bvh + lay.leaf_comp); long long* enc_box = (long long*)(bvh + lay.enc_box);
     uint32_t* ka = (uint32_t*)(bvh + lay.keys_a); uint32_t* kb = (uint32_t*)(bvh + lay.keys_b);
     uint32_t* va = (uint32_t*)(bvh + lay.vals_a); uint32_t* vb = (uint32_t*)(bvh + lay.vals_b);
-    uint32_t* hist = (uint32_t*)(bvh + lay.hist);
-    T* parts = (T*)(bvh + lay.part_bounds);
+    uint32_t* pka = (uint32_t*)(bvh + lay.pkeys_a); uint32_t* pkb = (uint32_t*)(bvh + lay.pkeys_b);
+    uint32_t* pva = (uint32_t*)(bvh + lay.pvals_a); uint32_t* pvb = (uint32_t*)(bvh + lay.pvals_b);
+    T* parts_g = (T*)(bvh + lay.parts_g); T* parts_p = (T*)(bvh + lay.parts_p);
     T* child_box = (T*)(bvh + lay.child_box);
-    if (BL > 0 && M > 0) {
+    uint32_t* g_keys = (uint32_t*)(bvh + lay.g_keys);
+    uint32_t* g_order = (uint32_t*)leaf_comp;                // the sorted payload IS the component id of every leaf
+    int* p_order = (int*)(bvh + lay.p_order);
+    const bool have_g = BL > 0 && M > 0, have_p = XL > 0 && N > 0;
+    const bool sort_p = have_p && xes != nullptr;
+    const int bpm = (M + kBlock - 1) / kBlock;               // workgroups per mixture (boxes, keys)
+    const int nbp = (N + kBoundsChunk - 1) / kBoundsChunk;   // partial bounds per point segment
+    const int bpx = (N + kBlock - 1) / kBlock;               // workgroups per point segment (keys)
+    const unsigned box_blocks = have_g ? unsigned(BL * bpm) : 0u, bound_blocks = sort_p ? unsigned(XL * nbp) : 0u;
+    if (box_blocks + bound_blocks > 0)
+        bvh_boxes_kernel<T, D><<<dim3(box_blocks + bound_blocks), dim3(kBlock), 0, st>>>(
+            mixture, box_lo, box_hi, M, bpm, double(cfg.aabb_threshold), cfg.aabb_mode, parts_g, box_blocks, xes, N, nbp,
+            parts_p);
+    MortonJob<T> mg = {}, mp = {};
+    if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm)};
+    if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx)};
+    if (mg.blocks + mp.blocks > 0) morton_kernel<T, D><<<dim3(mg.blocks + mp.blocks), dim3(kBlock), 0, st>>>(mg, mp);
+    // leaves: all 30 key bits; points: 16 Morton bits (65536 cells) are enough to make 64 consecutive points
+    // neighbours, and their sorted keys are not needed afterwards (they land in a spare buffer)
+    for (int pass = 0; pass < 4; ++pass) {
+        const SortJob jg = sort_job(ka, va, kb, vb, g_keys, g_order, (uint32_t*)(bvh + lay.hist_g), have_g ? BL : 0, M, 0, 4, pass);
+        const SortJob jp = sort_job(pka, pva, pkb, pvb, pka, (uint32_t*)p_order, (uint32_t*)(bvh + lay.hist_p),
+                                    sort_p ? XL : 0, N, 14, 2, pass);
+        if (jg.blocks + jp.blocks == 0) continue;
+        radix_hist_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
+        radix_scatter_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
+    }
+    if (have_g) {
         const size_t n = BL * M;
-        const int bpm = (M + kBlock - 1) / kBlock;          // workgroups per mixture
-        bvh_boxes_kernel<T, D><<<dim3(unsigned(BL * bpm)), dim3(kBlock), 0, st>>>(
-            mixture, box_lo, box_hi, M, bpm, double(cfg.aabb_threshold), cfg.aabb_mode, parts);
-        morton_kernel<T, D><<<dim3(unsigned(BL * bpm)), dim3(kBlock), 0, st>>>(mixture, G, 1, M, bpm, parts, bpm, ka, va);
-        uint32_t* g_keys = (uint32_t*)(bvh + lay.g_keys);
-        uint32_t* g_order = (uint32_t*)leaf_comp;            // the sorted payload IS the component id of every leaf
-        radix_sort(ka, va, kb, vb, g_keys, g_order, hist, int(BL), M, 0, 4, st);
         bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, g_keys,
                                                                            node_box, leaf_rec, enc_box, children, parent, M, n);
         if (M > 1) {
@@ -1167,20 +1214,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
             bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(children, enc_box, node_box, child_box, M, ni);
         }
     }
-    if (XL > 0 && N > 0) {
-        int* p_order = (int*)(bvh + lay.p_order);
-        const size_t n = XL * N;
-        if (xes) {
-            const int nb = (N + kBoundsChunk - 1) / kBoundsChunk, bpx = (N + kBlock - 1) / kBlock;
-            bounds_kernel<T, D><<<dim3(unsigned(XL * nb)), dim3(kBlock), 0, st>>>(xes, D, 0, N, kBoundsChunk, nb, parts);
-            morton_kernel<T, D><<<dim3(unsigned(XL * bpx)), dim3(kBlock), 0, st>>>(xes, D, 0, N, bpx, parts, nb, ka, va);
-            // 16 Morton bits (65536 cells) are enough to make 64 consecutive points neighbours
-            // the sorted keys are not needed afterwards: they land in the spare key buffer
-            radix_sort(ka, va, kb, vb, ka, (uint32_t*)p_order, hist, int(XL), N, 14, 2, st);
-        } else {
-            iota_segments_kernel<<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(p_order, N, n);
-        }
-    }
+    if (have_p && !sort_p) iota_segments_kernel<<<dim3(grid_for(XL * N)), dim3(kBlock), 0, st>>>(p_order, N, XL * N);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
