@@ -32,7 +32,10 @@ PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}     # MI355X vector peaks
 VALU_NOTE = ("compute-bound against the FP32 peak of 157.3 TFLOP/s (matrix = packed vector rate); the kernels issue "
              "unpacked FP32 vector instructions (measured issue rate: one wave64 FMA per 2.3 cycles and SIMD = 137 TFLOP/s), the float32 forward kernel takes y = u x - u b "
              "from the bf16 matrix cores")
-MEASURED_TRAFFIC_BYTES = {"C4": 157960 * 1024 * 2.0 + 524288 * 1024 * 1.0}
+MEASURED_TRAFFIC_BYTES = {"C4": 157960 * 1024 * 2.0 + 524288 * 1024 * 1.0,
+                          # LBVH traversal kernels of C5 (aabb_mode "reference"): backward, forward
+                          "C5": 32591.5 * 1024 * 2.0 + 34124.9 * 1024 * 1.0,
+                          "C5_fwd": 21314.8 * 1024 * 2.0 + 3202.6 * 1024 * 1.0}
 
 
 def cpu_baseline(name: str, seconds_budget: float = 20.0):
@@ -126,11 +129,16 @@ def bench_bvh(args):
         "evaluated_fraction_of_dense": hits / wl.pairs,
         "roofline": {"kernel": "bvh_traverse_kernel (backward mode; event pair also holds its zero-fill and epilogue)",
                      "bound": "hbm", "achieved": bytes_bwd / (bwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
-                     "frac": bytes_bwd / (bwd_ms * 1e-3) / 8e12, "traffic": None, "launch_ms": bwd_ms,
-                     "algorithmic_bytes": bytes_bwd},
+                     "frac": bytes_bwd / (bwd_ms * 1e-3) / 8e12,
+                     "traffic": MEASURED_TRAFFIC_BYTES["C5"] if args.aabb_mode == "reference" else None,
+                     "launch_ms": bwd_ms, "algorithmic_bytes": bytes_bwd,
+                     "bound_detail": "latency-bound: dependent tree-node fetches and double-precision leaf "
+                                     "evaluation; the tree (about 4 MB) is fetched once per XCD (8 L2 caches)"},
         "roofline_fwd": {"kernel": "bvh_traverse_kernel (forward mode)", "bound": "hbm",
                          "achieved": bytes_fwd / (fwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
-                         "frac": bytes_fwd / (fwd_ms * 1e-3) / 8e12, "launch_ms": fwd_ms, "algorithmic_bytes": bytes_fwd},
+                         "frac": bytes_fwd / (fwd_ms * 1e-3) / 8e12,
+                         "traffic": MEASURED_TRAFFIC_BYTES["C5_fwd"] if args.aabb_mode == "reference" else None,
+                         "launch_ms": fwd_ms, "algorithmic_bytes": bytes_fwd},
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_bvh(args.aabb_mode)

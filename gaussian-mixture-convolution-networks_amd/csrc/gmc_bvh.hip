@@ -610,6 +610,7 @@ __global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int* __restrict
     int node = parent[nbase + (M - 1) + leaf];
     // the radix tree over 64-bit keys is at most 64 levels deep; the bound also ends a walk on a malformed chain
     for (int level = 0; node >= 0 && node < M - 1 && level < 128; ++level) {
+        const int up = parent[nbase + node];        // fetched alongside the atomics: one round trip per level
         bool grew = false;
         long long* e = enc + size_t(node) * 2 * D;
         for (int d = 0; d < D; ++d) {
@@ -617,7 +618,7 @@ __global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int* __restrict
             grew |= hi[d] > atomicMax(&e[D + d], hi[d]);
         }
         if (!grew) break;
-        node = parent[nbase + node];
+        node = up;
     }
 }
 
