@@ -156,6 +156,33 @@ def test_several_point_groups_per_workgroup(dtype):
     _check_culled(mix, xes, gout, dtype, "tight", tag="wide, several groups")
 
 
+def test_culled_random_shapes():
+    """differential run of the culled path over random shapes (one to four point groups per workgroup, ragged and
+    empty trailing groups, broadcast points, identical Gaussians, narrow and wide boxes) against the masked sum"""
+    rng = np.random.default_rng(777)
+    for case in range(28):
+        D = 2 + case % 2
+        dtype = torch.float64 if case % 4 < 2 else torch.float32
+        kind = case % 7
+        if kind == 0:
+            B, L, M, N = int(rng.integers(20, 60)), int(rng.integers(4, 9)), int(rng.integers(1, 40)), int(rng.integers(1, 700))
+        elif kind == 1:
+            B, L, M, N = 1, 1, int(rng.integers(1, 900)), int(rng.integers(20000, 42000))
+        elif kind == 2:
+            B, L, M, N = int(rng.integers(1, 4)), int(rng.integers(1, 4)), int(rng.integers(200, 1500)), int(rng.integers(1, 200))
+        else:
+            B, L, M, N = int(rng.integers(1, 9)), int(rng.integers(1, 9)), int(rng.integers(1, 120)), int(rng.integers(1, 9000))
+        while B * L * M * N > 2.5e7:
+            N = max(1, N // 2)
+        cov = float(rng.choice([0.02, 0.3, 3.0]))
+        mix, xes, gout = _case(B, L, M, N, D, 9000 + case, broadcast=(case % 5 == 3), spread=float(rng.choice([1.0, 4.0])),
+                               cov_radius=cov)
+        if case % 6 == 5 and M > 3:
+            mix[:, :, 1:M // 2] = mix[:, :, :1]          # identical Gaussians: equal Morton keys and boxes
+        _check_culled(mix, xes, gout, dtype, "tight" if case % 3 else "reference",
+                      tag=f"case {case}: B{B} L{L} M{M} N{N} D{D} cov {cov} {dtype}")
+
+
 def test_points_outside_every_box_and_need_flags():
     mix, xes, gout = _case(1, 2, 40, 64, 3, seed=400)
     far = xes + 1000.0
