@@ -750,9 +750,11 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     __shared__ int pids[kGroupsMax][kWave];                 // index of every point, -1 beyond the end
     __shared__ T pts[kGroupsMax][D + 1][kWave];             // coordinates and upstream gradient of every point
     __shared__ T gbox[kGroupsMax][2 * D];                   // bounding box of every group's points
-    __shared__ T result[kGroupsMax][kVals][kWave];
+    // results per point, in double: the forward sums are added wavefront by wavefront (deterministic), dL/dx with
+    // LDS atomics (cheap for doubles on distinct words, unlike floats)
+    __shared__ double result[kGroupsMax][kVals][kWave];
     // per wavefront: the staged leaf records of a batch; between two groups its partial results per point
-    static_assert(kStageBatch * LS >= kVals * kWave, "staging area too small for the partial results");
+    static_assert(kStageBatch * LS >= kWave, "staging area too small for the partial results");
     __shared__ __attribute__((aligned(16))) T staged_mem[kTravWaves][kStageBatch * LS];
     // double in both precisions: LDS atomic adds of doubles on distinct addresses cost a few cycles per
     // instruction, those of floats are serialised lane by lane
@@ -800,7 +802,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
         }
         sp = (any && M > 1) ? 1 : 0;
     }
-    for (int i = threadIdx.x; i < kGroupsMax * kVals * kWave; i += kTravBlock) (&result[0][0][0])[i] = T(0);
+    for (int i = threadIdx.x; i < kGroupsMax * kVals * kWave; i += kTravBlock) (&result[0][0][0])[i] = 0.0;
 
     const T* cboxes = child_box + size_t(bl) * (M - 1) * 4 * D;
     const int2* kids = children + size_t(bl) * (M - 1);
@@ -958,9 +960,11 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             }
             wave_lds_fence();
         }
-        if (MODE == 0 || NEED_GX) {
+        if (MODE == 0) {
+            staged[lane] = acc;                         // the staging area is idle now
+        } else if (NEED_GX) {
 #pragma unroll
-            for (int d = 0; d < kVals; ++d) staged[d * kWave + lane] = MODE == 0 ? acc : gx[d];   // staging area is idle now
+            for (int d = 0; d < D; ++d) atomic_add(&result[gi][d][lane], double(gx[d]));
         }
     };
 
@@ -1021,14 +1025,18 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             left_on_stack |= state[gi][1] > 0;
             if (n_leaf == 0) continue;                                  // uniform over the workgroup
             evaluate_share(gi);
-            __syncthreads();
-            if ((MODE == 0 || NEED_GX) && wave < kVals) {
-                T v = T(0);
+            if (MODE == 0) {
+                // forward: the wavefronts' partial sums are added in a fixed order (the backward pass has added
+                // its dL/dx with atomics and goes on to the next group without waiting for the other wavefronts)
+                __syncthreads();
+                if (wave == 0) {
+                    T v = T(0);
 #pragma unroll
-                for (int w = 0; w < kTravWaves; ++w) v += staged_mem[w][wave * kWave + lane];
-                result[gi][wave][lane] += v;
+                    for (int w = 0; w < kTravWaves; ++w) v += staged_mem[w][lane];
+                    result[gi][0][lane] += double(v);
+                }
+                __syncthreads();
             }
-            __syncthreads();
         }
         if (!left_on_stack) break;
         __syncthreads();                                                // every wavefront has read this round's state
@@ -1041,13 +1049,13 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     const int pid = pids[wave][lane];
     if (pid < 0) return;
     if (MODE == 0) {
-        out[size_t(bl) * N + pid] = result[wave][0][lane];
+        out[size_t(bl) * N + pid] = T(result[wave][0][lane]);
     } else if (NEED_GX) {
         const T g = pts[wave][D][lane];
         T* dst = grad_xes + (xseg * N + pid) * D;
 #pragma unroll
         for (int d = 0; d < D; ++d) {
-            const T v = -g * result[wave][d][lane];
+            const T v = -g * T(result[wave][d][lane]);
             if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
         }
     }
