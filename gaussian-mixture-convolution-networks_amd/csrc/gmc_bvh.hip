@@ -193,15 +193,20 @@ __device__ inline bool ref_symeig3(const double a[3][3], double lam[3], double v
 
 // half extents of the cutoff box of one Gaussian (record g: weight, position, inverse covariance)
 template <typename T, int D>
-__device__ inline void box_half_extent(const T* __restrict__ g, double threshold, int mode, double* delta) {
+__device__ inline void box_half_extent(const T* __restrict__ g, double threshold, int mode, bool covariance_form,
+                                       double* delta) {
     const double w = fabs(double(g[0]));
     double s2 = -2.0 * log(threshold / w);
     s2 = fmax(s2, kSqFloor);
     const double s = sqrt(s2);
     const T* c = g + 1 + D;
     double sigma[D][D];
-    // the reference inverts the stored matrix read column-major, i.e. C^T (util/glm.h:108-128)
-    if constexpr (D == 2) {
+    // the reference inverts the stored matrix read column-major, i.e. C^T (util/glm.h:108-128); a record in
+    // covariance form holds S with C = (S^-1)^T (src/gmc/mixture.py:149), so that inverse is S itself
+    if (covariance_form) {
+        for (int i = 0; i < D; ++i)
+            for (int j = 0; j < D; ++j) sigma[i][j] = double(c[i * D + j]);
+    } else if constexpr (D == 2) {
         const double m00 = c[0], m01 = c[2], m10 = c[1], m11 = c[3];
         const double det = m00 * m11 - m01 * m10;
         sigma[0][0] = m11 / det; sigma[0][1] = -m01 / det; sigma[1][0] = -m10 / det; sigma[1][1] = m00 / det;
@@ -269,8 +274,8 @@ __device__ __forceinline__ T block_bounds(const T (&lo)[D], const T (&hi)[D], T 
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
                                                           T* __restrict__ box_hi, int M, int blocks_per_mixture,
-                                                          double threshold, int mode, T* __restrict__ parts_g,
-                                                          unsigned box_blocks, const T* __restrict__ xes, int N,
+                                                          double threshold, int mode, bool covariance_form,
+                                                          T* __restrict__ parts_g, unsigned box_blocks, const T* __restrict__ xes, int N,
                                                           int blocks_per_xseg, T* __restrict__ parts_p) {
     constexpr int G = 1 + D + D * D;
     __shared__ T red[2 * D][kBlock];
@@ -283,7 +288,7 @@ __global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__
             const size_t i = size_t(seg) * M + m;
             const T* g = mixture + i * G;
             double delta[D];
-            box_half_extent<T, D>(g, threshold, mode, delta);
+            box_half_extent<T, D>(g, threshold, mode, covariance_form, delta);
             for (int k = 0; k < D; ++k) {
                 box_lo[i * D + k] = T(double(g[1 + k]) - delta[k]);
                 box_hi[i * D + k] = T(double(g[1 + k]) + delta[k]);
@@ -545,7 +550,7 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
                                                            const uint32_t* __restrict__ keys, T* __restrict__ node_box,
                                                            T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
                                                            int2* __restrict__ children, int* __restrict__ parent, int M,
-                                                           size_t total) {
+                                                           size_t total, bool covariance_form) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
     const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
@@ -570,15 +575,17 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
     T* r = leaf_rec + i * RS;
     for (int d = 0; d < D; ++d) { r[d] = box_lo[gi * D + d]; r[D + d] = box_hi[gi * D + d]; }
     r += 2 * D;
-    const T* c = g + 1 + D;
+    double cm[D][D];                                  // inverse covariance as evaluate_inversed takes it
+    load_inverse_covariance<T, D>(g + 1 + D, covariance_form, cm);
     for (int d = 0; d < D; ++d) r[d] = g[1 + d];
     if constexpr (D == 2) {
-        const double det = double(c[0]) * double(c[3]) - double(c[1]) * double(c[2]);
-        r[2] = c[0]; r[3] = T(0.5 * (double(c[1]) + double(c[2]))); r[4] = c[3];
+        const double det = cm[0][0] * cm[1][1] - cm[0][1] * cm[1][0];
+        r[2] = T(cm[0][0]); r[3] = T(0.5 * (cm[0][1] + cm[1][0])); r[4] = T(cm[1][1]);
         r[5] = T(double(g[0]) * Kappa<2>::v * sqrt(det));
         reinterpret_cast<int*>(r + 6)[0] = comp;
     } else {
-        const double c00 = c[0], c01 = c[1], c02 = c[2], c10 = c[3], c11 = c[4], c12 = c[5], c20 = c[6], c21 = c[7], c22 = c[8];
+        const double c00 = cm[0][0], c01 = cm[0][1], c02 = cm[0][2], c10 = cm[1][0], c11 = cm[1][1], c12 = cm[1][2],
+                     c20 = cm[2][0], c21 = cm[2][1], c22 = cm[2][2];
         const double det = c00 * (c11 * c22 - c12 * c21) - c01 * (c10 * c22 - c12 * c20) + c02 * (c10 * c21 - c11 * c20);
         r[3] = T(c00); r[4] = T(0.5 * (c01 + c10)); r[5] = T(0.5 * (c02 + c20));
         r[6] = T(c11); r[7] = T(0.5 * (c12 + c21)); r[8] = T(c22);
@@ -1061,10 +1068,14 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     }
 }
 
-// (R0, sum r t, sum r t t^T) -> (dw, db, dC); see the dense epilogue for the formulas (here y = t, u = identity)
+// (R0, sum r t, sum r t t^T) -> (dw, db, dC); see the dense epilogue for the formulas (here y = t, u = identity).
+// covariance_form: the record holds S with C = (S^-1)^T; the matrix gradient is carried on to S as
+// MatrixInverse.backward does (src/gmc/cpp/extensions/math/matrix_inverse.py:30-33: -S^-1 g S^-1 without transposes,
+// which is the derivative for symmetric matrices only): dS = -(C dC C)^T.
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __restrict__ mixture, const T* __restrict__ sums,
-                                                                 T* __restrict__ grad_mixture, size_t n) {
+                                                                 T* __restrict__ grad_mixture, size_t n,
+                                                                 bool covariance_form) {
     constexpr int G = 1 + D + D * D;
     constexpr int NR = BvhSums<D>::k;
     const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
@@ -1074,8 +1085,7 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
     T* o = grad_mixture + i * G;
     const double w = double(g[0]);
     double c[D][D];
-    for (int r = 0; r < D; ++r)
-        for (int q = 0; q < D; ++q) c[r][q] = double(g[1 + D + r * D + q]);
+    load_inverse_covariance<T, D>(g + 1 + D, covariance_form, c);
     double det;
     if constexpr (D == 2) det = c[0][0] * c[1][1] - c[0][1] * c[1][0];
     else det = c[0][0] * (c[1][1] * c[2][2] - c[1][2] * c[2][1]) - c[0][1] * (c[1][0] * c[2][2] - c[1][2] * c[2][0]) +
@@ -1096,6 +1106,7 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
     for (int a = 0; a < D; ++a)
         for (int q = a; q < D; ++q) { s2[a][q] = double(rs[k]); s2[q][a] = double(rs[k]); ++k; }
     const double kd = w * Kappa<D>::v * R0 / (2.0 * root);
+    double gc[D][D];
     for (int r = 0; r < D; ++r)
         for (int q = 0; q < D; ++q) {
             double cof;
@@ -1105,7 +1116,25 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
                 const int r1i = r == 0 ? 1 : 0, r2i = r == 2 ? 1 : 2, q1 = q == 0 ? 1 : 0, q2 = q == 2 ? 1 : 2;
                 cof = (((r + q) & 1) ? -1.0 : 1.0) * (c[r1i][q1] * c[r2i][q2] - c[r1i][q2] * c[r2i][q1]);
             }
-            o[1 + D + r * D + q] = T(-0.5 * w * norm * s2[r][q] + cof * kd);
+            gc[r][q] = -0.5 * w * norm * s2[r][q] + cof * kd;
+        }
+    if (!covariance_form) {
+        for (int r = 0; r < D; ++r)
+            for (int q = 0; q < D; ++q) o[1 + D + r * D + q] = T(gc[r][q]);
+        return;
+    }
+    double x1[D][D];
+    for (int r = 0; r < D; ++r)
+        for (int q = 0; q < D; ++q) {
+            double acc = 0.0;
+            for (int t = 0; t < D; ++t) acc += c[r][t] * gc[t][q];
+            x1[r][q] = acc;
+        }
+    for (int r = 0; r < D; ++r)
+        for (int q = 0; q < D; ++q) {
+            double acc = 0.0;
+            for (int t = 0; t < D; ++t) acc += x1[r][t] * c[t][q];
+            o[1 + D + q * D + r] = T(-acc);
         }
 }
 
@@ -1197,8 +1226,8 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     const unsigned box_blocks = have_g ? unsigned(BL * bpm) : 0u, bound_blocks = sort_p ? unsigned(XL * nbp) : 0u;
     if (box_blocks + bound_blocks > 0)
         bvh_boxes_kernel<T, D><<<dim3(box_blocks + bound_blocks), dim3(kBlock), 0, st>>>(
-            mixture, box_lo, box_hi, M, bpm, double(cfg.aabb_threshold), cfg.aabb_mode, parts_g, box_blocks, xes, N, nbp,
-            parts_p);
+            mixture, box_lo, box_hi, M, bpm, double(cfg.aabb_threshold), cfg.aabb_mode, cfg.covariance_form != 0, parts_g,
+            box_blocks, xes, N, nbp, parts_p);
     MortonJob<T> mg = {}, mp = {};
     if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm)};
     if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx)};
@@ -1216,7 +1245,8 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     if (have_g) {
         const size_t n = BL * M;
         bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, g_keys,
-                                                                           node_box, leaf_rec, enc_box, children, parent, M, n);
+                                                                           node_box, leaf_rec, enc_box, children, parent, M, n,
+                                                                           cfg.covariance_form != 0);
         if (M > 1) {
             const size_t ni = BL * (M - 1);
             bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(parent, node_box, enc_box, M, n);
@@ -1258,7 +1288,7 @@ static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, 
 
 template <typename T, int D>
 static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, const char* bvh, T* grad_mixture, T* grad_xes,
-                     T* sums, const gmc_shape& s, bool gm, bool gx, hipStream_t st) {
+                     T* sums, const gmc_shape& s, bool gm, bool gx, bool covariance_form, hipStream_t st) {
     constexpr int G = 1 + D + D * D;
     constexpr int NR = BvhSums<D>::k;
     const BvhLayout lay = bvh_layout(s);
@@ -1287,7 +1317,9 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, const ch
     else if (gm) GMC_TRAV(true, false);
     else if (gx) GMC_TRAV(false, true);
 #undef GMC_TRAV
-    if (gm) bvh_bwd_epilogue_kernel<T, D><<<dim3(grid_for(n_g)), dim3(kBlock), 0, st>>>(mixture, sums, grad_mixture, n_g);
+    if (gm)
+        bvh_bwd_epilogue_kernel<T, D><<<dim3(grid_for(n_g)), dim3(kBlock), 0, st>>>(mixture, sums, grad_mixture, n_g,
+                                                                                    covariance_form);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
@@ -1383,9 +1415,10 @@ int gmc_eval_bvh_fwd(const void* mixture, const void* xes, const void* bvh, void
 #undef ARGS
 }
 
-int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh, void* grad_mixture,
-                     void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
-                     int need_grad_mixture, int need_grad_xes, void* stream) {
+static int eval_bvh_bwd_impl(const void* grad_out, const void* mixture, const void* xes, const void* bvh,
+                             void* grad_mixture, void* grad_xes, void* workspace, size_t workspace_bytes,
+                             const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, bool covariance_form,
+                             void* stream) {
     const int rc = check_bvh_shape(shape);
     if (rc != GMC_OK) return rc;
     const bool gm = need_grad_mixture != 0, gx = need_grad_xes != 0;
@@ -1400,10 +1433,24 @@ int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes,
         if (workspace_bytes < need) return GMC_E_WORKSPACE;
         if (!workspace) return GMC_E_NULL;
     }
-#define ARGS(T) (const T*)grad_out, (const T*)mixture, (const T*)xes, (const char*)bvh, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, *shape, gm, gx, (hipStream_t)stream
+#define ARGS(T) (const T*)grad_out, (const T*)mixture, (const T*)xes, (const char*)bvh, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, *shape, gm, gx, covariance_form, (hipStream_t)stream
     if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_bwd_t<float, 2>(ARGS(float)) : gmc::bvh_bwd_t<float, 3>(ARGS(float));
     return shape->D == 2 ? gmc::bvh_bwd_t<double, 2>(ARGS(double)) : gmc::bvh_bwd_t<double, 3>(ARGS(double));
 #undef ARGS
+}
+
+int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh, void* grad_mixture,
+                     void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
+                     int need_grad_mixture, int need_grad_xes, void* stream) {
+    return eval_bvh_bwd_impl(grad_out, mixture, xes, bvh, grad_mixture, grad_xes, workspace, workspace_bytes, shape,
+                             need_grad_mixture, need_grad_xes, false, stream);
+}
+
+int gmc_eval_bvh_cov_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh, void* grad_mixture,
+                         void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
+                         int need_grad_mixture, int need_grad_xes, void* stream) {
+    return eval_bvh_bwd_impl(grad_out, mixture, xes, bvh, grad_mixture, grad_xes, workspace, workspace_bytes, shape,
+                             need_grad_mixture, need_grad_xes, true, stream);
 }
 
 }  // extern "C"

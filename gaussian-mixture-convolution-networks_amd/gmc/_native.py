@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class Shape(ctypes.Structure):
@@ -28,7 +28,7 @@ class ConvShape(ctypes.Structure):
 
 
 class BvhConfigC(ctypes.Structure):
-    _fields_ = [("aabb_mode", ctypes.c_int), ("aabb_threshold", ctypes.c_float)]
+    _fields_ = [("aabb_mode", ctypes.c_int), ("aabb_threshold", ctypes.c_float), ("covariance_form", ctypes.c_int)]
 
 
 def build(verbose: bool = False) -> str:
@@ -76,6 +76,7 @@ def lib() -> ctypes.CDLL:
         l.gmc_bvh_export_nodes.argtypes = [vp, vp, vp, shp, vp]
         l.gmc_eval_bvh_fwd.argtypes = [vp, vp, vp, vp, shp, vp]
         l.gmc_eval_bvh_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
+        l.gmc_eval_bvh_cov_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
     if l.gmc_abi_version() != ABI_VERSION:
         raise RuntimeError("libgmc_hip.so was built from a different include/gmc_hip.h; rebuild it")
     _lib = l
@@ -214,21 +215,23 @@ def eval_componentwise_bwd(grad_output, mixture, xes, need_mixture: bool, need_x
 _AABB_MODES = {"reference": GMC_AABB_REFERENCE, "tight": GMC_AABB_TIGHT}
 
 
-def _bvh_config(aabb_threshold: float, aabb_mode: str) -> BvhConfigC:
+def _bvh_config(aabb_threshold: float, aabb_mode: str, covariance_form: bool = False) -> BvhConfigC:
     if aabb_mode not in _AABB_MODES:
         raise RuntimeError(f"unknown aabb_mode {aabb_mode!r}; expected 'reference' or 'tight'")
     if not aabb_threshold > 0:
         raise RuntimeError("aabb_threshold must be positive")
-    return BvhConfigC(_AABB_MODES[aabb_mode], float(aabb_threshold))
+    return BvhConfigC(_AABB_MODES[aabb_mode], float(aabb_threshold), int(bool(covariance_form)))
 
 
 class Bvh:
-    """One LBVH per (batch, layer) mixture plus the Morton order of the query points, as an opaque device blob."""
+    """One LBVH per (batch, layer) mixture plus the Morton order of the query points, as an opaque device blob.
+    covariance_form: the mixture holds covariances (as gm.evaluate takes them) instead of inverse covariances."""
 
     def __init__(self, mixture: torch.Tensor, xes: torch.Tensor, aabb_threshold: float = 0.001,
-                 aabb_mode: str = "reference"):
+                 aabb_mode: str = "reference", covariance_form: bool = False):
         self.shape = check_input(mixture, xes)
-        cfg = _bvh_config(aabb_threshold, aabb_mode)
+        self.covariance_form = bool(covariance_form)
+        cfg = _bvh_config(aabb_threshold, aabb_mode, covariance_form)
         dev = mixture.device
         with torch.cuda.device(dev):
             nbytes = lib().gmc_bvh_bytes(ctypes.byref(self.shape))
@@ -282,9 +285,9 @@ def eval_bvh_bwd(grad_output, mixture, xes, bvh: Bvh, need_mixture: bool, need_x
     with torch.cuda.device(dev):
         ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
         ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
-        check(lib().gmc_eval_bvh_bwd(_p(grad_output), _p(mixture), _p(xes), _p(bvh.blob), _p(grad_mixture), _p(grad_xes),
-                                     _p(ws), ws_bytes, ctypes.byref(shape), int(need_mixture), int(need_xes),
-                                     _stream(dev)))
+        fn = lib().gmc_eval_bvh_cov_bwd if bvh.covariance_form else lib().gmc_eval_bvh_bwd
+        check(fn(_p(grad_output), _p(mixture), _p(xes), _p(bvh.blob), _p(grad_mixture), _p(grad_xes), _p(ws), ws_bytes,
+                 ctypes.byref(shape), int(need_mixture), int(need_xes), _stream(dev)))
     return grad_mixture, grad_xes
 
 

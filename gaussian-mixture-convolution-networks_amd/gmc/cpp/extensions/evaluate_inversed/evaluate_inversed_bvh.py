@@ -11,9 +11,9 @@ from .... import _native
 
 class EvaluateInversedBvh(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, mixture: torch.Tensor, xes: torch.Tensor, config):
+    def forward(ctx, mixture: torch.Tensor, xes: torch.Tensor, config, covariance_form: bool = False):
         mixture, xes = mixture.contiguous(), xes.contiguous()
-        bvh = _native.Bvh(mixture, xes, config.aabb_threshold, config.aabb_mode)
+        bvh = _native.Bvh(mixture, xes, config.aabb_threshold, config.aabb_mode, covariance_form)
         values = _native.eval_bvh_fwd(mixture, xes, bvh)
         ctx.save_for_backward(mixture, xes)
         ctx.bvh = bvh
@@ -26,7 +26,15 @@ class EvaluateInversedBvh(torch.autograd.Function):
         want_mixture, want_xes = ctx.needs_input_grad[:2]
         grad_mixture, grad_xes = _native.eval_bvh_bwd(grad_output.contiguous(), mixture, xes, ctx.bvh, want_mixture,
                                                       want_xes)
-        return (grad_mixture if want_mixture else None), (grad_xes if want_xes else None), None
+        return (grad_mixture if want_mixture else None), (grad_xes if want_xes else None), None, None
 
 
-apply = EvaluateInversedBvh.apply
+def apply(mixture: torch.Tensor, xes: torch.Tensor, config) -> torch.Tensor:
+    """mixture holds inverse covariances (gm.evaluate_inversed)"""
+    return EvaluateInversedBvh.apply(mixture, xes, config, False)
+
+
+def apply_covariance(mixture: torch.Tensor, xes: torch.Tensor, config) -> torch.Tensor:
+    """mixture holds covariances (gm.evaluate, src/gmc/mixture.py:144-149): the inversion, its transpose and the
+    repacking are fused into the LBVH build, the backward pass carries the matrix gradient on to the covariance"""
+    return EvaluateInversedBvh.apply(mixture, xes, config, True)

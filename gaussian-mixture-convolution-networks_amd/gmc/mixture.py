@@ -109,13 +109,13 @@ def evaluate_inversed_with_amplitude_mixture(mixture: Tensor, xes: Tensor) -> Te
 
 
 def evaluate(mixture: Tensor, xes: Tensor, bvh: typing.Optional[BvhConfig] = None) -> Tensor:
-    """mixture holds covariances; returns [batch, layers, n_points].  The dense path inverts the covariances
-    inside the evaluation kernels (one read of the mixture, no intermediate tensors); the culled path inverts and
-    repacks first, as the reference does."""
+    """mixture holds covariances; returns [batch, layers, n_points].  Both paths invert the covariances inside
+    their kernels (one read of the mixture, no intermediate tensors): the dense path while it stages the
+    Gaussians, the culled path while it builds the boxes and leaf records of the LBVH."""
     if bvh is None:
         return cppExtensionsEvaluateInversed.apply_covariance(mixture, xes)
-    inv = mat_tools.inverse(covariances(mixture)).transpose(-1, -2)
-    return evaluate_inversed(pack_mixture(weights(mixture), positions(mixture), inv), xes, bvh)
+    from .cpp.extensions.evaluate_inversed import evaluate_inversed_bvh
+    return evaluate_inversed_bvh.apply_covariance(mixture, xes, bvh)
 
 
 def evaluate_componentwise_inversed(gaussians: Tensor, xes: Tensor) -> Tensor:

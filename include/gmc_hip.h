@@ -115,6 +115,8 @@ enum { GMC_AABB_REFERENCE = 0, GMC_AABB_TIGHT = 1 };
 typedef struct gmc_bvh_config {
     int aabb_mode;          /* GMC_AABB_REFERENCE: the rule of lbvh/bvh.cu:190-223; GMC_AABB_TIGHT: exact box */
     float aabb_threshold;   /* lbvh/Config.h:9, default 0.001f */
+    int covariance_form;    /* != 0: `mixture` holds COVARIANCES as gm.evaluate takes them (src/gmc/mixture.py:144-149);
+                               the inversion is fused into the build (boxes, leaf records), as in gmc_eval_cov_* */
 } gmc_bvh_config;
 
 /* Bytes of the opaque BVH object for `shape` (nodes, boxes, sorted orders, build scratch). */
@@ -134,6 +136,12 @@ int gmc_eval_bvh_fwd(const void* mixture, const void* xes, const void* bvh, void
 int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh,
                      void* grad_mixture, void* grad_xes, void* workspace, size_t workspace_bytes,
                      const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, void* stream);
+/* Backward pass over a BVH that was built with covariance_form != 0: `mixture` holds covariances and grad_mixture
+ * receives the gradient with respect to them (the chain through the inversion as in gmc_eval_cov_bwd;
+ * math/matrix_inverse.py:30-33).  The forward pass is gmc_eval_bvh_fwd in both forms (it reads the BVH only). */
+int gmc_eval_bvh_cov_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh,
+                         void* grad_mixture, void* grad_xes, void* workspace, size_t workspace_bytes,
+                         const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -183,6 +183,46 @@ def test_culled_random_shapes():
                       tag=f"case {case}: B{B} L{L} M{M} N{N} D{D} cov {cov} {dtype}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+@pytest.mark.parametrize("mode", ["reference", "tight"])
+def test_covariance_form_matches_explicit_inversion(dtype, D, mode):
+    """gm.evaluate(mixture with covariances, bvh=...) inverts inside the LBVH build; it must agree with the route of
+    the reference's gm.evaluate (src/gmc/mixture.py:144-149): mat_tools.inverse, transpose, pack, evaluate_inversed --
+    same boxes, same values, and the same gradients after autograd has carried them through the inversion."""
+    from gmc import mat_tools
+    mix_inv, xes, gout = _case(2, 3, 90, 700, D, 611 + D)
+    cov = torch.linalg.inv(gm.covariances(mix_inv)).transpose(-1, -2)
+    skew = torch.randn(cov.shape, generator=torch.Generator().manual_seed(5), dtype=cov.dtype)
+    cov = cov @ (torch.eye(D, dtype=cov.dtype) + 0.05 * (skew - skew.transpose(-1, -2)))      # not symmetric, det > 0
+    mix_cov = gm.pack_mixture(gm.weights(mix_inv), gm.positions(mix_inv), cov)
+    cfg = gm.BvhConfig(aabb_mode=mode)
+    g = gout.to(dtype).to(DEV)
+
+    a = mix_cov.to(dtype).to(DEV).requires_grad_(True)
+    xa = xes.to(dtype).to(DEV).requires_grad_(True)
+    out_a = gm.evaluate(a, xa, bvh=cfg)
+    out_a.backward(g)
+
+    b = mix_cov.to(dtype).to(DEV).requires_grad_(True)
+    xb = xes.to(dtype).to(DEV).requires_grad_(True)
+    inv = mat_tools.inverse(gm.covariances(b)).transpose(-1, -2)      # backward as math/matrix_inverse.py:30-33
+    packed = gm.pack_mixture(gm.weights(b), gm.positions(b), inv)
+    out_b = gm.evaluate_inversed(packed, xb, bvh=cfg)
+    out_b.backward(g)
+
+    lo_a, up_a = _native.Bvh(a.detach(), xa.detach(), cfg.aabb_threshold, mode, True).boxes()
+    lo_b, up_b = _native.Bvh(packed.detach().contiguous(), xb.detach(), cfg.aabb_threshold, mode).boxes()
+    # float32: the second route rounds the inverse to float32 before the box rule sees it, and a point next to a
+    # box face may then fall on the other side; double precision keeps both routes on the same side
+    tol = 1e-11 if dtype == torch.float64 else 2e-3
+    n = lambda t: t.detach().cpu().numpy().astype(np.float64)
+    assert rel_l2(n(up_a - lo_a), n(up_b - lo_b)) <= (1e-11 if dtype == torch.float64 else 1e-4)
+    assert rel_l2(n(out_a), n(out_b), FLOOR[dtype]) <= tol
+    assert rel_l2(n(a.grad), n(b.grad), FLOOR[dtype]) <= tol
+    assert rel_l2(n(xa.grad), n(xb.grad), FLOOR[dtype]) <= tol
+
+
 def test_points_outside_every_box_and_need_flags():
     mix, xes, gout = _case(1, 2, 40, 64, 3, seed=400)
     far = xes + 1000.0

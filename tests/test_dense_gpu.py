@@ -273,6 +273,17 @@ def test_evaluate_covariance_form_fused_inverse(dtype, D):
     out2.backward(gout.to(DEV))
     assert rel_l2(out2.detach().cpu().numpy(), out.detach().cpu().numpy(), fl) <= tol
     assert rel_l2(m2.grad.cpu().numpy(), gmix, fl) <= tol * 2
+    # matrices that are not symmetric: the fused chain rule follows MatrixInverse.backward of the reference
+    # (math/matrix_inverse.py:30-33, -S^-1 g S^-1 without transposes), which gmc.mat_tools.inverse restates
+    skew = torch.randn(cov.shape, generator=g, dtype=torch.float64)
+    cov_ns = cov @ (torch.eye(D, dtype=torch.float64) + 0.05 * (skew - skew.transpose(-1, -2)))
+    mix_ns = gm.pack_mixture(w, pos, cov_ns).to(dtype)
+    m3 = mix_ns.to(DEV).requires_grad_(True)
+    gm.evaluate(m3, x.detach()).backward(gout.to(DEV))
+    m4 = mix_ns.to(DEV).requires_grad_(True)
+    inv = mat_tools.inverse(gm.covariances(m4)).transpose(-1, -2)
+    gm.evaluate_inversed(gm.pack_mixture(gm.weights(m4), gm.positions(m4), inv), x.detach()).backward(gout.to(DEV))
+    assert rel_l2(m3.grad.cpu().numpy(), m4.grad.cpu().numpy(), fl) <= tol * 2
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
