@@ -43,9 +43,17 @@ struct BvhLayout {
     size_t hist_g, hist_p;      // uint32 [segments][blocks][256] block histograms of one radix pass
     size_t p_order;             // int [BxLx][N]           Morton order of the query points
     size_t g_keys;              // uint32 [BL][M]          sorted Morton codes of the leaves
+    size_t cand_count;          // int [BL][ceil(N/64)]    candidate leaves of every point group, -1: not known
+    size_t cand_list;           // int [BL][ceil(N/64)][kLeafCap]  (both empty when they would exceed kCandCacheBytes)
+    bool cand_cache;
     size_t total;
 };
 
+constexpr int kLeafFlush = 512;         // traversal: candidate leaves are evaluated whenever this many have gathered
+constexpr int kLeafCap = kLeafFlush + 128;
+// The candidate list of a point group depends on the tree and the points only, so the first traversal after a
+// build leaves it in the BVH object and later ones (the backward pass after the forward pass) skip the descent.
+constexpr size_t kCandCacheBytes = size_t(64) << 20;    // no such lists for launches that would need more
 constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
 constexpr int kSortBlocksMax = 256;                 // radix blocks per segment (more items per lane beyond that)
 constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the partial bounds of the query points
@@ -98,6 +106,12 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.hist_p = take(XL * sort_blocks(N) * 256 * 4);
     l.p_order = take(XL * N * 4);
     l.g_keys = take(BL * M * 4);
+    {
+        const size_t point_groups = BL * ((N + kWave - 1) / kWave);
+        l.cand_cache = M > 1 && point_groups > 0 && point_groups * kLeafCap * 4 <= kCandCacheBytes;
+        l.cand_count = take(l.cand_cache ? point_groups * 4 : 0);
+        l.cand_list = take(l.cand_cache ? point_groups * kLeafCap * 4 : 0);
+    }
     l.total = o;
     return l;
 }
@@ -633,8 +647,11 @@ __global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int* __restrict
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __restrict__ children,
                                                                 const long long* __restrict__ enc_box, T* node_box,
-                                                                T* __restrict__ child_box, int M, size_t total) {
+                                                                T* __restrict__ child_box, int M, size_t total,
+                                                                int* __restrict__ cand_count, size_t point_groups) {
     const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (cand_count)                                  // a new tree: no candidate list is known yet
+        for (size_t j = t; j < point_groups; j += size_t(gridDim.x) * kBlock) cand_count[j] = -1;
     if (t >= total) return;
     const size_t bl = t / (M - 1);
     const int node = int(t - bl * (M - 1));
@@ -690,8 +707,6 @@ __device__ __forceinline__ T leaf_terms(const T* __restrict__ r, const T (&x)[D]
 template <int D> struct BvhSums { static constexpr int k = 1 + D + D * (D + 1) / 2; };
 
 constexpr int kStackCap = 512;          // soft capacity of a node stack (the array has 128 more)
-constexpr int kLeafFlush = 512;         // candidate leaves are evaluated whenever this many have gathered
-constexpr int kLeafCap = kLeafFlush + 128;
 constexpr int kTravWaves = 8;           // wavefronts per workgroup of the traversal
 constexpr int kTravBlock = kTravWaves * kWave;
 constexpr int kGroupsMax = 4;           // 64-point groups per workgroup (each descends the tree with its own wavefront)
@@ -745,8 +760,8 @@ template <typename T, int D, int MODE, bool NEED_GM, bool NEED_GX>
 __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4))) void bvh_traverse_kernel(
         const T* __restrict__ xes, const int* __restrict__ p_order, const T* __restrict__ child_box,
         const int2* __restrict__ children, const T* __restrict__ leaf_rec, T* __restrict__ out,
-        const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes, int L, int M, int N, int Bx,
-        int Lx, int chunks, int groups, int xes_shared) {
+        const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes, int* __restrict__ cand_count,
+        int* __restrict__ cand_list, int L, int M, int N, int Bx, int Lx, int chunks, int groups, int xes_shared) {
     constexpr int LS = LeafRec<D>::kStride;
     constexpr int NR = BvhSums<D>::k;
     constexpr int kVals = MODE == 0 ? 1 : D;
@@ -778,6 +793,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
 
     // wavefront i loads the points of group i and their bounding box
     int sp = 0;                                             // nodes on this wavefront's stack (wave-uniform)
+    size_t cache_slot = ~size_t(0);                         // where this wavefront's descent leaves its candidate list
     if (wave < groups) {
         // The groups of a workgroup lie far apart in Morton order, one in every quarter of the range and at
         // different places within the quarters: point groups with long candidate lists come in clusters (dense
@@ -808,6 +824,17 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             state[wave][1] = 0;
         }
         sp = (any && M > 1) ? 1 : 0;
+        // candidate list left by an earlier traversal of this tree: no descent
+        if (cand_count && sp > 0) {
+            cache_slot = size_t(bl) * ((N + kWave - 1) / kWave) + group;
+            const int known = __builtin_amdgcn_readfirstlane(cand_count[cache_slot]);
+            if (known >= 0 && known <= kLeafCap) {
+                for (int i = lane; i < known; i += kWave) leaves[wave][i] = cand_list[cache_slot * kLeafCap + i];
+                if (lane == 0) state[wave][0] = known;
+                sp = 0;
+                cache_slot = ~size_t(0);
+            }
+        }
     }
     for (int i = threadIdx.x; i < kGroupsMax * kVals * kWave; i += kTravBlock) (&result[0][0][0])[i] = 0.0;
 
@@ -1021,6 +1048,15 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                 }
             }
             if (lane == 0) { state[wave][0] = n_leaf; state[wave][1] = sp; }
+            // a descent that ends in the first round has the group's whole list: keep it for later traversals
+            if (cache_slot != ~size_t(0)) {
+                if (round == 0 && sp == 0) {
+                    wave_lds_fence();
+                    for (int i = lane; i < n_leaf; i += kWave) cand_list[cache_slot * kLeafCap + i] = cand[i];
+                    if (lane == 0) cand_count[cache_slot] = n_leaf;
+                }
+                cache_slot = ~size_t(0);
+            }
         }
         __syncthreads();
         bool left_on_stack = false;
@@ -1250,7 +1286,9 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         if (M > 1) {
             const size_t ni = BL * (M - 1);
             bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(parent, node_box, enc_box, M, n);
-            bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(children, enc_box, node_box, child_box, M, ni);
+            bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(
+                children, enc_box, node_box, child_box, M, ni, lay.cand_cache ? (int*)(bvh + lay.cand_count) : nullptr,
+                BL * ((size_t(N) + kWave - 1) / kWave));
         }
     }
     if (have_p && !sort_p) iota_segments_kernel<<<dim3(grid_for(XL * N)), dim3(kBlock), 0, st>>>(p_order, N, XL * N);
@@ -1269,7 +1307,7 @@ static int traversal_groups(size_t BL, int N) {
 }
 
 template <typename T, int D>
-static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, hipStream_t st) {
+static int bvh_fwd_t(const T* xes, char* bvh, T* out, const gmc_shape& s, hipStream_t st) {
     const BvhLayout lay = bvh_layout(s);
     const size_t BL = size_t(s.B) * s.L;
     if (BL == 0 || s.N == 0) return GMC_OK;
@@ -1282,12 +1320,13 @@ static int bvh_fwd_t(const T* xes, const char* bvh, T* out, const gmc_shape& s, 
     const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kTravBlock), 0, st>>>(
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children),
-        (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, 0);
+        (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, lay.cand_cache ? (int*)(bvh + lay.cand_count) : nullptr,
+        lay.cand_cache ? (int*)(bvh + lay.cand_list) : nullptr, s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, 0);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
 template <typename T, int D>
-static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, const char* bvh, T* grad_mixture, T* grad_xes,
+static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bvh, T* grad_mixture, T* grad_xes,
                      T* sums, const gmc_shape& s, bool gm, bool gx, bool covariance_form, hipStream_t st) {
     constexpr int G = 1 + D + D * D;
     constexpr int NR = BvhSums<D>::k;
@@ -1311,8 +1350,9 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, const ch
     const dim3 grid(unsigned(BL * chunks));
 #define GMC_TRAV(GM, GX) bvh_traverse_kernel<T, D, 1, GM, GX><<<grid, dim3(kTravBlock), 0, st>>>( \
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children), \
-        (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, \
-        xes_shared)
+        (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, \
+        lay.cand_cache ? (int*)(bvh + lay.cand_count) : nullptr, lay.cand_cache ? (int*)(bvh + lay.cand_list) : nullptr, \
+        s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, xes_shared)
     if (gm && gx) GMC_TRAV(true, true);
     else if (gm) GMC_TRAV(true, false);
     else if (gx) GMC_TRAV(false, true);
@@ -1402,20 +1442,20 @@ int gmc_bvh_export_nodes(const void* bvh, int32_t* nodes, void* node_boxes, cons
 #undef ARGS
 }
 
-int gmc_eval_bvh_fwd(const void* mixture, const void* xes, const void* bvh, void* out, const gmc_shape* shape,
+int gmc_eval_bvh_fwd(const void* mixture, const void* xes, void* bvh, void* out, const gmc_shape* shape,
                      void* stream) {
     (void)mixture;   // the leaf records inside the BVH hold everything the forward pass needs
     const int rc = check_bvh_shape(shape);
     if (rc != GMC_OK) return rc;
     if (size_t(shape->B) * shape->L * shape->N == 0) return GMC_OK;
     if (!out || !xes || (!bvh && shape->M > 0)) return GMC_E_NULL;
-#define ARGS(T) (const T*)xes, (const char*)bvh, (T*)out, *shape, (hipStream_t)stream
+#define ARGS(T) (const T*)xes, (char*)bvh, (T*)out, *shape, (hipStream_t)stream
     if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_fwd_t<float, 2>(ARGS(float)) : gmc::bvh_fwd_t<float, 3>(ARGS(float));
     return shape->D == 2 ? gmc::bvh_fwd_t<double, 2>(ARGS(double)) : gmc::bvh_fwd_t<double, 3>(ARGS(double));
 #undef ARGS
 }
 
-static int eval_bvh_bwd_impl(const void* grad_out, const void* mixture, const void* xes, const void* bvh,
+static int eval_bvh_bwd_impl(const void* grad_out, const void* mixture, const void* xes, void* bvh,
                              void* grad_mixture, void* grad_xes, void* workspace, size_t workspace_bytes,
                              const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, bool covariance_form,
                              void* stream) {
@@ -1433,20 +1473,20 @@ static int eval_bvh_bwd_impl(const void* grad_out, const void* mixture, const vo
         if (workspace_bytes < need) return GMC_E_WORKSPACE;
         if (!workspace) return GMC_E_NULL;
     }
-#define ARGS(T) (const T*)grad_out, (const T*)mixture, (const T*)xes, (const char*)bvh, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, *shape, gm, gx, covariance_form, (hipStream_t)stream
+#define ARGS(T) (const T*)grad_out, (const T*)mixture, (const T*)xes, (char*)bvh, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, *shape, gm, gx, covariance_form, (hipStream_t)stream
     if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_bwd_t<float, 2>(ARGS(float)) : gmc::bvh_bwd_t<float, 3>(ARGS(float));
     return shape->D == 2 ? gmc::bvh_bwd_t<double, 2>(ARGS(double)) : gmc::bvh_bwd_t<double, 3>(ARGS(double));
 #undef ARGS
 }
 
-int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh, void* grad_mixture,
+int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh, void* grad_mixture,
                      void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
                      int need_grad_mixture, int need_grad_xes, void* stream) {
     return eval_bvh_bwd_impl(grad_out, mixture, xes, bvh, grad_mixture, grad_xes, workspace, workspace_bytes, shape,
                              need_grad_mixture, need_grad_xes, false, stream);
 }
 
-int gmc_eval_bvh_cov_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh, void* grad_mixture,
+int gmc_eval_bvh_cov_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh, void* grad_mixture,
                          void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
                          int need_grad_mixture, int need_grad_xes, void* stream) {
     return eval_bvh_bwd_impl(grad_out, mixture, xes, bvh, grad_mixture, grad_xes, workspace, workspace_bytes, shape,

@@ -131,15 +131,18 @@ int gmc_bvh_export_boxes(const void* bvh, void* lower, void* upper, const gmc_sh
  * nodes first, and node boxes [B][L][2M-1][2*D] (lower, upper). */
 int gmc_bvh_export_nodes(const void* bvh, int32_t* nodes, void* node_boxes, const gmc_shape* shape, void* stream);
 
-int gmc_eval_bvh_fwd(const void* mixture, const void* xes, const void* bvh, void* out, const gmc_shape* shape,
+/* The first traversal after a build leaves the candidate leaves of every 64-point group in the BVH object
+ * (when they fit into 64 MiB) and later traversals of the same object skip the tree descent, so the object is
+ * written to by these calls: calls that use one BVH object must be ordered (same stream, or events). */
+int gmc_eval_bvh_fwd(const void* mixture, const void* xes, void* bvh, void* out, const gmc_shape* shape,
                      void* stream);
-int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh,
+int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh,
                      void* grad_mixture, void* grad_xes, void* workspace, size_t workspace_bytes,
                      const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, void* stream);
 /* Backward pass over a BVH that was built with covariance_form != 0: `mixture` holds covariances and grad_mixture
  * receives the gradient with respect to them (the chain through the inversion as in gmc_eval_cov_bwd;
  * math/matrix_inverse.py:30-33).  The forward pass is gmc_eval_bvh_fwd in both forms (it reads the BVH only). */
-int gmc_eval_bvh_cov_bwd(const void* grad_out, const void* mixture, const void* xes, const void* bvh,
+int gmc_eval_bvh_cov_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh,
                          void* grad_mixture, void* grad_xes, void* workspace, size_t workspace_bytes,
                          const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, void* stream);
 
