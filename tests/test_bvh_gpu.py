@@ -223,6 +223,34 @@ def test_covariance_form_matches_explicit_inversion(dtype, D, mode):
     assert rel_l2(n(xa.grad), n(xb.grad), FLOOR[dtype]) <= tol
 
 
+def test_candidate_lists_kept_in_the_bvh_object():
+    """The first traversal after a build leaves the candidate list of every point group in the BVH object and later
+    ones skip the descent: a second forward pass is bit-identical to the first, a backward pass gives the same
+    gradients with and without a forward pass before it, and a rebuild into the same object forgets the lists."""
+    import ctypes
+    mix, xes, gout = _case(2, 2, 300, 3000, 3, 640, cov_radius=0.1)
+    m, x, g = (t.to(DEV).contiguous() for t in (mix, xes, gout))
+    bvh = _native.Bvh(m, x, 0.001, "tight")
+    first = _native.eval_bvh_fwd(m, x, bvh)
+    second = _native.eval_bvh_fwd(m, x, bvh)
+    assert torch.equal(first, second)
+    gm_a, gx_a = _native.eval_bvh_bwd(g, m, x, bvh, True, True)              # lists known
+    fresh = _native.Bvh(m, x, 0.001, "tight")
+    gm_b, gx_b = _native.eval_bvh_bwd(g, m, x, fresh, True, True)            # descends itself
+    n = lambda t: t.cpu().numpy()
+    assert rel_l2(n(gm_a), n(gm_b)) <= 1e-13 and rel_l2(n(gx_a), n(gx_b)) <= 1e-13
+    # another mixture built into the same object
+    mix2, _, _ = _case(2, 2, 300, 3000, 3, 641, cov_radius=0.1)
+    m2 = mix2.to(DEV).contiguous()
+    cfg = _native._bvh_config(0.001, "tight")
+    with torch.cuda.device(m2.device):
+        _native.check(_native.lib().gmc_bvh_build(_native._p(m2), _native._p(x), _native._p(bvh.blob), bvh.blob.numel(),
+                                                  ctypes.byref(bvh.shape), ctypes.byref(cfg), _native._stream(m2.device)))
+    again = _native.eval_bvh_fwd(m2, x, bvh)
+    assert torch.equal(again, _native.eval_bvh_fwd(m2, x, _native.Bvh(m2, x, 0.001, "tight")))
+    assert not torch.equal(again, first)
+
+
 def test_points_outside_every_box_and_need_flags():
     mix, xes, gout = _case(1, 2, 40, 64, 3, seed=400)
     far = xes + 1000.0
