@@ -44,8 +44,14 @@ struct BvhLayout {
     size_t p_order;             // int [BxLx][N]           Morton order of the query points
     size_t g_keys;              // uint32 [BL][M]          sorted Morton codes of the leaves
     size_t cand_count;          // int [BL][ceil(N/64)]    candidate leaves of every point group, -1: not known
-    size_t cand_list;           // int [BL][ceil(N/64)][kLeafCap]  (both empty when they would exceed kCandCacheBytes)
+    size_t cand_list;           // int [BL][ceil(N/64)][kLeafCap], then a pool of pool_cap ints for the lists of
+                                // later rounds (all empty when the lists would exceed kCandCacheBytes)
+    size_t cand_ctl;            // int [2]                 pieces published, pool ints handed out
+    size_t pieces;              // int4 [pieces_max]       (point group, offset into cand_list, leaves, -)
+    size_t piece_gx;            // T [pieces_max][D][64]   dL/dx of the pieces, added to grad_xes by the epilogue
     bool cand_cache;
+    int pieces_max, pool_cap;
+    size_t point_groups;
     size_t total;
 };
 
@@ -54,6 +60,31 @@ constexpr int kLeafCap = kLeafFlush + 128;
 // The candidate list of a point group depends on the tree and the points only, so the first traversal after a
 // build leaves it in the BVH object and later ones (the backward pass after the forward pass) skip the descent.
 constexpr size_t kCandCacheBytes = size_t(64) << 20;    // no such lists for launches that would need more
+// Point groups in dense regions have candidate lists ten times the average, and the workgroup that owns such a
+// group would finish long after all others.  The first traversal therefore cuts a list of more than kPieceLeaves
+// leaves into equal pieces of at most that size and publishes all but the first as (group, offset, leaves); in a
+// backward pass on known lists the owner works on the first piece only and helper workgroups, one per published
+// piece, on the others (their dL/dx goes through piece_gx and the epilogue).  Lists of later rounds of a long
+// descent live in a pool behind the fixed slots and are handed out as pieces entirely.
+constexpr int kPieceLeaves = 240;        // measured 160 ... 480: shorter pieces cost more in fixed work per workgroup
+constexpr int kPiecesMax = 512;         // helper workgroups of a backward launch
+constexpr int kPendMax = 16;            // pieces of one point group
+constexpr int kCandSplit = 1 << 20;     // flag in cand_count: pieces of this group's list are published
+constexpr int kCandRounds = 1 << 21;    // flag in cand_count: the fixed slot holds the first round's list only
+constexpr int kCandMask = kCandSplit - 1;
+
+__host__ __device__ inline int own_share(int n) {
+    const int pieces = (n + kPieceLeaves - 1) / kPieceLeaves;
+    return pieces > 1 ? (n + pieces - 1) / pieces : n;
+}
+
+struct CandidateCache {
+    int* count;
+    int* list;
+    int* ctl;
+    int4* pieces;
+    int pieces_max, pool_cap, pool_base;
+};
 constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
 constexpr int kSortBlocksMax = 256;                 // radix blocks per segment (more items per lane beyond that)
 constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the partial bounds of the query points
@@ -108,12 +139,31 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.g_keys = take(BL * M * 4);
     {
         const size_t point_groups = BL * ((N + kWave - 1) / kWave);
+        l.point_groups = point_groups;
         l.cand_cache = M > 1 && point_groups > 0 && point_groups * kLeafCap * 4 <= kCandCacheBytes;
+        l.pieces_max = l.cand_cache ? int(point_groups / 2 < size_t(kPiecesMax) ? point_groups / 2 : size_t(kPiecesMax)) : 0;
+        l.pool_cap = l.cand_cache ? int(65536 + point_groups * 16) : 0;
         l.cand_count = take(l.cand_cache ? point_groups * 4 : 0);
-        l.cand_list = take(l.cand_cache ? point_groups * kLeafCap * 4 : 0);
+        l.cand_list = take(l.cand_cache ? (point_groups * kLeafCap + l.pool_cap) * 4 : 0);
+        l.cand_ctl = take(l.cand_cache ? 8 : 0);
+        l.pieces = take(size_t(l.pieces_max) * 16);
+        l.piece_gx = take(size_t(l.pieces_max) * D * kWave * e);
     }
     l.total = o;
     return l;
+}
+
+static CandidateCache candidate_cache(char* bvh, const BvhLayout& lay) {
+    CandidateCache c{};
+    if (!lay.cand_cache) return c;
+    c.count = (int*)(bvh + lay.cand_count);
+    c.list = (int*)(bvh + lay.cand_list);
+    c.ctl = (int*)(bvh + lay.cand_ctl);
+    c.pieces = (int4*)(bvh + lay.pieces);
+    c.pieces_max = lay.pieces_max;
+    c.pool_cap = lay.pool_cap;
+    c.pool_base = int(lay.point_groups * kLeafCap);
+    return c;
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -648,10 +698,12 @@ template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __restrict__ children,
                                                                 const long long* __restrict__ enc_box, T* node_box,
                                                                 T* __restrict__ child_box, int M, size_t total,
-                                                                int* __restrict__ cand_count, size_t point_groups) {
+                                                                CandidateCache cache, size_t point_groups) {
     const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
-    if (cand_count)                                  // a new tree: no candidate list is known yet
-        for (size_t j = t; j < point_groups; j += size_t(gridDim.x) * kBlock) cand_count[j] = -1;
+    if (cache.count) {                               // a new tree: no candidate list is known yet
+        for (size_t j = t; j < point_groups; j += size_t(gridDim.x) * kBlock) cache.count[j] = -1;
+        if (t < 2) cache.ctl[t] = 0;
+    }
     if (t >= total) return;
     const size_t bl = t / (M - 1);
     const int node = int(t - bl * (M - 1));
@@ -760,8 +812,9 @@ template <typename T, int D, int MODE, bool NEED_GM, bool NEED_GX>
 __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4))) void bvh_traverse_kernel(
         const T* __restrict__ xes, const int* __restrict__ p_order, const T* __restrict__ child_box,
         const int2* __restrict__ children, const T* __restrict__ leaf_rec, T* __restrict__ out,
-        const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes, int* __restrict__ cand_count,
-        int* __restrict__ cand_list, int L, int M, int N, int Bx, int Lx, int chunks, int groups, int xes_shared) {
+        const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes, CandidateCache cache,
+        T* __restrict__ piece_gx, int helpers, int L, int M, int N, int Bx, int Lx, int chunks, int groups_per_workgroup,
+        int xes_shared) {
     constexpr int LS = LeafRec<D>::kStride;
     constexpr int NR = BvhSums<D>::k;
     constexpr int kVals = MODE == 0 ? 1 : D;
@@ -781,8 +834,24 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     // double in both precisions: LDS atomic adds of doubles on distinct addresses cost a few cycles per
     // instruction, those of floats are serialised lane by lane
     __shared__ double rsum_mem[kTravWaves][NEED_GM ? kStageBatch * NR : 1];
-    const int bl = blockIdx.x / chunks;
-    const int chunk = blockIdx.x - bl * chunks;
+    __shared__ int2 pend[kGroupsMax][kPendMax];             // pieces of a group's list that wait to be published
+    const int per_mixture = (N + kWave - 1) / kWave;        // point groups of one mixture
+    // The last `helpers` workgroups of a backward launch each take one published piece of a long candidate list
+    // (no descent: one group, its points, a slice of its list); all others own `groups_per_workgroup` groups.
+    // (Last, because most of them find no piece: at the end of the grid they start when compute units run idle.)
+    const int owners = int(gridDim.x) - (MODE == 1 ? helpers : 0);
+    const int piece = int(blockIdx.x) >= owners ? int(blockIdx.x) - owners : -1;
+    int4 piece_desc = make_int4(0, 0, 0, 0);
+    if (piece >= 0) {
+        const int published = cache.ctl[0] < cache.pieces_max ? cache.ctl[0] : cache.pieces_max;
+        if (piece >= published) return;
+        piece_desc = cache.pieces[piece];
+        if (piece_desc.z <= 0) return;                      // a slot whose group could not publish all its pieces
+    }
+    const int groups = piece >= 0 ? 1 : groups_per_workgroup;
+    const int wg = piece >= 0 ? 0 : int(blockIdx.x);
+    const int bl = piece >= 0 ? piece_desc.x / per_mixture : wg / chunks;
+    const int chunk = wg - bl * chunks;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const size_t xseg = size_t(xb) * Lx + xl;
@@ -793,12 +862,15 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
 
     // wavefront i loads the points of group i and their bounding box
     int sp = 0;                                             // nodes on this wavefront's stack (wave-uniform)
-    size_t cache_slot = ~size_t(0);                         // where this wavefront's descent leaves its candidate list
+    int cache_slot = -1;                                    // the group whose candidate list this wavefront's descent leaves
+    bool cache_ok = true;                                   // ... as long as every part of it found room
+    int first_round_leaves = 0, n_pend = 0;
     if (wave < groups) {
         // The groups of a workgroup lie far apart in Morton order, one in every quarter of the range and at
         // different places within the quarters: point groups with long candidate lists come in clusters (dense
         // regions), often at matching places of a symmetric point set.
-        const int group = wave * chunks + (chunk + wave * (chunks / (groups + 1))) % chunks;
+        const int group = piece >= 0 ? piece_desc.x - bl * per_mixture
+                                     : wave * chunks + (chunk + wave * (chunks / (groups + 1))) % chunks;
         const int j = group * kWave + lane;
         const bool valid = j < N;
         const int pid = valid ? p_order[xseg * N + j] : 0;
@@ -824,15 +896,25 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             state[wave][1] = 0;
         }
         sp = (any && M > 1) ? 1 : 0;
-        // candidate list left by an earlier traversal of this tree: no descent
-        if (cand_count && sp > 0) {
-            cache_slot = size_t(bl) * ((N + kWave - 1) / kWave) + group;
-            const int known = __builtin_amdgcn_readfirstlane(cand_count[cache_slot]);
-            if (known >= 0 && known <= kLeafCap) {
-                for (int i = lane; i < known; i += kWave) leaves[wave][i] = cand_list[cache_slot * kLeafCap + i];
-                if (lane == 0) state[wave][0] = known;
-                sp = 0;
-                cache_slot = ~size_t(0);
+        if (piece >= 0) {
+            for (int i = lane; i < piece_desc.z; i += kWave) leaves[0][i] = cache.list[piece_desc.y + i];
+            if (lane == 0) state[0][0] = piece_desc.z;
+            sp = 0;
+        } else if (cache.count && sp > 0) {
+            // candidate list left by an earlier traversal of this tree: no descent.  The backward pass leaves the
+            // published pieces of a long list to the helper workgroups; the forward pass has no helpers, so it
+            // takes a whole single-round list and descends again for a list of several rounds.
+            cache_slot = bl * per_mixture + group;
+            const int known = __builtin_amdgcn_readfirstlane(cache.count[cache_slot]);
+            if (known >= 0) {
+                const int all = known & kCandMask;
+                const int n = (MODE == 1 && (known & kCandSplit)) ? own_share(all) : all;
+                if (MODE == 1 || !(known & kCandRounds)) {
+                    for (int i = lane; i < n; i += kWave) leaves[wave][i] = cache.list[size_t(cache_slot) * kLeafCap + i];
+                    if (lane == 0) state[wave][0] = n;
+                    sp = 0;
+                }
+                cache_slot = -1;
             }
         }
     }
@@ -1048,14 +1130,50 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                 }
             }
             if (lane == 0) { state[wave][0] = n_leaf; state[wave][1] = sp; }
-            // a descent that ends in the first round has the group's whole list: keep it for later traversals
-            if (cache_slot != ~size_t(0)) {
-                if (round == 0 && sp == 0) {
-                    wave_lds_fence();
-                    for (int i = lane; i < n_leaf; i += kWave) cand_list[cache_slot * kLeafCap + i] = cand[i];
-                    if (lane == 0) cand_count[cache_slot] = n_leaf;
+            // Keep the group's list for later traversals: the first round's in the group's fixed slot, those of
+            // later rounds in the pool; what exceeds the owner's share becomes pieces for helper workgroups,
+            // published when the descent has ended and every part has found room.  Only the forward pass publishes
+            // pieces (a backward launch has helpers running that read the piece table).
+            if (cache_slot >= 0) {
+                if (cache_ok && n_leaf > 0) {
+                    int base = cache_slot * kLeafCap, own = 0, share = n_leaf;
+                    if (n_leaf > kPieceLeaves) share = own_share(n_leaf);
+                    if (round == 0) {
+                        first_round_leaves = n_leaf;
+                        own = share;
+                    } else {
+                        int at = lane == 0 ? atomicAdd(&cache.ctl[1], n_leaf) : 0;
+                        at = __builtin_amdgcn_readfirstlane(at);
+                        cache_ok = at + n_leaf <= cache.pool_cap;
+                        base = cache.pool_base + at;
+                    }
+                    const int wanted = (n_leaf - own + share - 1) / share;
+                    if (wanted > 0 && (MODE != 0 || n_pend + wanted > kPendMax)) cache_ok = false;
+                    if (cache_ok) {
+                        wave_lds_fence();
+                        for (int i = lane; i < n_leaf; i += kWave) cache.list[size_t(base) + i] = cand[i];
+                        if (lane < wanted) {
+                            const int from = own + lane * share;
+                            pend[wave][n_pend + lane] = make_int2(base + from, n_leaf - from < share ? n_leaf - from : share);
+                        }
+                        n_pend += wanted;
+                    }
                 }
-                cache_slot = ~size_t(0);
+                if (sp == 0) {
+                    if (cache_ok && n_pend > 0) {
+                        int slot = lane == 0 ? atomicAdd(&cache.ctl[0], n_pend) : 0;
+                        slot = __builtin_amdgcn_readfirstlane(slot);
+                        cache_ok = slot + n_pend <= cache.pieces_max;
+                        wave_lds_fence();
+                        // slots in range are always filled: a helper must never read an unwritten piece
+                        if (lane < n_pend && slot + lane < cache.pieces_max)
+                            cache.pieces[slot + lane] = cache_ok ? make_int4(cache_slot, pend[wave][lane].x, pend[wave][lane].y, 0)
+                                                                 : make_int4(0, 0, 0, 0);
+                    }
+                    if (cache_ok && lane == 0)
+                        cache.count[cache_slot] = first_round_leaves | (n_pend > 0 ? kCandSplit : 0) | (round > 0 ? kCandRounds : 0);
+                    cache_slot = -1;
+                }
             }
         }
         __syncthreads();
@@ -1095,6 +1213,11 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
         out[size_t(bl) * N + pid] = T(result[wave][0][lane]);
     } else if (NEED_GX) {
         const T g = pts[wave][D][lane];
+        if (piece >= 0) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) piece_gx[(size_t(piece) * D + d) * kWave + lane] = -g * T(result[0][d][lane]);
+            return;
+        }
         T* dst = grad_xes + (xseg * N + pid) * D;
 #pragma unroll
         for (int d = 0; d < D; ++d) {
@@ -1111,9 +1234,31 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __restrict__ mixture, const T* __restrict__ sums,
                                                                  T* __restrict__ grad_mixture, size_t n,
-                                                                 bool covariance_form) {
+                                                                 bool covariance_form, CandidateCache cache,
+                                                                 const T* __restrict__ piece_gx,
+                                                                 const int* __restrict__ p_order, T* __restrict__ grad_xes,
+                                                                 int L, int N, int Bx, int Lx) {
     constexpr int G = 1 + D + D * D;
     constexpr int NR = BvhSums<D>::k;
+    // dL/dx of the pieces that helper workgroups of the traversal worked on: one wavefront per piece, added to
+    // what the owners of the point groups have stored (several pieces of a group meet here, hence atomics)
+    if (cache.count) {
+        const int published = cache.ctl[0] < cache.pieces_max ? cache.ctl[0] : cache.pieces_max;
+        const int per_mixture = (N + kWave - 1) / kWave;
+        const int lane = threadIdx.x & 63;
+        for (int p = blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6); p < published; p += gridDim.x * (kBlock / kWave)) {
+            const int4 desc = cache.pieces[p];
+            if (desc.z <= 0) continue;
+            const int bl = desc.x / per_mixture, group = desc.x - bl * per_mixture;
+            const int b = bl / L, l = bl - b * L;
+            const size_t xseg = size_t(b < Bx ? b : Bx - 1) * Lx + (l < Lx ? l : Lx - 1);
+            const int j = group * kWave + lane;
+            if (j >= N) continue;
+            const int pid = p_order[xseg * N + j];
+            for (int d = 0; d < D; ++d)
+                atomic_add(&grad_xes[(xseg * N + pid) * D + d], piece_gx[(size_t(p) * D + d) * kWave + lane]);
+        }
+    }
     const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
     if (i >= n) return;
     const T* g = mixture + i * G;
@@ -1287,8 +1432,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
             const size_t ni = BL * (M - 1);
             bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(parent, node_box, enc_box, M, n);
             bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(
-                children, enc_box, node_box, child_box, M, ni, lay.cand_cache ? (int*)(bvh + lay.cand_count) : nullptr,
-                BL * ((size_t(N) + kWave - 1) / kWave));
+                children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups);
         }
     }
     if (have_p && !sort_p) iota_segments_kernel<<<dim3(grid_for(XL * N)), dim3(kBlock), 0, st>>>(p_order, N, XL * N);
@@ -1320,8 +1464,8 @@ static int bvh_fwd_t(const T* xes, char* bvh, T* out, const gmc_shape& s, hipStr
     const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kTravBlock), 0, st>>>(
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children),
-        (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, lay.cand_cache ? (int*)(bvh + lay.cand_count) : nullptr,
-        lay.cand_cache ? (int*)(bvh + lay.cand_list) : nullptr, s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, 0);
+        (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, candidate_cache(bvh, lay), nullptr, 0,
+        s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, 0);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
@@ -1347,19 +1491,26 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bv
     if (gx && xes_shared) zero(grad_xes, n_x);
     const int groups = traversal_groups(BL, s.N);
     const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
-    const dim3 grid(unsigned(BL * chunks));
+    // one helper workgroup per piece that a forward pass may have published, behind the owners
+    const int helpers = lay.pieces_max;
+    const dim3 grid(unsigned(BL * chunks + helpers));
+    const CandidateCache cache = candidate_cache(bvh, lay);
+    T* piece_gx = (T*)(bvh + lay.piece_gx);
 #define GMC_TRAV(GM, GX) bvh_traverse_kernel<T, D, 1, GM, GX><<<grid, dim3(kTravBlock), 0, st>>>( \
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children), \
-        (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, \
-        lay.cand_cache ? (int*)(bvh + lay.cand_count) : nullptr, lay.cand_cache ? (int*)(bvh + lay.cand_list) : nullptr, \
+        (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, cache, piece_gx, helpers, \
         s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, xes_shared)
     if (gm && gx) GMC_TRAV(true, true);
     else if (gm) GMC_TRAV(true, false);
     else if (gx) GMC_TRAV(false, true);
 #undef GMC_TRAV
-    if (gm)
-        bvh_bwd_epilogue_kernel<T, D><<<dim3(grid_for(n_g)), dim3(kBlock), 0, st>>>(mixture, sums, grad_mixture, n_g,
-                                                                                    covariance_form);
+    const bool pieces_gx = gx && helpers > 0;
+    if (gm || pieces_gx) {
+        const unsigned blocks = gm ? grid_for(n_g) : unsigned((helpers + 3) / 4);
+        bvh_bwd_epilogue_kernel<T, D><<<dim3(blocks), dim3(kBlock), 0, st>>>(
+            mixture, sums, grad_mixture, gm ? n_g : 0, covariance_form, pieces_gx ? cache : CandidateCache{}, piece_gx,
+            (const int*)(bvh + lay.p_order), grad_xes, s.L, s.N, s.Bx, s.Lx);
+    }
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
@@ -1440,6 +1591,20 @@ int gmc_bvh_export_nodes(const void* bvh, int32_t* nodes, void* node_boxes, cons
     if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_export_t<float, 2>(ARGS(float)) : gmc::bvh_export_t<float, 3>(ARGS(float));
     return shape->D == 2 ? gmc::bvh_export_t<double, 2>(ARGS(double)) : gmc::bvh_export_t<double, 3>(ARGS(double));
 #undef ARGS
+}
+
+int gmc_bvh_export_candidate_stats(const void* bvh, int32_t* stats, const gmc_shape* shape, void* stream) {
+    const int rc = check_bvh_shape(shape);
+    if (rc != GMC_OK) return rc;
+    if (!stats) return GMC_E_NULL;
+    const gmc::BvhLayout lay = gmc::bvh_layout(*shape);
+    if (lay.cand_cache && !bvh) return GMC_E_NULL;
+    if (lay.cand_cache)
+        gmc::copy_kernel<int32_t><<<dim3(1), dim3(gmc::kBlock), 0, (hipStream_t)stream>>>(
+            (const int32_t*)((const char*)bvh + lay.cand_ctl), stats, 2);
+    else
+        gmc::fill_zero_kernel<int32_t><<<dim3(1), dim3(gmc::kBlock), 0, (hipStream_t)stream>>>(stats, 2);
+    return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
 int gmc_eval_bvh_fwd(const void* mixture, const void* xes, void* bvh, void* out, const gmc_shape* shape,

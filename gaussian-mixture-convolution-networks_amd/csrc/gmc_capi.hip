@@ -26,7 +26,7 @@ int check_shape(const gmc_shape* s) {
 
 extern "C" {
 
-int gmc_abi_version(void) { return 4; }
+int gmc_abi_version(void) { return 5; }
 
 const char* gmc_error_string(int code) {
     switch (code) {

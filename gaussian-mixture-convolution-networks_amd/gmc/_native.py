@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class Shape(ctypes.Structure):
@@ -74,6 +74,7 @@ def lib() -> ctypes.CDLL:
         l.gmc_bvh_build.argtypes = [vp, vp, vp, sz, shp, cfg, vp]
         l.gmc_bvh_export_boxes.argtypes = [vp, vp, vp, shp, vp]
         l.gmc_bvh_export_nodes.argtypes = [vp, vp, vp, shp, vp]
+        l.gmc_bvh_export_candidate_stats.argtypes = [vp, vp, shp, vp]
         l.gmc_eval_bvh_fwd.argtypes = [vp, vp, vp, vp, shp, vp]
         l.gmc_eval_bvh_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
         l.gmc_eval_bvh_cov_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
@@ -258,6 +259,14 @@ class Bvh:
         with torch.cuda.device(self.device):
             check(lib().gmc_bvh_export_nodes(_p(self.blob), _p(nodes), _p(nb), ctypes.byref(s), _stream(self.device)))
         return nodes, nb
+
+    def candidate_stats(self):
+        """int32 [2]: pieces of long candidate lists published for the backward pass, pool ints in use"""
+        stats = torch.empty((2,), dtype=torch.int32, device=self.device)
+        with torch.cuda.device(self.device):
+            check(lib().gmc_bvh_export_candidate_stats(_p(self.blob), _p(stats), ctypes.byref(self.shape),
+                                                       _stream(self.device)))
+        return stats
 
 
 def eval_bvh_fwd(mixture, xes, bvh: Bvh) -> torch.Tensor:

@@ -131,9 +131,17 @@ int gmc_bvh_export_boxes(const void* bvh, void* lower, void* upper, const gmc_sh
  * nodes first, and node boxes [B][L][2M-1][2*D] (lower, upper). */
 int gmc_bvh_export_nodes(const void* bvh, int32_t* nodes, void* node_boxes, const gmc_shape* shape, void* stream);
 
+/* Diagnostics for tests (no counterpart in the reference): stats[0] = pieces of long candidate lists that the
+ * forward traversals since the last build have handed to helper workgroups of the backward pass, stats[1] = ints
+ * of the pool of later rounds' lists in use; `stats` is device memory for two int32. */
+int gmc_bvh_export_candidate_stats(const void* bvh, int32_t* stats, const gmc_shape* shape, void* stream);
+
 /* The first traversal after a build leaves the candidate leaves of every 64-point group in the BVH object
  * (when they fit into 64 MiB) and later traversals of the same object skip the tree descent, so the object is
- * written to by these calls: calls that use one BVH object must be ordered (same stream, or events). */
+ * written to by these calls: calls that use one BVH object must be ordered (same stream, or events).  A forward
+ * pass also cuts candidate lists of more than 240 leaves into pieces; the backward pass that follows gives every
+ * piece but the first to a workgroup of its own, so that a few point groups in dense regions do not hold up the
+ * launch. */
 int gmc_eval_bvh_fwd(const void* mixture, const void* xes, void* bvh, void* out, const gmc_shape* shape,
                      void* stream);
 int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh,

@@ -251,6 +251,52 @@ def test_candidate_lists_kept_in_the_bvh_object():
     assert not torch.equal(again, first)
 
 
+def _crowded_case(B, seed, broadcast):
+    """800 Gaussians crowd around the origin and 200 lie scattered; a twentieth of the points sit inside the crowd,
+    so a few point groups have several hundred candidate leaves and most have a handful"""
+    g = torch.Generator().manual_seed(seed)
+    D = 3
+    crowd = synthetic.random_inversed_mixture(B, 1, 800, D, g, pos_radius=0.3, cov_radius=0.05, dtype=torch.float64)
+    far = synthetic.random_inversed_mixture(B, 1, 200, D, g, pos_radius=6.0, cov_radius=0.3, dtype=torch.float64)
+    mix = torch.cat([crowd, far], dim=2).contiguous()
+    Bx = 1 if broadcast else B
+    inner = (torch.rand((Bx, 1, 1280, D), generator=g, dtype=torch.float64) * 2 - 1) * 0.3
+    outer = (torch.rand((Bx, 1, 64 * 380, D), generator=g, dtype=torch.float64) * 2 - 1) * 6.0
+    xes = torch.cat([inner, outer], dim=2).contiguous()
+    gout = torch.randn((B, 1, xes.shape[2]), generator=g, dtype=torch.float64)
+    return mix, xes, gout
+
+
+@pytest.mark.parametrize("broadcast", [False, True])
+def test_long_candidate_lists_are_shared_between_workgroups(broadcast):
+    """A forward pass cuts candidate lists of several hundred leaves (also those gathered in several rounds) into
+    pieces, and the backward pass on the same BVH object gives the pieces to helper workgroups: the gradients must
+    equal those of a backward pass that descends itself and works through every list alone, with every combination
+    of the need flags, and a second forward pass (which walks the long lists itself) must repeat the first."""
+    mix, xes, gout = _crowded_case(2, 660, broadcast)
+    n = lambda t: t.cpu().numpy()
+    for dtype in (torch.float64, torch.float32):
+        m, x, g = (t.to(dtype).to(DEV).contiguous() for t in (mix, xes, gout))
+        bvh = _native.Bvh(m, x, 0.001, "tight")
+        assert n(bvh.candidate_stats()).tolist() == [0, 0]
+        first = _native.eval_bvh_fwd(m, x, bvh)
+        stats = n(bvh.candidate_stats()).tolist()
+        assert stats[0] > 20 and stats[1] > 0, "the case is meant to publish pieces, some from later rounds"
+        assert torch.equal(first, _native.eval_bvh_fwd(m, x, bvh))
+        assert n(bvh.candidate_stats()).tolist() == stats
+        gm_a, gx_a = _native.eval_bvh_bwd(g, m, x, bvh, True, True)
+        gm_b, gx_b = _native.eval_bvh_bwd(g, m, x, _native.Bvh(m, x, 0.001, "tight"), True, True)
+        tol = 1e-13 if dtype == torch.float64 else 2e-6       # two summation orders of the same terms
+        assert rel_l2(n(gm_a), n(gm_b)) <= tol and rel_l2(n(gx_a), n(gx_b)) <= tol
+        gm_c, gx_c = _native.eval_bvh_bwd(g, m, x, bvh, True, False)
+        gm_d, gx_d = _native.eval_bvh_bwd(g, m, x, bvh, False, True)
+        assert rel_l2(n(gm_c), n(gm_b)) <= tol and rel_l2(n(gx_d), n(gx_b)) <= tol
+        assert not gx_c.any() and not gm_d.any()
+    # and against the brute-force masked sum, through the autograd binding
+    _check_culled(mix, xes, gout, torch.float64, "tight", tag=f"crowded, broadcast {broadcast}")
+    _check_culled(mix, xes, gout, torch.float32, "tight", tag=f"crowded, broadcast {broadcast}")
+
+
 def test_points_outside_every_box_and_need_flags():
     mix, xes, gout = _case(1, 2, 40, 64, 3, seed=400)
     far = xes + 1000.0
