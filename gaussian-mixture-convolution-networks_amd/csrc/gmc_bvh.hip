@@ -35,6 +35,7 @@ struct BvhLayout {
     size_t leaf_rec;            // T [BL][M][RS]           evaluation records in leaf order
     size_t children;            // int2 [BL][M-1]          left, right: >= 0 internal node, < 0 leaf ~index
     size_t parent;              // int [BL][2M-1]
+    size_t node_range;          // int2 [BL][M-1]          first and last leaf below every internal node
     size_t leaf_comp;           // int [BL][M]             component id of each leaf
     size_t enc_box;             // int64 [BL][M-1][2D]     boxes of the internal nodes as order-preserving integers
     size_t parts_g, parts_p;    // T [segments][blocks][2D] per-block partial bounds of the centres / the query points
@@ -87,6 +88,7 @@ struct CandidateCache {
 };
 constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
 constexpr int kSortBlocksMax = 256;                 // radix blocks per segment (more items per lane beyond that)
+constexpr int kCoarseOrderMax = 8192;               // point segments up to this size are ordered by 8 Morton bits only
 constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the partial bounds of the query points
 
 // items per lane of a radix block for segments of `count` keys
@@ -121,6 +123,7 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.leaf_rec = take(BL * M * rs * e);
     l.children = take(BL * (M > 0 ? M - 1 : 0) * 8);
     l.parent = take(BL * nodes * 4);
+    l.node_range = take(BL * (M > 0 ? M - 1 : 0) * 8);
     l.leaf_comp = take(BL * M * 4);
     l.enc_box = take(BL * (M > 0 ? M - 1 : 0) * 2 * D * 8);
     l.parts_g = take(BL * ((M + kBlock - 1) / kBlock) * 2 * D * e);
@@ -572,7 +575,8 @@ __device__ __forceinline__ int common_prefix(const uint32_t* __restrict__ keys, 
 
 // internal node i of the radix tree of mixture bl (Karras 2012; lbvh/building.h:11-103)
 __device__ __forceinline__ void build_internal_node(const uint32_t* __restrict__ keys, int2* __restrict__ children,
-                                                    int* __restrict__ parent, int M, size_t bl, int i) {
+                                                    int* __restrict__ parent, int2* __restrict__ node_range, int M,
+                                                    size_t bl, int i) {
     const size_t t = bl * (M - 1) + i;
     const uint32_t* k = keys + bl * M;
     // range of keys covered by internal node i
@@ -602,6 +606,7 @@ __device__ __forceinline__ void build_internal_node(const uint32_t* __restrict__
     const int left = (split == first) ? ~split : split;               // leaf `split` or internal node `split`
     const int right = (split + 1 == last) ? ~(split + 1) : split + 1;
     children[t] = make_int2(left, right);
+    node_range[t] = make_int2(first, last);
     int* par = parent + bl * (2 * size_t(M) - 1);
     par[left >= 0 ? left : (M - 1) + ~left] = i;
     par[right >= 0 ? right : (M - 1) + ~right] = i;
@@ -613,8 +618,9 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
                                                            const T* __restrict__ box_hi, const uint32_t* __restrict__ order,
                                                            const uint32_t* __restrict__ keys, T* __restrict__ node_box,
                                                            T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
-                                                           int2* __restrict__ children, int* __restrict__ parent, int M,
-                                                           size_t total, bool covariance_form) {
+                                                           int2* __restrict__ children, int* __restrict__ parent,
+                                                           int2* __restrict__ node_range, int M, size_t total,
+                                                           bool covariance_form) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
     const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
@@ -657,7 +663,7 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         reinterpret_cast<int*>(r + 10)[0] = comp;
     }
     // the same lane builds internal node `leaf` of the tree (there are M-1 of them); nothing above depends on it
-    if (leaf < M - 1) build_internal_node(keys, children, parent, M, bl, leaf);
+    if (leaf < M - 1) build_internal_node(keys, children, parent, node_range, M, bl, leaf);
 }
 
 // Bottom-up boxes without inter-lane ordering: one lane per leaf walks towards the root and merges ITS OWN leaf
@@ -666,30 +672,74 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
 // therefore walks on itself, so all higher ancestors end up containing the stopped leaf as well: the final boxes
 // are the exact unions of the leaves below each node.  Nothing is read back except the atomics' own return
 // values, so no fences are needed; the decoded boxes are produced by the next kernel.
+// A walk is a chain of atomic round trips, one per tree level.  The lower levels stay inside the workgroup: an
+// internal node whose leaves all belong to the kMergeBlock leaves of this workgroup is touched by these lanes only, so its
+// box lives in LDS while the walks run (internal node i lies inside its own leaf range, hence slot i - first leaf
+// of the workgroup is free for it) and is stored once at the end; only the ancestors that reach beyond the
+// workgroup's leaves are merged with global atomics.
+// leaves per workgroup of the box merge (1024 keep two more tree levels in LDS but occupy too few compute units: slower)
+constexpr int kMergeBlock = 256;
+
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_merge_kernel(const int* __restrict__ parent, const T* __restrict__ node_box,
-                                                          long long* enc_box, int M, size_t total) {
-    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
-    if (t >= total) return;
-    const size_t bl = t / M;
+__global__ __launch_bounds__(kMergeBlock) void bvh_merge_kernel(const int* __restrict__ parent, const int2* __restrict__ node_range,
+                                                          const T* __restrict__ node_box, long long* enc_box, int M,
+                                                          size_t total) {
+    __shared__ long long local_box[kMergeBlock][2 * D];
+    __shared__ int local_parent[kMergeBlock];
+    __shared__ int is_local[kMergeBlock];
+    const size_t first_leaf = size_t(blockIdx.x) * kMergeBlock;          // leaves of all mixtures, numbered through
+    const size_t t = first_leaf + threadIdx.x;
+    const size_t bl = t < total ? t / M : 0;
     const int leaf = int(t - bl * M);
     const size_t nbase = bl * (2 * size_t(M) - 1);
-    const T* box = node_box + (nbase + (M - 1) + leaf) * 2 * D;
-    long long* enc = enc_box + bl * (M - 1) * 2 * D;
-    long long lo[D], hi[D];
-    for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(double(box[d])); hi[d] = ordered_bits(double(box[D + d])); }
-    int node = parent[nbase + (M - 1) + leaf];
-    // the radix tree over 64-bit keys is at most 64 levels deep; the bound also ends a walk on a malformed chain
-    for (int level = 0; node >= 0 && node < M - 1 && level < 128; ++level) {
-        const int up = parent[nbase + node];        // fetched alongside the atomics: one round trip per level
-        bool grew = false;
-        long long* e = enc + size_t(node) * 2 * D;
-        for (int d = 0; d < D; ++d) {
-            grew |= lo[d] < atomicMin(&e[d], lo[d]);
-            grew |= hi[d] > atomicMax(&e[D + d], hi[d]);
+    // lane <-> internal node `leaf` of its mixture (there are M-1 of them)
+    bool mine = false;
+    if (t < total && leaf < M - 1) {
+        const int2 r = node_range[bl * (M - 1) + leaf];
+        const size_t lo = bl * M + r.x, hi = bl * M + r.y;
+        mine = lo >= first_leaf && hi < first_leaf + kMergeBlock && hi < total;
+        local_parent[threadIdx.x] = parent[nbase + leaf];
+    }
+    is_local[threadIdx.x] = mine ? 1 : 0;
+    for (int d = 0; d < D; ++d) {
+        local_box[threadIdx.x][d] = 0x7fffffffffffffffll;           // empty: lower = +inf, upper = -inf
+        local_box[threadIdx.x][D + d] = -0x7fffffffffffffffll - 1;
+    }
+    __syncthreads();
+    if (t < total) {
+        const T* box = node_box + (nbase + (M - 1) + leaf) * 2 * D;
+        long long* enc = enc_box + bl * (M - 1) * 2 * D;
+        long long lo[D], hi[D];
+        for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(double(box[d])); hi[d] = ordered_bits(double(box[D + d])); }
+        int node = parent[nbase + (M - 1) + leaf];
+        // the radix tree over 64-bit keys is at most 64 levels deep; the bound also ends a walk on a malformed chain
+        for (int level = 0; node >= 0 && node < M - 1 && level < 128; ++level) {
+            const long long slot = (long long)(bl * M + node) - (long long)first_leaf;
+            const bool local = slot >= 0 && slot < kMergeBlock && is_local[slot];
+            bool grew = false;
+            int up;
+            if (local) {
+                up = local_parent[slot];
+                for (int d = 0; d < D; ++d) {
+                    grew |= lo[d] < atomicMin(&local_box[slot][d], lo[d]);
+                    grew |= hi[d] > atomicMax(&local_box[slot][D + d], hi[d]);
+                }
+            } else {
+                up = parent[nbase + node];          // fetched alongside the atomics: one round trip per level
+                long long* e = enc + size_t(node) * 2 * D;
+                for (int d = 0; d < D; ++d) {
+                    grew |= lo[d] < atomicMin(&e[d], lo[d]);
+                    grew |= hi[d] > atomicMax(&e[D + d], hi[d]);
+                }
+            }
+            if (!grew) break;
+            node = up;
         }
-        if (!grew) break;
-        node = up;
+    }
+    __syncthreads();
+    if (mine) {
+        long long* e = enc_box + (bl * (M - 1) + leaf) * 2 * D;
+        for (int d = 0; d < 2 * D; ++d) e[d] = local_box[threadIdx.x][d];
     }
 }
 
@@ -873,7 +923,8 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                                      : wave * chunks + (chunk + wave * (chunks / (groups + 1))) % chunks;
         const int j = group * kWave + lane;
         const bool valid = j < N;
-        const int pid = valid ? p_order[xseg * N + j] : 0;
+        int pid = valid ? p_order[xseg * N + j] : 0;
+        pid = unsigned(pid) < unsigned(N) ? pid : 0;        // a permutation by construction; never index out of bounds
         T x[D];
 #pragma unroll
         for (int d = 0; d < D; ++d) x[d] = xes[(xseg * N + pid) * D + d];
@@ -1254,7 +1305,8 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
             const size_t xseg = size_t(b < Bx ? b : Bx - 1) * Lx + (l < Lx ? l : Lx - 1);
             const int j = group * kWave + lane;
             if (j >= N) continue;
-            const int pid = p_order[xseg * N + j];
+            int pid = p_order[xseg * N + j];
+            pid = unsigned(pid) < unsigned(N) ? pid : 0;
             for (int d = 0; d < D; ++d)
                 atomic_add(&grad_xes[(xseg * N + pid) * D + d], piece_gx[(size_t(p) * D + d) * kWave + lane]);
         }
@@ -1389,6 +1441,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     T* box_lo = (T*)(bvh + lay.box_lo); T* box_hi = (T*)(bvh + lay.box_hi);
     T* node_box = (T*)(bvh + lay.node_box); T* leaf_rec = (T*)(bvh + lay.leaf_rec);
     int2* children = (int2*)(bvh + lay.children); int* parent = (int*)(bvh + lay.parent);
+    int2* node_range = (int2*)(bvh + lay.node_range);
     int* leaf_comp = (int*)(bvh + lay.leaf_comp); long long* enc_box = (long long*)(bvh + lay.enc_box);
     uint32_t* ka = (uint32_t*)(bvh + lay.keys_a); uint32_t* kb = (uint32_t*)(bvh + lay.keys_b);
     uint32_t* va = (uint32_t*)(bvh + lay.vals_a); uint32_t* vb = (uint32_t*)(bvh + lay.vals_b);
@@ -1413,12 +1466,15 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm)};
     if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx)};
     if (mg.blocks + mp.blocks > 0) morton_kernel<T, D><<<dim3(mg.blocks + mp.blocks), dim3(kBlock), 0, st>>>(mg, mp);
-    // leaves: all 30 key bits; points: 16 Morton bits (65536 cells) are enough to make 64 consecutive points
-    // neighbours, and their sorted keys are not needed afterwards (they land in a spare buffer)
+    // leaves: all 30 key bits; points: the top 16 Morton bits (65536 cells) are enough to make 64 consecutive
+    // points neighbours, the top 8 bits for segments of at most kCoarseOrderMax points (32 points per cell; measured:
+    // same traversal times, one sort pass less).  The sorted keys of the points are not needed afterwards: they
+    // land in a spare buffer, which must not be the input of the last pass.
+    const int p_passes = N > kCoarseOrderMax ? 2 : 1;
     for (int pass = 0; pass < 4; ++pass) {
         const SortJob jg = sort_job(ka, va, kb, vb, g_keys, g_order, (uint32_t*)(bvh + lay.hist_g), have_g ? BL : 0, M, 0, 4, pass);
-        const SortJob jp = sort_job(pka, pva, pkb, pvb, pka, (uint32_t*)p_order, (uint32_t*)(bvh + lay.hist_p),
-                                    sort_p ? XL : 0, N, 14, 2, pass);
+        const SortJob jp = sort_job(pka, pva, pkb, pvb, p_passes == 1 ? pkb : pka, (uint32_t*)p_order,
+                                    (uint32_t*)(bvh + lay.hist_p), sort_p ? XL : 0, N, 30 - 8 * p_passes, p_passes, pass);
         if (jg.blocks + jp.blocks == 0) continue;
         radix_hist_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
         radix_scatter_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
@@ -1426,11 +1482,12 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     if (have_g) {
         const size_t n = BL * M;
         bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, g_keys,
-                                                                           node_box, leaf_rec, enc_box, children, parent, M, n,
+                                                                           node_box, leaf_rec, enc_box, children, parent, node_range, M, n,
                                                                            cfg.covariance_form != 0);
         if (M > 1) {
             const size_t ni = BL * (M - 1);
-            bvh_merge_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(parent, node_box, enc_box, M, n);
+            bvh_merge_kernel<T, D><<<dim3(unsigned((n + kMergeBlock - 1) / kMergeBlock)), dim3(kMergeBlock), 0, st>>>(
+                parent, node_range, node_box, enc_box, M, n);
             bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(
                 children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups);
         }
