@@ -478,6 +478,7 @@ __global__ __launch_bounds__(kBlock) void radix_hist_kernel(SortJob a, SortJob b
 __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJob b) {
     __shared__ uint32_t running[256];        // next output slot of every digit for this block
     __shared__ uint32_t wave_count[4][256];
+    __shared__ uint32_t wave_total[4];
     const bool first = blockIdx.x < a.blocks;
     const SortJob& j = first ? a : b;
     const unsigned id = first ? blockIdx.x : blockIdx.x - a.blocks;
@@ -486,11 +487,27 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJo
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     // thread d: keys of digit d in the whole segment and in the blocks before this one (at most kSortBlocksMax
     // counts per digit, so no separate scan pass is needed)
+    const size_t seg_off = size_t(seg) * count;
+    const int begin = blk * j.items * kBlock;
+    // the keys of the first round are fetched while the histogram columns are summed
+    uint32_t next_key = 0, next_val = 0;
+    if (begin + int(threadIdx.x) < count) {
+        next_key = j.keys_in[seg_off + begin + threadIdx.x];
+        next_val = j.vals_in[seg_off + begin + threadIdx.x];
+    }
     uint32_t mine = 0, earlier = 0;
     {
         const uint32_t* col = j.hist + size_t(seg) * blocks_per_seg * 256 + threadIdx.x;
+        // the loop is latency-bound: groups of 32, then of 8 independent loads in flight
         int q0 = 0;
-        for (; q0 + 8 <= blocks_per_seg; q0 += 8) {         // eight independent loads in flight
+        for (; q0 + 32 <= blocks_per_seg; q0 += 32) {
+            uint32_t c[32];
+#pragma unroll
+            for (int q = 0; q < 32; ++q) c[q] = col[size_t(q0 + q) * 256];
+#pragma unroll
+            for (int q = 0; q < 32; ++q) { mine += c[q]; earlier += q0 + q < blk ? c[q] : 0u; }
+        }
+        for (; q0 + 8 <= blocks_per_seg; q0 += 8) {
             uint32_t c[8];
 #pragma unroll
             for (int q = 0; q < 8; ++q) c[q] = col[size_t(q0 + q) * 256];
@@ -503,26 +520,30 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJo
             earlier += q0 < blk ? c : 0u;
         }
     }
-    // exclusive scan of the segment's digit totals (Hillis-Steele on LDS) = first slot of every digit
-    running[threadIdx.x] = mine;
+    // exclusive scan of the segment's digit totals = first slot of every digit: inclusive scan inside each
+    // wavefront, then the totals of the wavefronts before
+    uint32_t scan = mine;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const uint32_t up = __shfl_up(scan, off, kWave);
+        scan += lane >= off ? up : 0u;
+    }
+    if (lane == kWave - 1) wave_total[wave] = scan;
 #pragma unroll
     for (int w = 0; w < 4; ++w) wave_count[w][threadIdx.x] = 0;
     __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {
-        const uint32_t add = int(threadIdx.x) >= off ? running[threadIdx.x - off] : 0u;
-        __syncthreads();
-        running[threadIdx.x] += add;
-        __syncthreads();
-    }
-    running[threadIdx.x] += earlier - mine;
+    for (int w = 0; w < wave; ++w) scan += wave_total[w];
+    running[threadIdx.x] = scan - mine + earlier;
     __syncthreads();
-    const size_t seg_off = size_t(seg) * count;
-    const int begin = blk * j.items * kBlock;
     for (int round = 0; round < j.items; ++round) {
         const int i = begin + round * kBlock + threadIdx.x;
         const bool valid = i < count;
-        uint32_t key = 0, val = 0, digit = 0;
-        if (valid) { key = j.keys_in[seg_off + i]; val = j.vals_in[seg_off + i]; digit = (key >> shift) & 255u; }
+        const uint32_t key = next_key, val = next_val;
+        const uint32_t digit = valid ? (key >> shift) & 255u : 0u;
+        if (round + 1 < j.items && i + kBlock < count) {
+            next_key = j.keys_in[seg_off + i + kBlock];
+            next_val = j.vals_in[seg_off + i + kBlock];
+        }
         // lanes of this wavefront holding the same digit
         unsigned long long same = __ballot(valid);
 #pragma unroll
@@ -623,10 +644,20 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
                                                            bool covariance_form) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
-    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    // The records of the leaves and the internal nodes of the tree do not depend on each other, and both are
+    // short chains of dependent memory reads: the first half of the grid writes the records, the second half
+    // builds the nodes, side by side on different compute units.
+    const unsigned half = gridDim.x / 2;
+    const bool tree_job = blockIdx.x >= half;
+    const size_t i = size_t(tree_job ? blockIdx.x - half : blockIdx.x) * kBlock + threadIdx.x;
     if (i >= total) return;
     const size_t bl = i / M;
     const int leaf = int(i - bl * M);
+    if (tree_job) {
+        // lane <-> internal node `leaf` of its mixture (there are M-1 of them)
+        if (leaf < M - 1) build_internal_node(keys, children, parent, node_range, M, bl, leaf);
+        return;
+    }
     int comp = int(order[i]);
     comp = (comp >= 0 && comp < M) ? comp : 0;      // a permutation by construction; never index out of bounds
     const size_t gi = bl * M + comp;
@@ -662,8 +693,6 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         r[9] = T(double(g[0]) * Kappa<3>::v * sqrt(det));
         reinterpret_cast<int*>(r + 10)[0] = comp;
     }
-    // the same lane builds internal node `leaf` of the tree (there are M-1 of them); nothing above depends on it
-    if (leaf < M - 1) build_internal_node(keys, children, parent, node_range, M, bl, leaf);
 }
 
 // Bottom-up boxes without inter-lane ordering: one lane per leaf walks towards the root and merges ITS OWN leaf
@@ -1481,7 +1510,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     }
     if (have_g) {
         const size_t n = BL * M;
-        bvh_leaves_kernel<T, D><<<dim3(grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, g_keys,
+        bvh_leaves_kernel<T, D><<<dim3(2 * grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, g_keys,
                                                                            node_box, leaf_rec, enc_box, children, parent, node_range, M, n,
                                                                            cfg.covariance_form != 0);
         if (M > 1) {
