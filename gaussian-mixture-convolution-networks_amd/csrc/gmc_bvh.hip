@@ -1317,28 +1317,30 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
                                                                  bool covariance_form, CandidateCache cache,
                                                                  const T* __restrict__ piece_gx,
                                                                  const int* __restrict__ p_order, T* __restrict__ grad_xes,
-                                                                 int L, int N, int Bx, int Lx) {
+                                                                 unsigned gaussian_blocks, int L, int N, int Bx, int Lx) {
     constexpr int G = 1 + D + D * D;
     constexpr int NR = BvhSums<D>::k;
-    // dL/dx of the pieces that helper workgroups of the traversal worked on: one wavefront per piece, added to
-    // what the owners of the point groups have stored (several pieces of a group meet here, hence atomics)
-    if (cache.count) {
+    // Workgroups behind the first `gaussian_blocks`: dL/dx of the pieces that helper workgroups of the traversal
+    // worked on, one wavefront per piece, added to what the owners of the point groups have stored (several
+    // pieces of a group meet here, hence atomics).
+    if (blockIdx.x >= gaussian_blocks) {
         const int published = cache.ctl[0] < cache.pieces_max ? cache.ctl[0] : cache.pieces_max;
         const int per_mixture = (N + kWave - 1) / kWave;
         const int lane = threadIdx.x & 63;
-        for (int p = blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6); p < published; p += gridDim.x * (kBlock / kWave)) {
-            const int4 desc = cache.pieces[p];
-            if (desc.z <= 0) continue;
-            const int bl = desc.x / per_mixture, group = desc.x - bl * per_mixture;
-            const int b = bl / L, l = bl - b * L;
-            const size_t xseg = size_t(b < Bx ? b : Bx - 1) * Lx + (l < Lx ? l : Lx - 1);
-            const int j = group * kWave + lane;
-            if (j >= N) continue;
-            int pid = p_order[xseg * N + j];
-            pid = unsigned(pid) < unsigned(N) ? pid : 0;
-            for (int d = 0; d < D; ++d)
-                atomic_add(&grad_xes[(xseg * N + pid) * D + d], piece_gx[(size_t(p) * D + d) * kWave + lane]);
-        }
+        const int p = int(blockIdx.x - gaussian_blocks) * (kBlock / kWave) + int(threadIdx.x >> 6);
+        if (p >= published) return;
+        const int4 desc = cache.pieces[p];
+        if (desc.z <= 0) return;
+        const int bl = desc.x / per_mixture, group = desc.x - bl * per_mixture;
+        const int b = bl / L, l = bl - b * L;
+        const size_t xseg = size_t(b < Bx ? b : Bx - 1) * Lx + (l < Lx ? l : Lx - 1);
+        const int j = group * kWave + lane;
+        if (j >= N) return;
+        int pid = p_order[xseg * N + j];
+        pid = unsigned(pid) < unsigned(N) ? pid : 0;
+        for (int d = 0; d < D; ++d)
+            atomic_add(&grad_xes[(xseg * N + pid) * D + d], piece_gx[(size_t(p) * D + d) * kWave + lane]);
+        return;
     }
     const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
     if (i >= n) return;
@@ -1592,10 +1594,11 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bv
 #undef GMC_TRAV
     const bool pieces_gx = gx && helpers > 0;
     if (gm || pieces_gx) {
-        const unsigned blocks = gm ? grid_for(n_g) : unsigned((helpers + 3) / 4);
-        bvh_bwd_epilogue_kernel<T, D><<<dim3(blocks), dim3(kBlock), 0, st>>>(
-            mixture, sums, grad_mixture, gm ? n_g : 0, covariance_form, pieces_gx ? cache : CandidateCache{}, piece_gx,
-            (const int*)(bvh + lay.p_order), grad_xes, s.L, s.N, s.Bx, s.Lx);
+        const unsigned gaussian_blocks = gm ? grid_for(n_g) : 0u;
+        const unsigned piece_blocks = pieces_gx ? unsigned((helpers + kBlock / kWave - 1) / (kBlock / kWave)) : 0u;
+        bvh_bwd_epilogue_kernel<T, D><<<dim3(gaussian_blocks + piece_blocks), dim3(kBlock), 0, st>>>(
+            mixture, sums, grad_mixture, n_g, covariance_form, cache, piece_gx, (const int*)(bvh + lay.p_order), grad_xes,
+            gaussian_blocks, s.L, s.N, s.Bx, s.Lx);
     }
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
