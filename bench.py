@@ -38,14 +38,14 @@ MEASURED_TRAFFIC_BYTES = {"C4": 157960 * 1024 * 2.0 + 524288 * 1024 * 1.0,
                           "C5_fwd": 21532.1 * 1024 * 2.0 + 4092.3 * 1024 * 1.0}
 
 
-def cpu_baseline(name: str, seconds_budget: float = 20.0):
+def cpu_baseline(name: str):
     """Times oracle/libcpu_ref.so (checker code, used here only as the reported CPU baseline)."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import cpu_ref
     from gmc import synthetic
     base = synthetic.WORKLOADS[name]
-    # bounded sample of the same distributions: one batch entry, a few layers
-    kw = dict(B=1) if name != "C5" else dict(N=2000)
+    # bounded sample of the same distributions (about 10 s of CPU work at C4): four batch entries
+    kw = dict(B=4) if name != "C5" else dict(N=2000)
     wl, mix, xes, gout = synthetic.make_workload(name, **kw)
     m, x, g = mix.numpy(), xes.numpy(), gout.numpy()
     threads = 128                                    # the reference's own choice (parallel_start.h:94-99)
@@ -147,26 +147,30 @@ def bench_bvh(args):
 
 def cpu_baseline_bvh(mode: str):
     """CPU comparison for the culled path: the C restatement of the reference CPU loops with the per-pair box
-    test in front of each evaluation (the reference has no CPU BVH evaluator to restate), on 20000 query
-    points of the C5 distribution with the boxes of the oracle's rule."""
+    test in front of each evaluation (the reference has no CPU BVH evaluator to restate), on the whole C5
+    workload with the boxes of the oracle's rule, five repetitions."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import cpu_ref
     import gm_oracle
     from gmc import synthetic
-    wl, mix, xes, gout = synthetic.make_workload("C5", N=20000)
+    wl, mix, xes, gout = synthetic.make_workload("C5")
     m, x, g = mix.numpy(), xes.numpy(), gout.numpy()
     lo, up = gm_oracle.gaussian_aabbs(m, mode=mode)
     threads, cores = 128, len(os.sched_getaffinity(0))
+    reps = 5
+    cpu_ref.forward(m, x[:, :, :2000], lo, up, n_threads=threads)        # warm-up (thread pool, page faults)
     t0 = time.perf_counter()
-    cpu_ref.forward(m, x, lo, up, n_threads=threads)
-    t_fwd = time.perf_counter() - t0
+    for _ in range(reps):
+        cpu_ref.forward(m, x, lo, up, n_threads=threads)
+    t_fwd = (time.perf_counter() - t0) / reps
     t0 = time.perf_counter()
-    cpu_ref.backward(g, m, x, lo, up, n_threads=threads)
-    t_bwd = time.perf_counter() - t0
+    for _ in range(reps):
+        cpu_ref.backward(g, m, x, lo, up, n_threads=threads)
+    t_bwd = (time.perf_counter() - t0) / reps
     return {"value": wl.pairs / (t_fwd + t_bwd), "unit": "dense-equivalent pairs/s (fwd+bwd)", "cores": cores,
             "threads": threads, "kind": "port",
-            "sample": f"C5 slice N=20000 of 100000 points, M=16384 ({wl.pairs:.3g} dense-equivalent pairs), brute-force "
-                      f"box test per pair, fwd {t_fwd:.2f} s + bwd {t_bwd:.2f} s"}
+            "sample": f"the whole C5 workload, {reps} repetitions (M=16384, N=100000: {wl.pairs:.3g} dense-equivalent pairs "
+                      f"each), brute-force box test per pair, fwd {t_fwd:.2f} s + bwd {t_bwd:.2f} s per repetition"}
 
 
 def bench_convolution(args):
