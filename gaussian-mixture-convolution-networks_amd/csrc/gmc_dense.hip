@@ -100,36 +100,43 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
         T rs[NR];
 #pragma unroll
         for (int i = 0; i < NR; ++i) rs[i] = T(0);
+        // dL/dx takes the products k*y against amp*u (formed once per Gaussian), the sums take them against y.
+        // With the sums wanted k = e*g (g: upstream gradient of the point), so that the same three products serve
+        // both; the dL/dx accumulators then hold g * (sum over Gaussians) and the kernel's last step must not
+        // multiply by g again.  With dL/dx alone k = e.
+        T ua[Rec<T, D>::kU];
+        if (NEED_GX) {
+#pragma unroll
+            for (int i = 0; i < Rec<T, D>::kU; ++i) ua[i] = r[Rec<T, D>::kAmp] * r[i];
+        }
 #pragma unroll
         for (int p = 0; p < P; ++p) {
             T y[D];
             const T q = quad_form<T, D, CENTRED>(r, x[p], y);
             const T e = fast_exp2(-q);
+            const T k = NEED_GM ? e * go[p] : e;
+            T ky[D];
+#pragma unroll
+            for (int d = 0; d < D; ++d) ky[d] = k * y[d];
             if (NEED_GX) {
-                const T s = r[Rec<T, D>::kAmp] * e;
                 if constexpr (D == 2) {
-                    const T sy0 = s * y[0], sy1 = s * y[1];
-                    gx[p][0] = fma_(r[0], sy0, gx[p][0]);
-                    gx[p][1] = fma_(r[1], sy0, fma_(r[2], sy1, gx[p][1]));
+                    gx[p][0] = fma_(ua[0], ky[0], gx[p][0]);
+                    gx[p][1] = fma_(ua[1], ky[0], fma_(ua[2], ky[1], gx[p][1]));
                 } else {
-                    const T sy0 = s * y[0], sy1 = s * y[1], sy2 = s * y[2];
-                    gx[p][0] = fma_(r[0], sy0, gx[p][0]);
-                    gx[p][1] = fma_(r[1], sy0, fma_(r[3], sy1, gx[p][1]));
-                    gx[p][2] = fma_(r[2], sy0, fma_(r[4], sy1, fma_(r[5], sy2, gx[p][2])));
+                    gx[p][0] = fma_(ua[0], ky[0], gx[p][0]);
+                    gx[p][1] = fma_(ua[1], ky[0], fma_(ua[3], ky[1], gx[p][1]));
+                    gx[p][2] = fma_(ua[2], ky[0], fma_(ua[4], ky[1], fma_(ua[5], ky[2], gx[p][2])));
                 }
             }
             if (NEED_GM) {
-                const T eg = e * go[p];
-                rs[0] += eg;
+                rs[0] += k;
                 if constexpr (D == 2) {
-                    const T a0 = eg * y[0], a1 = eg * y[1];
-                    rs[1] += a0; rs[2] += a1;
-                    rs[3] = fma_(a0, y[0], rs[3]); rs[4] = fma_(a0, y[1], rs[4]); rs[5] = fma_(a1, y[1], rs[5]);
+                    rs[1] += ky[0]; rs[2] += ky[1];
+                    rs[3] = fma_(ky[0], y[0], rs[3]); rs[4] = fma_(ky[0], y[1], rs[4]); rs[5] = fma_(ky[1], y[1], rs[5]);
                 } else {
-                    const T a0 = eg * y[0], a1 = eg * y[1], a2 = eg * y[2];
-                    rs[1] += a0; rs[2] += a1; rs[3] += a2;
-                    rs[4] = fma_(a0, y[0], rs[4]); rs[5] = fma_(a0, y[1], rs[5]); rs[6] = fma_(a0, y[2], rs[6]);
-                    rs[7] = fma_(a1, y[1], rs[7]); rs[8] = fma_(a1, y[2], rs[8]); rs[9] = fma_(a2, y[2], rs[9]);
+                    rs[1] += ky[0]; rs[2] += ky[1]; rs[3] += ky[2];
+                    rs[4] = fma_(ky[0], y[0], rs[4]); rs[5] = fma_(ky[0], y[1], rs[5]); rs[6] = fma_(ky[0], y[2], rs[6]);
+                    rs[7] = fma_(ky[1], y[1], rs[7]); rs[8] = fma_(ky[1], y[2], rs[8]); rs[9] = fma_(ky[2], y[2], rs[9]);
                 }
             }
         }
@@ -225,7 +232,8 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_rc_kernel(const T* __restrict
                     T* dst = grad_xes + (x_off + n) * D;
 #pragma unroll
                     for (int d = 0; d < D; ++d) {
-                        const T v = -go[p] * gx[p][d];
+                        // with both gradients the pair loop has folded the upstream gradient into the sum
+                        const T v = (NEED_GM && NEED_GX) ? -gx[p][d] : -go[p] * gx[p][d];
                         if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
                     }
                 }
