@@ -98,8 +98,6 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
 #pragma unroll
         for (int i = 0; i < Rec<T, D>::kUsed; ++i) r[i] = lds[g * S + i];
         T rs[NR];
-#pragma unroll
-        for (int i = 0; i < NR; ++i) rs[i] = T(0);
         // dL/dx takes the products k*y against amp*u (formed once per Gaussian), the sums take them against y.
         // With the sums wanted k = e*g (g: upstream gradient of the point), so that the same three products serve
         // both; the dL/dx accumulators then hold g * (sum over Gaussians) and the kernel's last step must not
@@ -129,20 +127,37 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
                 }
             }
             if (NEED_GM) {
-                rs[0] += k;
-                if constexpr (D == 2) {
-                    rs[1] += ky[0]; rs[2] += ky[1];
-                    rs[3] = fma_(ky[0], y[0], rs[3]); rs[4] = fma_(ky[0], y[1], rs[4]); rs[5] = fma_(ky[1], y[1], rs[5]);
+                if (p == 0) {
+                    // the first point starts the sums (no zero fill, no additions)
+                    rs[0] = k;
+#pragma unroll
+                    for (int d = 0; d < D; ++d) rs[1 + d] = ky[d];
+                    int at = 1 + D;
+#pragma unroll
+                    for (int a = 0; a < D; ++a)
+#pragma unroll
+                        for (int c = a; c < D; ++c) rs[at++] = ky[a] * y[c];
                 } else {
-                    rs[1] += ky[0]; rs[2] += ky[1]; rs[3] += ky[2];
-                    rs[4] = fma_(ky[0], y[0], rs[4]); rs[5] = fma_(ky[0], y[1], rs[5]); rs[6] = fma_(ky[0], y[2], rs[6]);
-                    rs[7] = fma_(ky[1], y[1], rs[7]); rs[8] = fma_(ky[1], y[2], rs[8]); rs[9] = fma_(ky[2], y[2], rs[9]);
+                    rs[0] += k;
+                    if constexpr (D == 2) {
+                        rs[1] += ky[0]; rs[2] += ky[1];
+                        rs[3] = fma_(ky[0], y[0], rs[3]); rs[4] = fma_(ky[0], y[1], rs[4]); rs[5] = fma_(ky[1], y[1], rs[5]);
+                    } else {
+                        rs[1] += ky[0]; rs[2] += ky[1]; rs[3] += ky[2];
+                        rs[4] = fma_(ky[0], y[0], rs[4]); rs[5] = fma_(ky[0], y[1], rs[5]); rs[6] = fma_(ky[0], y[2], rs[6]);
+                        rs[7] = fma_(ky[1], y[1], rs[7]); rs[8] = fma_(ky[1], y[2], rs[8]); rs[9] = fma_(ky[2], y[2], rs[9]);
+                    }
                 }
             }
         }
         if (NEED_GM) {
 #pragma unroll
-            for (int i = 0; i < NR; ++i) rs[i] = row_sum_to_lane15(rs[i]);
+            for (int i = 0; i < NR; ++i) {
+                rs[i] = row_sum_to_lane15(rs[i]);
+                // keeps the last addition in front of the branch below, where it stays one DPP instruction (sunk
+                // into the branch it becomes a zero fill, a DPP move and an addition)
+                asm volatile("" : "+v"(rs[i]));
+            }
             if ((threadIdx.x & 15) == 15) {
                 const int idx = record_index<T, D>(lds + g * S);
                 if (idx >= 0) {
