@@ -436,11 +436,13 @@ static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T
     // A workgroup covers 4 wavefronts x 16 P points.  Larger P amortises the per-Gaussian row reductions (about
     // 4 (1 + D + D(D+1)/2) instructions per step and lane) over more pairs but pads the last chunk more; pick the P
     // with the least modelled work that still leaves enough workgroups for the 256 CUs.
-    const int p_max = sizeof(T) == 8 ? 8 : 16;
-    const double pair_cost = D == 2 ? 21.0 : 34.0, reduce_cost = 4.0 * Sums<D>::k;
+    // Every P from 2 to 16 (8 in double) has its instance: with powers of two only, 784 points (a 28 x 28 grid) ran
+    // as one chunk of 1024 with 23 % of the lanes' points padding; P = 13 covers them with 832.
+    constexpr int p_max = sizeof(T) == 8 ? 8 : 16;
+    const double pair_cost = D == 2 ? 18.0 : 30.0, reduce_cost = 5.0 * Sums<D>::k;
     int P = 2;
     double best = 1e300;
-    for (int cand = p_max; cand >= 2; cand >>= 1) {
+    for (int cand = p_max; cand >= 2; --cand) {
         const int span = 64 * cand;
         const size_t chunks = (size_t(s.N) + span - 1) / span;
         if (cand > 2 && chunks * BL < 256) continue;
@@ -451,10 +453,26 @@ static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T
     const int chunks = (s.N + span - 1) / span;
     const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
 #define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL), cov)
+    if constexpr (p_max > 8) {
+        switch (P) {
+            case 16: GMC_BWD(16); return;
+            case 15: GMC_BWD(15); return;
+            case 14: GMC_BWD(14); return;
+            case 13: GMC_BWD(13); return;
+            case 12: GMC_BWD(12); return;
+            case 11: GMC_BWD(11); return;
+            case 10: GMC_BWD(10); return;
+            case 9: GMC_BWD(9); return;
+            default: break;
+        }
+    }
     switch (P) {
-        case 16: GMC_BWD(16); break;
         case 8: GMC_BWD(8); break;
+        case 7: GMC_BWD(7); break;
+        case 6: GMC_BWD(6); break;
+        case 5: GMC_BWD(5); break;
         case 4: GMC_BWD(4); break;
+        case 3: GMC_BWD(3); break;
         default: GMC_BWD(2); break;
     }
 #undef GMC_BWD
