@@ -177,7 +177,7 @@ def bench_convolution(args):
     """Closed-form convolution on a layer-sized problem (2-D, float32, batch 100, 8 -> 16 channels, 128 data and 5
     kernel components per channel: 8.2e6 output Gaussians, 229 MB).  A step is forward plus backward (both
     gradients).  The path is streaming: the unit is output Gaussians per second and the roofline is HBM with the
-    compulsory bytes (forward: operands in, result out; backward: grad_out is read once per gradient)."""
+    compulsory bytes (forward: operands in, result out; backward: grad_out once, operands in, gradients out)."""
     import torch
     from gmc import _native
     from gmc import mixture as gm
@@ -222,7 +222,7 @@ def bench_convolution(args):
     fwd_ms, bwd_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(2))
     small = (data.numel() + kernels.numel()) * 4
     bytes_fwd = n_out * G * 4 + small
-    bytes_bwd = 2 * n_out * G * 4 + 3 * small
+    bytes_bwd = n_out * G * 4 + 2 * small                    # grad_out once; operands in, gradients out
     line = {
         "metric": "closed-form mixture convolution, output Gaussians per second (forward + backward step)",
         "value": n_out / (ms_step * 1e-3), "unit": "output Gaussians/s (forward + backward step)",
@@ -231,7 +231,7 @@ def bench_convolution(args):
         "config": {"workload": f"conv: D={D} f32 data [{B},{Cin},{Nd}] * kernels [{Cout},{Cin},{Nk}] -> "
                                f"[{B},{Cout},{Nd * Cin * Nk}], {n_out:.4g} output Gaussians per step"},
         "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
-        "roofline": {"kernel": "conv_bwd_data_kernel + conv_bwd_kernels_kernel (one event pair)", "bound": "hbm",
+        "roofline": {"kernel": "conv_bwd_fused_kernel (with the zero fill of grad_kernels in the event pair)", "bound": "hbm",
                      "achieved": bytes_bwd / (bwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
                      "frac": bytes_bwd / (bwd_ms * 1e-3) / 8e12, "traffic": None, "launch_ms": bwd_ms,
                      "algorithmic_bytes": bytes_bwd},

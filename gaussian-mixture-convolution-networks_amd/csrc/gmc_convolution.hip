@@ -118,6 +118,133 @@ __global__ __launch_bounds__(kBlock) void conv_bwd_kernels_kernel(const T* __res
     }
 }
 
+// Both gradients from ONE pass over grad_out (the two kernels above read it once each).  A workgroup owns 64 data
+// Gaussians cd of one (b, ci) -- a lane per Gaussian -- and its four wavefronts share the Cout Nk runs of grad_out
+// that were built from them (each run is Nd G contiguous scalars; wavefront w takes the runs w, w + 4, ...).  A
+// wavefront fetches the 64 G scalars of a run with coalesced loads (kConvDepth of its runs ahead of the one it works
+// on: the walk is bound by memory latency and instruction issue, hence many wavefronts with several loads in
+// flight each), turns them into one Gaussian per lane through its own LDS staging area (odd stride G: no bank
+// conflicts), adds them to its grad_data registers and reduces the grad_kernels terms over the wavefront (DPP) into
+// the workgroup's LDS copy of grad_kernels[:, ci, :].  At the end the four partial grad_data are added through LDS
+// and stored once (no atomics), and the copy goes out with one atomic per scalar and workgroup, so only
+// B * chunks additions meet on an address.
+constexpr int kConvWaves = 4;
+constexpr int kConvBlock = kConvWaves * kWave;
+constexpr int kConvDepth = 4;
+
+__device__ __forceinline__ void conv_wave_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <typename T, int D, bool NEED_DATA, bool NEED_KERNELS>
+__global__ __launch_bounds__(kConvBlock) void conv_bwd_fused_kernel(const T* __restrict__ grad_out, const T* __restrict__ data,
+                                                                   const T* __restrict__ kernels, T* __restrict__ grad_data,
+                                                                   T* __restrict__ grad_kernels, ConvDims n, int chunks) {
+    constexpr int G = 1 + D + D * D;
+    __shared__ T stage[kConvWaves][kWave * G];
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv_dynamic_lds[];
+    const int terms = n.Cout * n.Nk;
+    T* sums = reinterpret_cast<T*>(conv_dynamic_lds);               // [terms][G] sums of this workgroup for grad_kernels
+    T* kernel_weight = sums + size_t(terms) * G;                    // [terms]    weights of kernels[:, ci, :]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int bc = blockIdx.x / chunks, chunk = blockIdx.x - bc * chunks;
+    const int b = bc / n.Cin, ci = bc - b * n.Cin;
+    for (int i = threadIdx.x; i < terms; i += kConvBlock) {
+        const int co = i / n.Nk, k = i - co * n.Nk;
+        kernel_weight[i] = kernels[((size_t(co) * n.Cin + ci) * n.Nk + k) * G];
+    }
+    __syncthreads();
+    const int cd0 = chunk * kWave;
+    const int count = n.Nd - cd0 < kWave ? n.Nd - cd0 : kWave;      // Gaussians of this workgroup, > 0
+    const int scalars = count * G;
+    const size_t per_b = size_t(n.Nd) * G * n.Cin;                  // scalars of one (b, co, k)
+    const size_t slab = per_b * n.Nk;                               // scalars of one (b, co)
+    const T* __restrict__ base = grad_out + size_t(b) * n.Cout * slab + (size_t(ci) * n.Nd + cd0) * G;
+    const T data_weight = lane < count ? data[((size_t(b) * n.Cin + ci) * n.Nd + cd0 + lane) * G] : T(0);
+    T* mine = stage[wave];
+    T acc[G];
+#pragma unroll
+    for (int el = 0; el < G; ++el) acc[el] = T(0);
+    // run i = (co, k) in flattened order; the fetches run kConvDepth of this wavefront's runs ahead
+    int fetch_i = wave, fetch_co = wave / n.Nk, fetch_k = wave - fetch_co * n.Nk;
+    auto fetch = [&](T (&v)[G]) {
+        if (fetch_i < terms) {
+            const T* __restrict__ src = base + size_t(fetch_co) * slab + size_t(fetch_k) * per_b;
+            // scalars beyond the workgroup's Gaussians are read from its first one (no branches) and zeroed when the
+            // run is worked on: nothing here may wait for the loads
+#pragma unroll
+            for (int r = 0; r < G; ++r) {
+                const int idx = lane + r * kWave;
+                v[r] = src[idx < scalars ? idx : 0];
+            }
+        }
+        fetch_i += kConvWaves;
+        fetch_k += kConvWaves;
+        while (fetch_k >= n.Nk) { fetch_k -= n.Nk; ++fetch_co; }
+    };
+    auto work = [&](int i, const T (&v)[G]) {
+#pragma unroll
+        for (int r = 0; r < G; ++r) mine[lane + r * kWave] = lane + r * kWave < scalars ? v[r] : T(0);
+        conv_wave_fence();
+        T g[G];
+#pragma unroll
+        for (int el = 0; el < G; ++el) g[el] = mine[lane * G + el];
+        conv_wave_fence();
+        if (NEED_DATA) {
+            acc[0] = fma_(g[0], kernel_weight[i], acc[0]);
+#pragma unroll
+            for (int el = 1; el < G; ++el) acc[el] += g[el];
+        }
+        if (NEED_KERNELS) {
+            g[0] *= data_weight;
+#pragma unroll
+            for (int el = 0; el < G; ++el) g[el] = wave_sum_to_lane63(g[el]);
+            if (lane == kWave - 1) {
+                // plain stores: every run belongs to one wavefront
+#pragma unroll
+                for (int el = 0; el < G; ++el) sums[i * G + el] = g[el];
+            }
+        }
+    };
+    T v[kConvDepth][G];
+#pragma unroll
+    for (int q = 0; q < kConvDepth; ++q) fetch(v[q]);
+    for (int i = wave; i < terms; i += kConvDepth * kConvWaves) {
+#pragma unroll
+        for (int q = 0; q < kConvDepth; ++q) {
+            if (i + q * kConvWaves < terms) {
+                work(i + q * kConvWaves, v[q]);
+                fetch(v[q]);
+            }
+        }
+    }
+    if (NEED_DATA) {
+#pragma unroll
+        for (int el = 0; el < G; ++el) mine[lane * G + el] = acc[el];
+    }
+    __syncthreads();
+    if (NEED_DATA && wave == 0) {
+        T* __restrict__ dst = grad_data + ((size_t(b) * n.Cin + ci) * n.Nd + cd0) * G;
+#pragma unroll
+        for (int r = 0; r < G; ++r) {
+            const int idx = lane + r * kWave;
+            T total = T(0);
+#pragma unroll
+            for (int w = 0; w < kConvWaves; ++w) total += stage[w][idx];
+            if (idx < scalars) dst[idx] = total;
+        }
+    }
+    if (NEED_KERNELS) {
+        for (int idx = threadIdx.x; idx < terms * G; idx += kConvBlock) {
+            const int i = idx / G, el = idx - i * G;
+            const int co = i / n.Nk, k = i - co * n.Nk;
+            atomic_add(&grad_kernels[((size_t(co) * n.Cin + ci) * n.Nk + k) * G + el], sums[idx]);
+        }
+    }
+}
+
 template <typename T, int D>
 static int conv_forward_t(const T* data, const T* kernels, T* out, const ConvDims& n, hipStream_t st) {
     constexpr int G = 1 + D + D * D;
@@ -142,6 +269,16 @@ static int conv_backward_t(const T* grad_out, const T* data, const T* kernels, T
     constexpr int G = 1 + D + D * D;
     const size_t n_data = size_t(n.B) * n.Cin * n.Nd * G, n_kern = size_t(n.Cout) * n.Cin * n.Nk * G;
     const bool empty_sum = n.Cout == 0 || n.Nk == 0 || n.B == 0 || n.Nd == 0 || n.Cin == 0;
+    // both gradients: one pass over grad_out, as long as the workgroup's copy of grad_kernels[:, ci, :] fits in LDS
+    const size_t fused_lds = (size_t(n.Cout) * n.Nk * (G + 1)) * sizeof(T);
+    if (need_data && need_kernels && !empty_sum && fused_lds <= size_t(32) << 10) {
+        const int chunks = (n.Nd + kWave - 1) / kWave;
+        if (size_t(n.B) * n.Cin * chunks > 0x7fffffffull) return GMC_E_SHAPE;
+        zero_async(grad_kernels, n_kern, st);
+        conv_bwd_fused_kernel<T, D, true, true><<<dim3(unsigned(n.B) * n.Cin * chunks), dim3(kConvBlock), fused_lds, st>>>(
+            grad_out, data, kernels, grad_data, grad_kernels, n, chunks);
+        return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+    }
     if (need_data && n_data > 0) {
         if (empty_sum) zero_async(grad_data, n_data, st);
         else {
