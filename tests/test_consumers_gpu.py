@@ -28,8 +28,10 @@ def _cov_mixture(rng, B, L, M, D, cov=0.5):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("dims", [(3, 5, 7, 2, 4, 2), (2, 3, 1, 4, 1, 3), (1, 1, 300, 1, 5, 3), (5, 8, 33, 16, 5, 2),
-                                  (70, 2, 9, 3, 2, 3), (700, 1, 2, 100, 1, 2)])
+                                  (70, 2, 9, 3, 2, 3), (700, 1, 2, 100, 1, 2), (2, 3, 130, 64, 9, 3)])
 def test_convolution_forward_backward(dims, dtype):
+    """(B, Cin, Nd, Cout, Nk, D); the last case has 576 kernel Gaussians per input channel: in float32 their sums
+    just fit the fused backward kernel's LDS copy, in float64 they do not and the two single-gradient kernels run"""
     B, Cin, Nd, Cout, Nk, D = dims
     rng = np.random.default_rng(sum(dims))
     npdt = np.float32 if dtype == torch.float32 else np.float64
