@@ -93,6 +93,17 @@ def test_tile_and_chunk_boundaries(dtype, D):
     _check(mix, xes, gout, dtype, tag="broadcast large")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_every_points_per_lane_instance(dtype):
+    """The backward pair kernel has one instance per number of points per lane, 2 to 16 (8 in float64), chosen from
+    the point count: with 256 mixtures a launch takes one chunk of 64 p points whenever that covers N, so N = 64 p - 3
+    runs instance p (ragged last lanes included)."""
+    for p in range(2, 17 if dtype == torch.float32 else 9):
+        D = 2 + p % 2
+        mix, xes, gout = _case(16, 16, 5, 64 * p - 3, D, 8000 + p, p % 4 == 0)
+        _check(mix, xes, gout, dtype, tag=f"points per lane {p}, D{D}")
+
+
 @pytest.mark.parametrize("D", [2, 3])
 def test_matrix_core_forward_shapes(D):
     """float32 shapes that take the wide matrix-core forward kernel (more than 128 components and either many
