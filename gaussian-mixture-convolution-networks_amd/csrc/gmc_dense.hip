@@ -84,6 +84,75 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
     }
 }
 
+// Forward pair kernel in the "4 x 16" wavefront layout of the backward kernel below (row r of a wavefront works on
+// Gaussian 4k + r in step k, column c on the points {c, c + 16, ...} of the wavefront's 16 P points): a workgroup
+// covers 64 P points for any P from 2 to 16, where the kernel above covers 256 P with P a power of two.  Used when
+// that pads the last chunk less (784 points: 832 instead of 1024).
+template <typename T, int D, int P, bool CENTRED>
+__device__ __forceinline__ void fwd_rc_pairs(const T* __restrict__ lds, int begin, int end, int row, const T (&x)[P][D],
+                                             T (&acc)[P]) {
+    constexpr int S = Rec<T, D>::kStride;
+#pragma unroll 2
+    for (int g = begin + row; g < end; g += 4) {
+        T r[Rec<T, D>::kUsed];
+#pragma unroll
+        for (int i = 0; i < Rec<T, D>::kUsed; ++i) r[i] = lds[g * S + i];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            T y[D];
+            const T q = quad_form<T, D, CENTRED>(r, x[p], y);
+            acc[p] = fma_(r[Rec<T, D>::kAmp], fast_exp2(-q), acc[p]);
+        }
+    }
+}
+
+template <typename T, int D, int P>
+__global__ __launch_bounds__(kBlock) void eval_fwd_rc_kernel(const T* __restrict__ mixture, const T* __restrict__ xes,
+                                                             T* __restrict__ out, int L, int M, int N, int Bx, int Lx,
+                                                             int chunks, int n_mixtures, bool covariance_form) {
+    constexpr int G = 1 + D + D * D;
+    constexpr int S = Rec<T, D>::kStride;
+    __shared__ __attribute__((aligned(16))) T lds[(kTile + 6) * S];
+    __shared__ int counts[10];
+
+    int bl, chunk;
+    map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
+    if (bl >= n_mixtures) return;
+    const int b = bl / L, l = bl - b * L;
+    const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
+    const T* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
+    const T* __restrict__ x_bl = xes + (size_t(xb) * Lx + xl) * N * D;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = lane >> 4, col = lane & 15;
+    T x[P][D];
+    T acc[P];
+    const int n0 = (chunk * 4 + wave) * (16 * P) + col;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        int n = n0 + p * 16;
+        n = n < N ? n : N - 1;
+#pragma unroll
+        for (int d = 0; d < D; ++d) x[p][d] = x_bl[size_t(n) * D + d];
+        acc[p] = T(0);
+    }
+    for (int g0 = 0; g0 < M; g0 += kTile) {
+        const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
+        stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts, covariance_form);
+        const int centred_start = counts[8], padded_total = counts[9];
+        fwd_rc_pairs<T, D, P, false>(lds, 0, centred_start, row, x, acc);
+        fwd_rc_pairs<T, D, P, true>(lds, centred_start, padded_total, row, x, acc);
+    }
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        T v = acc[p];
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        const int n = n0 + p * 16;
+        if (row == 0 && n < N) out[size_t(bl) * N + n] = v;
+    }
+}
+
 // Backward pair kernel, "4 x 16" wavefront layout.  The 64 lanes of a wavefront form 4 DPP rows of 16 lanes:
 // row r works on Gaussian 4k + r of the tile in step k, column c on the points {c, c + 16, ..., c + 16 (P-1)} of
 // the wavefront's 16 P points.  The per-Gaussian sums are then reduced over one DPP row only (4 shifts, no
@@ -417,6 +486,37 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
     }
     const int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
     const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
+    {
+        // the 4 x 16 layout covers the points in steps of 64 q: taken when that pads the last chunk clearly less
+        constexpr int q_max = sizeof(T) == 8 ? 8 : 16;
+        int q_best = 0;
+        size_t covered_best = size_t(chunks) * kBlock * P;
+        covered_best -= covered_best / 16;                              // the other layout has to win by 6 %
+        for (int q = q_max; q >= 2; --q) {
+            const size_t q_chunks = (size_t(s.N) + 64 * q - 1) / (64 * q);
+            if (q > 2 && q_chunks * BL < 256) continue;
+            if (q_chunks * 64 * q < covered_best) { covered_best = q_chunks * 64 * q; q_best = q; }
+        }
+        if (q_best > 0) {
+            const int q_chunks = (s.N + 64 * q_best - 1) / (64 * q_best);
+            const dim3 q_grid(unsigned(grid_mixtures(BL) * q_chunks));
+#define GMC_FWD_RC(QQ) case QQ: eval_fwd_rc_kernel<T, D, QQ><<<q_grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, q_chunks, int(BL), cov); break
+            switch (q_best) {
+                GMC_FWD_RC(2); GMC_FWD_RC(3); GMC_FWD_RC(4); GMC_FWD_RC(5); GMC_FWD_RC(6); GMC_FWD_RC(7); GMC_FWD_RC(8);
+                default:
+                    if constexpr (q_max > 8) {
+                        switch (q_best) {
+                            GMC_FWD_RC(9); GMC_FWD_RC(10); GMC_FWD_RC(11); GMC_FWD_RC(12); GMC_FWD_RC(13); GMC_FWD_RC(14);
+                            GMC_FWD_RC(15); GMC_FWD_RC(16);
+                            default: break;
+                        }
+                    }
+                    break;
+            }
+#undef GMC_FWD_RC
+            return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+        }
+    }
     const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
 #define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks, int(BL), cov)
     switch (P) {
