@@ -47,7 +47,8 @@ struct BvhLayout {
     size_t cand_count;          // int [BL][ceil(N/64)]    candidate leaves of every point group, -1: not known
     size_t cand_list;           // int [BL][ceil(N/64)][kLeafCap], then a pool of pool_cap ints for the lists of
                                 // later rounds (all empty when the lists would exceed kCandCacheBytes)
-    size_t cand_ctl;            // int [2]                 pieces published, pool ints handed out
+    size_t cand_ctl;            // int [4]                 pieces published, pool ints handed out, address of the points
+                                //                         the object was built for (64 bits)
     size_t pieces;              // int4 [pieces_max]       (point group, offset into cand_list, leaves, -)
     size_t piece_gx;            // T [pieces_max][D][64]   dL/dx of the pieces, added to grad_xes by the epilogue
     bool cand_cache;
@@ -85,6 +86,12 @@ struct CandidateCache {
     int* ctl;
     int4* pieces;
     int pieces_max, pool_cap, pool_base;
+    // The lists describe the points the object was built for.  A traversal may be given other points (the order of
+    // the build is then only a poor grouping, the result is still right), so the lists are used and written only
+    // when the traversal's points live where the build's points lived.
+    __device__ bool built_for(const void* xes) const {
+        return count != nullptr && reinterpret_cast<const unsigned long long*>(ctl)[1] == (unsigned long long)(size_t)xes;
+    }
 };
 constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
 constexpr int kSortBlocksMax = 256;                 // radix blocks per segment (more items per lane beyond that)
@@ -148,7 +155,7 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
         l.pool_cap = l.cand_cache ? int(65536 + point_groups * 16) : 0;
         l.cand_count = take(l.cand_cache ? point_groups * 4 : 0);
         l.cand_list = take(l.cand_cache ? (point_groups * kLeafCap + l.pool_cap) * 4 : 0);
-        l.cand_ctl = take(l.cand_cache ? 8 : 0);
+        l.cand_ctl = take(l.cand_cache ? 16 : 0);
         l.pieces = take(size_t(l.pieces_max) * 16);
         l.piece_gx = take(size_t(l.pieces_max) * D * kWave * e);
     }
@@ -777,11 +784,13 @@ template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __restrict__ children,
                                                                 const long long* __restrict__ enc_box, T* node_box,
                                                                 T* __restrict__ child_box, int M, size_t total,
-                                                                CandidateCache cache, size_t point_groups) {
+                                                                CandidateCache cache, size_t point_groups,
+                                                                const void* xes) {
     const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
     if (cache.count) {                               // a new tree: no candidate list is known yet
         for (size_t j = t; j < point_groups; j += size_t(gridDim.x) * kBlock) cache.count[j] = -1;
         if (t < 2) cache.ctl[t] = 0;
+        if (t == 2) reinterpret_cast<unsigned long long*>(cache.ctl)[1] = (unsigned long long)(size_t)xes;
     }
     if (t >= total) return;
     const size_t bl = t / (M - 1);
@@ -920,8 +929,10 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     // (Last, because most of them find no piece: at the end of the grid they start when compute units run idle.)
     const int owners = int(gridDim.x) - (MODE == 1 ? helpers : 0);
     const int piece = int(blockIdx.x) >= owners ? int(blockIdx.x) - owners : -1;
+    if (!cache.built_for(xes)) cache.count = nullptr;       // other points than the build's: no lists, no pieces
     int4 piece_desc = make_int4(0, 0, 0, 0);
     if (piece >= 0) {
+        if (!cache.count) return;
         const int published = cache.ctl[0] < cache.pieces_max ? cache.ctl[0] : cache.pieces_max;
         if (piece >= published) return;
         piece_desc = cache.pieces[piece];
@@ -1317,13 +1328,15 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
                                                                  bool covariance_form, CandidateCache cache,
                                                                  const T* __restrict__ piece_gx,
                                                                  const int* __restrict__ p_order, T* __restrict__ grad_xes,
-                                                                 unsigned gaussian_blocks, int L, int N, int Bx, int Lx) {
+                                                                 const T* __restrict__ xes, unsigned gaussian_blocks, int L,
+                                                                 int N, int Bx, int Lx) {
     constexpr int G = 1 + D + D * D;
     constexpr int NR = BvhSums<D>::k;
     // Workgroups behind the first `gaussian_blocks`: dL/dx of the pieces that helper workgroups of the traversal
     // worked on, one wavefront per piece, added to what the owners of the point groups have stored (several
     // pieces of a group meet here, hence atomics).
     if (blockIdx.x >= gaussian_blocks) {
+        if (!cache.built_for(xes)) return;                  // the traversal had no helpers then
         const int published = cache.ctl[0] < cache.pieces_max ? cache.ctl[0] : cache.pieces_max;
         const int per_mixture = (N + kWave - 1) / kWave;
         const int lane = threadIdx.x & 63;
@@ -1520,7 +1533,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
             bvh_merge_kernel<T, D><<<dim3(unsigned((n + kMergeBlock - 1) / kMergeBlock)), dim3(kMergeBlock), 0, st>>>(
                 parent, node_range, node_box, enc_box, M, n);
             bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(
-                children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups);
+                children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups, xes);
         }
     }
     if (have_p && !sort_p) iota_segments_kernel<<<dim3(grid_for(XL * N)), dim3(kBlock), 0, st>>>(p_order, N, XL * N);
@@ -1598,7 +1611,7 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bv
         const unsigned piece_blocks = pieces_gx ? unsigned((helpers + kBlock / kWave - 1) / (kBlock / kWave)) : 0u;
         bvh_bwd_epilogue_kernel<T, D><<<dim3(gaussian_blocks + piece_blocks), dim3(kBlock), 0, st>>>(
             mixture, sums, grad_mixture, n_g, covariance_form, cache, piece_gx, (const int*)(bvh + lay.p_order), grad_xes,
-            gaussian_blocks, s.L, s.N, s.Bx, s.Lx);
+            xes, gaussian_blocks, s.L, s.N, s.Bx, s.Lx);
     }
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }

@@ -141,7 +141,9 @@ int gmc_bvh_export_candidate_stats(const void* bvh, int32_t* stats, const gmc_sh
  * written to by these calls: calls that use one BVH object must be ordered (same stream, or events).  A forward
  * pass also cuts candidate lists of more than 240 leaves into pieces; the backward pass that follows gives every
  * piece but the first to a workgroup of its own, so that a few point groups in dense regions do not hold up the
- * launch. */
+ * launch.  The lists belong to the points the object was built for: a traversal whose `xes` is another address than
+ * the build's neither uses nor writes them (it is correct, only slower); the points at that address must not be
+ * changed between the build and the traversals that use it. */
 int gmc_eval_bvh_fwd(const void* mixture, const void* xes, void* bvh, void* out, const gmc_shape* shape,
                      void* stream);
 int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh,

@@ -297,6 +297,31 @@ def test_long_candidate_lists_are_shared_between_workgroups(broadcast):
     _check_culled(mix, xes, gout, torch.float32, "tight", tag=f"crowded, broadcast {broadcast}")
 
 
+def test_traversal_with_other_points_than_the_build():
+    """The lists and pieces kept in the BVH object describe the points it was built for.  A traversal that is given
+    other points (at another address) must neither use nor overwrite them: it gives what a BVH built for those points
+    gives, and the first points still find their lists afterwards."""
+    mix, xes, gout = _crowded_case(1, 670, False)
+    n = lambda t: t.cpu().numpy()
+    m, xa, g = (t.to(DEV).contiguous() for t in (mix, xes, gout))
+    xb = torch.roll(xa, 5000, dims=2).mul(0.9).contiguous()
+    bvh = _native.Bvh(m, xa, 0.001, "tight")
+    first = _native.eval_bvh_fwd(m, xa, bvh)
+    stats = n(bvh.candidate_stats()).tolist()
+    assert stats[0] > 0
+    fresh = _native.Bvh(m, xb, 0.001, "tight")
+    other = _native.eval_bvh_fwd(m, xb, bvh)
+    assert rel_l2(n(other), n(_native.eval_bvh_fwd(m, xb, fresh))) <= 1e-13
+    assert n(bvh.candidate_stats()).tolist() == stats
+    gm_a, gx_a = _native.eval_bvh_bwd(g, m, xb, bvh, True, True)
+    gm_b, gx_b = _native.eval_bvh_bwd(g, m, xb, fresh, True, True)
+    assert rel_l2(n(gm_a), n(gm_b)) <= 1e-13 and rel_l2(n(gx_a), n(gx_b)) <= 1e-13
+    assert torch.equal(first, _native.eval_bvh_fwd(m, xa, bvh))
+    gm_c, gx_c = _native.eval_bvh_bwd(g, m, xa, bvh, True, True)
+    gm_d, gx_d = _native.eval_bvh_bwd(g, m, xa, _native.Bvh(m, xa, 0.001, "tight"), True, True)
+    assert rel_l2(n(gm_c), n(gm_d)) <= 1e-13 and rel_l2(n(gx_c), n(gx_d)) <= 1e-13
+
+
 def test_points_outside_every_box_and_need_flags():
     mix, xes, gout = _case(1, 2, 40, 64, 3, seed=400)
     far = xes + 1000.0
