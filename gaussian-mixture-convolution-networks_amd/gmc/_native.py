@@ -269,8 +269,17 @@ class Bvh:
         return stats
 
 
+def _check_bvh_shape(shape: Shape, bvh: "Bvh"):
+    """the layout of the opaque BVH object follows from the shape it was built for"""
+    for name, _ in Shape._fields_:
+        if getattr(shape, name) != getattr(bvh.shape, name):
+            raise RuntimeError(f"the BVH was built for another shape or dtype ({name}: {getattr(bvh.shape, name)} at the "
+                               f"build, {getattr(shape, name)} now)")
+
+
 def eval_bvh_fwd(mixture, xes, bvh: Bvh) -> torch.Tensor:
     shape = check_input(mixture, xes)
+    _check_bvh_shape(shape, bvh)
     out = torch.empty((shape.B, shape.L, shape.N), dtype=mixture.dtype, device=mixture.device)
     with torch.cuda.device(mixture.device):
         check(lib().gmc_eval_bvh_fwd(_p(mixture), _p(xes), _p(bvh.blob), _p(out), ctypes.byref(shape),
@@ -280,6 +289,7 @@ def eval_bvh_fwd(mixture, xes, bvh: Bvh) -> torch.Tensor:
 
 def eval_bvh_bwd(grad_output, mixture, xes, bvh: Bvh, need_mixture: bool, need_xes: bool):
     shape = check_input(mixture, xes)
+    _check_bvh_shape(shape, bvh)
     if tuple(grad_output.shape) != (shape.B, shape.L, shape.N):
         raise RuntimeError("grad_output has wrong shape")
     if grad_output.dtype != mixture.dtype:

@@ -349,6 +349,13 @@ def test_empty_and_config_errors():
         gm.evaluate_inversed(mix, xes, bvh=gm.BvhConfig(aabb_mode="loose"))
     with pytest.raises(RuntimeError, match="positive"):
         gm.evaluate_inversed(mix, xes, bvh=gm.BvhConfig(aabb_threshold=0.0))
+    # the opaque object is laid out for the shape it was built for
+    mix[..., [4, 8, 12]] = 1.0
+    bvh = _native.Bvh(mix, xes)
+    with pytest.raises(RuntimeError, match="another shape"):
+        _native.eval_bvh_fwd(mix, torch.zeros(1, 1, 3, 3, device=DEV), bvh)
+    with pytest.raises(RuntimeError, match="another shape"):
+        _native.eval_bvh_bwd(torch.zeros(1, 1, 2, device=DEV, dtype=torch.float64), mix.double(), xes.double(), bvh, True, True)
 
 
 def test_gradcheck_culled_fp64():
