@@ -143,7 +143,8 @@ int gmc_bvh_export_candidate_stats(const void* bvh, int32_t* stats, const gmc_sh
  * piece but the first to a workgroup of its own, so that a few point groups in dense regions do not hold up the
  * launch.  The lists belong to the points the object was built for: a traversal whose `xes` is another address than
  * the build's neither uses nor writes them (it is correct, only slower); the points at that address must not be
- * changed between the build and the traversals that use it. */
+ * changed between the build and the traversals that use it.  `shape` must be the shape the object was built for:
+ * the layout of the object follows from it and is not stored inside. */
 int gmc_eval_bvh_fwd(const void* mixture, const void* xes, void* bvh, void* out, const gmc_shape* shape,
                      void* stream);
 int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh,
