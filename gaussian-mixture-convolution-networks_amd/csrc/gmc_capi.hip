@@ -20,6 +20,10 @@ int check_shape(const gmc_shape* s) {
     // per-(b,l) index arithmetic inside the kernels is 32-bit
     if (size_t(s->M) * 13 > 0x7fffffffull || size_t(s->N) * 3 > 0x7fffffffull) return GMC_E_SHAPE;
     if (size_t(s->B) * s->L > 0x7fffffffull / 64) return GMC_E_SHAPE;
+    // launch grids: at most one workgroup per mixture, 64 points and 256 components (such tensors exceed the
+    // memory of the device long before; the bound keeps the 32-bit grid sizes honest)
+    const size_t groups = size_t(s->B) * s->L * (size_t(s->N) / 64 + 1);
+    if (groups > 0x7fffffffull || groups * (size_t(s->M) / 256 + 1) > 0x7fffffffull) return GMC_E_SHAPE;
     return GMC_OK;
 }
 }  // namespace gmc
