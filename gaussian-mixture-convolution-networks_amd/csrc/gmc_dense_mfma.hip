@@ -1,13 +1,13 @@
 // Dense float32 Gaussian-mixture evaluation with the affine part of every pair on the matrix cores of gfx950.
 //
-// Same mathematics and the same reference entry points as gmc_dense.hip
-// (src/gmc/cpp/extensions/evaluate_inversed/parallel_implementation.cu:23-55 forward, :133-173 backward); what
+// Same mathematics and the same reference entry point as the forward kernel of gmc_dense.hip
+// (src/gmc/cpp/extensions/evaluate_inversed/parallel_implementation.cu:23-55); what
 // changes is where y = u x - u b is computed.  y is bilinear in (per-Gaussian constants, homogeneous point
 // coordinates), i.e. a small matrix product, and v_mfma_f32_16x16x32_bf16 delivers 16 Gaussians x 16 points of it
 // per instruction while the vector ALU works on the previous results.  The vector ALU is left with |y|^2, the
 // exponential and the accumulation: 4 instructions + 1 transcendental per forward pair (10 + 1 in the all-vector
-// kernel).  The backward kernel additionally takes v = u^T y (the direction of dL/dx) from the matrix cores and
-// keeps, per pair, only the products with e and the per-Gaussian sums.
+// kernel).  The backward pass stays on the vector ALU (gmc_dense.hip): with y and u^T y from the matrix cores it
+// was slower in every layout tried, because each matrix instruction costs the vector ALU about 9 issue cycles.
 //
 // float32 accuracy from bf16 operands: every coefficient (from its double value) and every coordinate is split
 // into three bf16 pieces h + m + l (round to nearest, 8 significant bits each) and the K dimension of the matrix
