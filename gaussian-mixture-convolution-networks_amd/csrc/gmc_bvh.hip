@@ -11,12 +11,15 @@
 //   radix sort (8 bits per pass, stable, keys uint32 + index payload) -> leaves in Morton order with their
 //   evaluation records -> Karras radix tree over the unique keys (morton << 32 | rank), as lbvh/building.h:11-103
 //   -> bottom-up union of boxes with integer atomic min/max on order-preserving encodings.
-// Query points are Morton-sorted the same way so that a wavefront owns 64 neighbouring points.
+// Query points are Morton-sorted the same way (on their top 16 or 8 key bits) so that a wavefront owns 64
+// neighbouring points.
 //
 // Traversal: 64 sorted points form a group with ONE node stack (LDS); lanes work on tree nodes while the tree is
 // descended and on points while the gathered leaves are evaluated; a workgroup serves up to four groups, whose
 // descents overlap (see bvh_traverse_kernel).  Backward collects the per-Gaussian sums of a batch of leaves in LDS
-// and issues one global atomic per non-zero scalar, leaf and wavefront.
+// and issues one global atomic per non-zero scalar, leaf and wavefront.  The candidate leaves of every group stay
+// in the BVH object after the first traversal, so the backward pass after a forward pass does not descend, and
+// long lists are cut into pieces that helper workgroups of the backward launch take over (see kPieceLeaves).
 #include "gmc_common.h"
 
 namespace gmc {

@@ -6,7 +6,8 @@
 // The work is pure streaming (HBM-bound: the output is Nk Cout / 1 times larger than the data), so the kernels are
 // laid out for coalescing and for single passes over the big tensor:
 //   forward   one lane per scalar of the data: one load, then Cout Nk coalesced stores;
-//   backward  grad_data: one lane per scalar of grad_data gathers its Cout Nk terms, every read of grad_out is
+//   backward  both gradients: one pass over grad_out (conv_bwd_fused_kernel); one gradient only:
+//             grad_data: one lane per scalar of grad_data gathers its Cout Nk terms, every read of grad_out is
 //             coalesced and no atomics are needed (the reference adds every term atomically);
 //             grad_kernels: one workgroup per (co, ci, k) and slice of the batch sums B Nd terms per scalar with
 //             lanes striding over whole Gaussians, then an LDS reduction; slices > 1 finish with one atomic each.
