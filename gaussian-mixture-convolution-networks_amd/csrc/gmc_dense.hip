@@ -220,18 +220,30 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
             }
         }
         if (NEED_GM) {
+            // Row reduction of the NR sums, two at a time: the two halves of a row first exchange the sum they do not
+            // keep (lanes 0-7 keep the even one, lanes 8-15 the odd one), then three shifts are left; the totals
+            // arrive in lanes 7 and 15.  4 instructions per sum instead of 5 and half as many LDS atomics.
+            static_assert(NR % 2 == 0, "the sums are reduced in pairs");
+            const bool high = (threadIdx.x & 8) != 0;
+            T half[NR / 2];
 #pragma unroll
-            for (int i = 0; i < NR; ++i) {
-                rs[i] = row_sum_to_lane15(rs[i]);
+            for (int i = 0; i < NR / 2; ++i) {
+                const T keep = high ? rs[2 * i + 1] : rs[2 * i], send = high ? rs[2 * i] : rs[2 * i + 1];
+                T v = keep + dpp_mov<0x128>(send);          // row_ror:8
+                v += dpp_mov<0x111>(v);                     // row_shr:1
+                v += dpp_mov<0x112>(v);                     // row_shr:2
+                v += dpp_mov<0x114>(v);                     // row_shr:4 -> lanes 7 and 15 hold the sums of lanes 0-7, 8-15
                 // keeps the last addition in front of the branch below, where it stays one DPP instruction (sunk
                 // into the branch it becomes a zero fill, a DPP move and an addition)
-                asm volatile("" : "+v"(rs[i]));
+                asm volatile("" : "+v"(v));
+                half[i] = v;
             }
-            if ((threadIdx.x & 15) == 15) {
+            if ((threadIdx.x & 7) == 7) {
                 const int idx = record_index<T, D>(lds + g * S);
                 if (idx >= 0) {
+                    T* dst = block_sums + idx * NR + (high ? 1 : 0);
 #pragma unroll
-                    for (int i = 0; i < NR; ++i) atomic_add(&block_sums[idx * NR + i], rs[i]);
+                    for (int i = 0; i < NR / 2; ++i) atomic_add(&dst[2 * i], half[i]);
                 }
             }
         }
