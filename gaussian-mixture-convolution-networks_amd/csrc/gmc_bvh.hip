@@ -1022,7 +1022,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     // leaf records of the NEXT batch (possibly of the next group) are fetched into registers before the current
     // batch is tested and evaluated, so their memory round trip overlaps that work and the group's barriers.
     constexpr int kPre = (kStageBatch * LS + kWave - 1) / kWave;
-    constexpr int kDenseHits = sizeof(T) == 8 ? 32 : 12;    // lanes per leaf from which the reduction is cheaper
+    constexpr int kDenseHits = sizeof(T) == 8 ? 16 : 6;    // lanes per leaf from which the reduction is cheaper
     int cur_group = -1, cur_base = 0, cur_end = 0;
     T pre[kPre];
     auto next_batch = [&]() {
@@ -1113,11 +1113,14 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                     for (int a = 0; a < D; ++a)
 #pragma unroll
                         for (int c = a; c < D; ++c) rs[k++] = rs[1 + a] * t[c];
+                    // four sums at a time; the lane at the end of row r receives sum {0, 2, 1, 3}[r] of the four
+                    const int row = lane >> 4, mine = ((row & 1) << 1) | (row >> 1);
 #pragma unroll
-                    for (int q = 0; q < NR; ++q) rs[q] = wave_sum_to_lane63(rs[q]);
-                    if (lane == 63) {
-#pragma unroll
-                        for (int q = 0; q < NR; ++q) rsum[i * NR + q] += double(rs[q]);
+                    for (int q0 = 0; q0 < NR; q0 += 4) {
+                        const T total = wave_sum4_to_row_ends(rs[q0], q0 + 1 < NR ? rs[q0 + 1] : T(0),
+                                                              q0 + 2 < NR ? rs[q0 + 2] : T(0),
+                                                              q0 + 3 < NR ? rs[q0 + 3] : T(0), lane);
+                        if ((lane & 15) == 15 && q0 + mine < NR) rsum[i * NR + q0 + mine] += double(total);
                     }
                 }
                 mask = ((mask >> rot) | (mask << (kStageBatch - rot))) & ((1u << kStageBatch) - 1u);

@@ -62,24 +62,6 @@ __global__ __launch_bounds__(kBlock) void componentwise_fwd_kernel(const T* __re
 // LDS copy, which leaves with one atomic (or, when one workgroup sees all Gaussians of the point, one store) per
 // scalar.
 constexpr int kCwUnroll = 8;
-
-// Sums four values per lane (a, b, c, d) over the 64 lanes at once: the half-wavefronts first exchange the values
-// they do not keep (lower half keeps a and c, upper half b and d), then the 16-lane rows of each half do the same,
-// and one row reduction is left: the total of a arrives in lane 15, of c in lane 31, of b in lane 47, of d in lane
-// 63.  13 vector instructions and 3 cross-lane moves instead of 24 for four separate wavefront sums.
-template <typename T>
-__device__ __forceinline__ T wave_sum4_to_row_ends(T a, T b, T c, T d, int lane) {
-    const bool upper = lane >= 32;
-    T keep0 = upper ? b : a, keep1 = upper ? d : c;
-    const T send0 = upper ? a : b, send1 = upper ? c : d;
-    keep0 += __shfl_xor(send0, 32, 64);
-    keep1 += __shfl_xor(send1, 32, 64);
-    const bool odd_row = (lane & 16) != 0;
-    T keep = odd_row ? keep1 : keep0;
-    const T send = odd_row ? keep0 : keep1;
-    keep += __shfl_xor(send, 16, 64);
-    return row_sum_to_lane15(keep);
-}
 constexpr int kCwPointsMax = 1024;  // points per workgroup of the backward pass (a multiple of kCwPoints, chosen per launch)
 
 template <typename T, int D, bool NEED_GM, bool NEED_GX>
