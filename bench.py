@@ -34,8 +34,8 @@ VALU_NOTE = ("compute-bound against the FP32 peak of 157.3 TFLOP/s (matrix = pac
              "from the bf16 matrix cores")
 MEASURED_TRAFFIC_BYTES = {"C4": 157960 * 1024 * 2.0 + 524288 * 1024 * 1.0,
                           # LBVH traversal kernels of C5 (aabb_mode "reference"): backward, forward
-                          "C5": 29849.3 * 1024 * 2.0 + 50524.4 * 1024 * 1.0,
-                          "C5_fwd": 21532.1 * 1024 * 2.0 + 4092.3 * 1024 * 1.0}
+                          "C5": 18586.3 * 1024 * 2.0 + 18644.2 * 1024 * 1.0,
+                          "C5_fwd": 21522.2 * 1024 * 2.0 + 4090.9 * 1024 * 1.0}
 
 
 def cpu_baseline(name: str):
