@@ -958,6 +958,8 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     int cache_slot = -1;                                    // the group whose candidate list this wavefront's descent leaves
     bool cache_ok = true;                                   // ... as long as every part of it found room
     int first_round_leaves = 0, n_pend = 0;
+    bool publish = false;                                   // the group's descent has ended with all parts in place
+    int piece_slot = 0, publish_slot = 0, publish_flags = 0;
     if (wave < groups) {
         // The groups of a workgroup lie far apart in Morton order, one in every quarter of the range and at
         // different places within the quarters: point groups with long candidate lists come in clusters (dense
@@ -1191,6 +1193,10 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             T glo[D], ghi[D];
 #pragma unroll
             for (int d = 0; d < D; ++d) { glo[d] = gbox[wave][d]; ghi[d] = gbox[wave][D + d]; }
+            // room in the pool for the list of a later round is asked for before the descent, so that the atomic's
+            // round trip is over when the list is there (a whole list's worth; what is not used stays unused)
+            int pool_at = 0;
+            if (cache_slot >= 0 && cache_ok && round > 0 && lane == 0) pool_at = atomicAdd(&cache.ctl[1], kLeafCap);
             for (int iter = 0; sp > 0 && n_leaf < kLeafFlush && iter < M; ++iter) {
                 wave_lds_fence();
                 // wide pops only while the stack has room for 128 more entries; a narrow pop is a depth-first
@@ -1239,9 +1245,8 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                         first_round_leaves = n_leaf;
                         own = share;
                     } else {
-                        int at = lane == 0 ? atomicAdd(&cache.ctl[1], n_leaf) : 0;
-                        at = __builtin_amdgcn_readfirstlane(at);
-                        cache_ok = at + n_leaf <= cache.pool_cap;
+                        const int at = __builtin_amdgcn_readfirstlane(pool_at);
+                        cache_ok = at + kLeafCap <= cache.pool_cap;
                         base = cache.pool_base + at;
                     }
                     const int wanted = (n_leaf - own + share - 1) / share;
@@ -1257,18 +1262,12 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                     }
                 }
                 if (sp == 0) {
-                    if (cache_ok && n_pend > 0) {
-                        int slot = lane == 0 ? atomicAdd(&cache.ctl[0], n_pend) : 0;
-                        slot = __builtin_amdgcn_readfirstlane(slot);
-                        cache_ok = slot + n_pend <= cache.pieces_max;
-                        wave_lds_fence();
-                        // slots in range are always filled: a helper must never read an unwritten piece
-                        if (lane < n_pend && slot + lane < cache.pieces_max)
-                            cache.pieces[slot + lane] = cache_ok ? make_int4(cache_slot, pend[wave][lane].x, pend[wave][lane].y, 0)
-                                                                 : make_int4(0, 0, 0, 0);
-                    }
-                    if (cache_ok && lane == 0)
-                        cache.count[cache_slot] = first_round_leaves | (n_pend > 0 ? kCandSplit : 0) | (round > 0 ? kCandRounds : 0);
+                    // the descent has ended: ask for the slots of the pieces now, fill them after this round's
+                    // evaluation (the atomic's round trip then overlaps the first record fetches)
+                    publish = cache_ok;
+                    if (cache_ok && n_pend > 0 && lane == 0) piece_slot = atomicAdd(&cache.ctl[0], n_pend);
+                    publish_flags = first_round_leaves | (n_pend > 0 ? kCandSplit : 0) | (round > 0 ? kCandRounds : 0);
+                    publish_slot = cache_slot;
                     cache_slot = -1;
                 }
             }
@@ -1295,6 +1294,20 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                 }
                 __syncthreads();
             }
+        }
+        if (publish) {
+            publish = false;
+            bool fits = true;
+            if (n_pend > 0) {
+                const int slot = __builtin_amdgcn_readfirstlane(piece_slot);
+                fits = slot + n_pend <= cache.pieces_max;
+                wave_lds_fence();
+                // slots in range are always filled: a helper must never read an unwritten piece
+                if (lane < n_pend && slot + lane < cache.pieces_max)
+                    cache.pieces[slot + lane] = fits ? make_int4(publish_slot, pend[wave][lane].x, pend[wave][lane].y, 0)
+                                                     : make_int4(0, 0, 0, 0);
+            }
+            if (fits && lane == 0) cache.count[publish_slot] = publish_flags;
         }
         if (!left_on_stack) break;
         __syncthreads();                                                // every wavefront has read this round's state
