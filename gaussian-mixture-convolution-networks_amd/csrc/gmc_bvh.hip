@@ -99,7 +99,7 @@ struct CandidateCache {
 constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
 constexpr int kSortBlocksMax = 256;                 // radix blocks per segment (more items per lane beyond that)
 constexpr int kCoarseOrderMax = 8192;               // point segments up to this size are ordered by 8 Morton bits only
-constexpr int kBoundsChunk = kBlock * 16;           // points per workgroup of the partial bounds of the query points
+constexpr int kBoundsChunk = kBlock * 2;            // points per workgroup of the partial bounds of the query points
 
 // items per lane of a radix block for segments of `count` keys
 static int sort_items(size_t count) {
@@ -344,16 +344,15 @@ __device__ __forceinline__ T block_bounds(const T (&lo)[D], const T (&hi)[D], T 
 }
 
 // One launch for two independent jobs.
-// Workgroups [0, box_blocks): cutoff box of every Gaussian; workgroup (blk, seg) also leaves the bounds of its 256
-// centres in parts_g[seg][blk].
+// Workgroups [0, box_blocks): workgroup (blk, seg) leaves the bounds of its 256 centres in parts_g[seg][blk].  (The
+// cutoff boxes of the Gaussians, a long chain of double arithmetic, are not needed before the leaves are written:
+// bvh_leaves_kernel computes them, next to the tree build, off the critical path of the sort.)
 // Workgroups behind them: partial bounds of the query points; workgroup (blk, seg) reduces kBoundsChunk points to
 // parts_p[seg][blk] = (min_0..min_D-1, max_0..max_D-1).  The Morton kernel combines the partial records.
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
-                                                          T* __restrict__ box_hi, int M, int blocks_per_mixture,
-                                                          double threshold, int mode, bool covariance_form,
-                                                          T* __restrict__ parts_g, unsigned box_blocks, const T* __restrict__ xes, int N,
-                                                          int blocks_per_xseg, T* __restrict__ parts_p) {
+__global__ __launch_bounds__(kBlock) void bvh_bounds_kernel(const T* __restrict__ mixture, int M, int blocks_per_mixture,
+                                                           T* __restrict__ parts_g, unsigned box_blocks, const T* __restrict__ xes, int N,
+                                                           int blocks_per_xseg, T* __restrict__ parts_p) {
     constexpr int G = 1 + D + D * D;
     __shared__ T red[2 * D][kBlock];
     T lo[D], hi[D];
@@ -364,11 +363,7 @@ __global__ __launch_bounds__(kBlock) void bvh_boxes_kernel(const T* __restrict__
         if (m < M) {
             const size_t i = size_t(seg) * M + m;
             const T* g = mixture + i * G;
-            double delta[D];
-            box_half_extent<T, D>(g, threshold, mode, covariance_form, delta);
             for (int k = 0; k < D; ++k) {
-                box_lo[i * D + k] = T(double(g[1 + k]) - delta[k]);
-                box_hi[i * D + k] = T(double(g[1 + k]) + delta[k]);
                 lo[k] = g[1 + k] < lo[k] ? g[1 + k] : lo[k];       // a NaN coordinate is skipped
                 hi[k] = g[1 + k] > hi[k] ? g[1 + k] : hi[k];
             }
@@ -645,8 +640,9 @@ __device__ __forceinline__ void build_internal_node(const uint32_t* __restrict__
 }
 
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, const T* __restrict__ box_lo,
-                                                           const T* __restrict__ box_hi, const uint32_t* __restrict__ order,
+__global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
+                                                           T* __restrict__ box_hi, double threshold, int mode,
+                                                           const uint32_t* __restrict__ order,
                                                            const uint32_t* __restrict__ keys, T* __restrict__ node_box,
                                                            T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
                                                            int2* __restrict__ children, int* __restrict__ parent,
@@ -672,9 +668,22 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
     comp = (comp >= 0 && comp < M) ? comp : 0;      // a permutation by construction; never index out of bounds
     const size_t gi = bl * M + comp;
     const size_t node = bl * (2 * size_t(M) - 1) + (M - 1) + leaf;
+    const T* g = mixture + gi * G;
+    // cutoff box of the Gaussian (lbvh/bvh.cu:164-231), kept in component order too (gmc_bvh_export_boxes)
+    T blo[D], bhi[D];
+    {
+        double delta[D];
+        box_half_extent<T, D>(g, threshold, mode, covariance_form, delta);
+        for (int d = 0; d < D; ++d) {
+            blo[d] = T(double(g[1 + d]) - delta[d]);
+            bhi[d] = T(double(g[1 + d]) + delta[d]);
+            box_lo[gi * D + d] = blo[d];
+            box_hi[gi * D + d] = bhi[d];
+        }
+    }
     for (int d = 0; d < D; ++d) {
-        node_box[node * 2 * D + d] = box_lo[gi * D + d];
-        node_box[node * 2 * D + D + d] = box_hi[gi * D + d];
+        node_box[node * 2 * D + d] = blo[d];
+        node_box[node * 2 * D + D + d] = bhi[d];
     }
     if (leaf < M - 1) {
         // empty box of internal node `leaf`: lower = +inf, upper = -inf in the ordered-integer encoding
@@ -682,9 +691,8 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         for (int d = 0; d < D; ++d) { e[d] = ordered_bits(double(INFINITY)); e[D + d] = ordered_bits(double(-INFINITY)); }
     }
     if (M == 1) parent[node] = -1;                  // a single leaf is its own root
-    const T* g = mixture + gi * G;
     T* r = leaf_rec + i * RS;
-    for (int d = 0; d < D; ++d) { r[d] = box_lo[gi * D + d]; r[D + d] = box_hi[gi * D + d]; }
+    for (int d = 0; d < D; ++d) { r[d] = blo[d]; r[D + d] = bhi[d]; }
     r += 2 * D;
     double cm[D][D];                                  // inverse covariance as evaluate_inversed takes it
     load_inverse_covariance<T, D>(g + 1 + D, covariance_form, cm);
@@ -1522,9 +1530,8 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     const int bpx = (N + kBlock - 1) / kBlock;               // workgroups per point segment (keys)
     const unsigned box_blocks = have_g ? unsigned(BL * bpm) : 0u, bound_blocks = sort_p ? unsigned(XL * nbp) : 0u;
     if (box_blocks + bound_blocks > 0)
-        bvh_boxes_kernel<T, D><<<dim3(box_blocks + bound_blocks), dim3(kBlock), 0, st>>>(
-            mixture, box_lo, box_hi, M, bpm, double(cfg.aabb_threshold), cfg.aabb_mode, cfg.covariance_form != 0, parts_g,
-            box_blocks, xes, N, nbp, parts_p);
+        bvh_bounds_kernel<T, D><<<dim3(box_blocks + bound_blocks), dim3(kBlock), 0, st>>>(
+            mixture, M, bpm, parts_g, box_blocks, xes, N, nbp, parts_p);
     MortonJob<T> mg = {}, mp = {};
     if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm)};
     if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx)};
@@ -1544,7 +1551,8 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     }
     if (have_g) {
         const size_t n = BL * M;
-        bvh_leaves_kernel<T, D><<<dim3(2 * grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi, g_order, g_keys,
+        bvh_leaves_kernel<T, D><<<dim3(2 * grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi,
+                                                                                  double(cfg.aabb_threshold), cfg.aabb_mode, g_order, g_keys,
                                                                            node_box, leaf_rec, enc_box, children, parent, node_range, M, n,
                                                                            cfg.covariance_form != 0);
         if (M > 1) {
