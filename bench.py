@@ -332,15 +332,101 @@ def bench_componentwise(args):
     print(json.dumps(line))
 
 
+def bench_layer(args):
+    """The callers either side of the evaluation in a network layer, on the C2 shape (2-D float32, B=100, L=8, M=128):
+    `gm.evaluate` on a mixture that holds covariances (the inverse is taken inside the kernels) forward + backward
+    at the N=784 grid points, the ReLU fixed-point fitting (two evaluations at the mixture's own 128 centres plus
+    the multiplicative update) and BatchNorm (one evaluation at 100 random samples per channel, moments, rescale).
+    A step runs the three one after the other through the autograd-level API; the value counts the pairs of all
+    evaluations in it."""
+    import torch
+    from gmc import fitting, mat_tools, modules, synthetic
+    from gmc import mixture as gm
+    wl, mix, xes, gout = synthetic.make_workload("C2")
+    dev = torch.device("cuda:0")
+    mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)
+    mix_cov = gm.pack_mixture(gm.weights(mix), gm.positions(mix), mat_tools.inverse(gm.covariances(mix))).contiguous()
+    constant = torch.randn((wl.B, wl.L), generator=torch.Generator().manual_seed(20248)).to(dev)
+    norm = modules.BatchNorm(wl.L).to(dev)
+    leaf = mix_cov.clone().requires_grad_(True)
+    torch.cuda.synchronize()
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        leaf.grad = None
+        gm.evaluate(leaf, xes).backward(gout)
+        if ev:
+            ev[1].record()
+        with torch.no_grad():
+            fitted, _ = fitting.fixed_point_iteration_to_relu(mix_cov, constant, mix_cov, n_iter=1)
+        if ev:
+            ev[2].record()
+        with torch.no_grad():
+            scaled, _ = norm((mix_cov, constant))
+        if ev:
+            ev[3].record()
+        return fitted, scaled
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        step(events[k])
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    eval_ms, fit_ms, norm_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(3))
+    mixtures = wl.B * wl.L
+    pairs_eval = 2 * wl.pairs                                   # forward and backward
+    pairs_fit = 2 * mixtures * wl.M * wl.M
+    pairs_norm = mixtures * wl.M * (10000 // wl.B)
+    pairs = pairs_eval + pairs_fit + pairs_norm
+    line = {
+        "metric": "Gaussian-point evaluations per second through gm.evaluate and its callers (autograd-level API)",
+        "value": pairs / (ms_step * 1e-3), "unit": "Gaussian-point pairs/s (forward pairs + backward pairs)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"layer on C2: D=2 f32 B={wl.B} L={wl.L} M={wl.M}; evaluate(covariances) forward + "
+                               f"backward at N={wl.N}, fixed_point_iteration_to_relu (n_iter=1), BatchNorm.forward"},
+        "evaluate_fwd_bwd": {"ms": eval_ms, "pairs": pairs_eval},
+        "fixed_point_iteration_to_relu": {"ms": fit_ms, "pairs": pairs_fit},
+        "batch_norm_forward": {"ms": norm_ms, "pairs": pairs_norm},
+        "roofline": {"kernel": "eval_bwd_rc_kernel (covariance form, inside evaluate_fwd_bwd)", "bound": "mfma",
+                     "bound_detail": "launch-bound at this size: the step is a chain of small launches and "
+                                     "element-wise torch operations; the fraction is that of the whole evaluate "
+                                     "forward + backward against the FP32 peak at 12 + 30 flop per pair",
+                     "achieved": (FLOP_FWD[2] + FLOP_BWD[2]) * wl.pairs / (eval_ms * 1e-3) / 1e12,
+                     "peak": PEAK_TFLOPS["f32"], "unit": "TFLOP/s",
+                     "frac": (FLOP_FWD[2] + FLOP_BWD[2]) * wl.pairs / (eval_ms * 1e-3) / 1e12 / PEAK_TFLOPS["f32"],
+                     "traffic": None, "launch_ms": eval_ms},
+    }
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import gm_oracle
+        m = mix_cov[:2].cpu().numpy().astype("float64")
+        c = constant[:2].cpu().numpy().astype("float64")
+        t0 = time.perf_counter()
+        gm_oracle.fixed_point_iteration_to_relu(m, c, m, 1)
+        t = time.perf_counter() - t0
+        line["cpu_baseline"] = {"value": 2 * 2 * wl.L * wl.M * wl.M / t, "unit": "pairs/s (fixed-point fitting only)",
+                                "cores": 1, "kind": "port",
+                                "sample": f"the oracle's fixed_point_iteration_to_relu (numpy float64) on two batch "
+                                          f"entries, {t:.2f} s"}
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5", "conv", "cw"],
+    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5", "conv", "cw", "layer"],
                     help="C1..C4: dense all-pairs path; C5: LBVH-culled path (build + forward + backward per step); "
                          "conv: closed-form convolution; cw: component-wise evaluation on the C2 shape (forward + "
-                         "backward per step)")
+                         "backward per step); layer: gm.evaluate on covariances forward + backward, the ReLU fixed-point "
+                         "fitting and BatchNorm on the C2 shape")
     ap.add_argument("--aabb-mode", default="reference", choices=["reference", "tight"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -361,6 +447,8 @@ def main():
         return bench_convolution(args)
     if args.workload == "cw":
         return bench_componentwise(args)
+    if args.workload == "layer":
+        return bench_layer(args)
     wl, mix, xes, gout = synthetic.make_workload(args.workload)
     dev = torch.device("cuda:0")
     mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)
