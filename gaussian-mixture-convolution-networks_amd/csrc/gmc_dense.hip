@@ -194,6 +194,13 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
                     gx[p][1] = fma_(ua[1], ky[0], fma_(ua[3], ky[1], gx[p][1]));
                     gx[p][2] = fma_(ua[2], ky[0], fma_(ua[4], ky[1], fma_(ua[5], ky[2], gx[p][2])));
                 }
+                if (NEED_GM) {
+                    // keeps these additions here: left alone they sink behind the branch of the row reduction below
+                    // (their results are not needed before the next step) and the products k*y of all P points stay
+                    // in registers until then
+#pragma unroll
+                    for (int d = 0; d < D; ++d) asm volatile("" : "+v"(gx[p][d]));
+                }
             }
             if (NEED_GM) {
                 if (p == 0) {
@@ -251,7 +258,7 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
 }
 
 template <typename T, int D, int P, bool NEED_GM, bool NEED_GX>
-__global__ __launch_bounds__(kBlock) void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 3 : 1))) void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture,
                                                              const T* __restrict__ xes, T* __restrict__ sums,
                                                              T* __restrict__ grad_xes, int L, int M, int N, int Bx, int Lx,
                                                              int chunks, int xes_shared, int n_mixtures,
@@ -321,9 +328,13 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_rc_kernel(const T* __restrict
             }
         }
         if (row == 0) {
+            // the indices are formed again from one register: taken from the prologue, all P of them would stay in
+            // registers through the pair loop
+            int n_first = n0;
+            asm volatile("" : "+v"(n_first));
 #pragma unroll
             for (int p = 0; p < P; ++p) {
-                const int n = n0 + p * 16;
+                const int n = n_first + p * 16;
                 if (n < N) {
                     T* dst = grad_xes + (x_off + n) * D;
 #pragma unroll
