@@ -166,6 +166,10 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
         T r[Rec<T, D>::kUsed];
 #pragma unroll
         for (int i = 0; i < Rec<T, D>::kUsed; ++i) r[i] = lds[g * S + i];
+        // the index of the Gaussian comes with the record (one wider LDS read) instead of a read of its own, with its
+        // wait, inside the branch of the row totals
+        int idx = NEED_GM ? record_index<T, D>(lds + g * S) : -1;
+        if (NEED_GM) asm volatile("" : "+v"(idx));
         T rs[NR];
         // dL/dx takes the products k*y against amp*u (formed once per Gaussian), the sums take them against y.
         // With the sums wanted k = e*g (g: upstream gradient of the point), so that the same three products serve
@@ -246,7 +250,6 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
                 half[i] = v;
             }
             if ((threadIdx.x & 7) == 7) {
-                const int idx = record_index<T, D>(lds + g * S);
                 if (idx >= 0) {
                     T* dst = block_sums + idx * NR + (high ? 1 : 0);
 #pragma unroll
