@@ -260,12 +260,18 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
     }
 }
 
-template <typename T, int D, int P, bool NEED_GM, bool NEED_GX>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 3 : 1))) void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture,
-                                                             const T* __restrict__ xes, T* __restrict__ sums,
-                                                             T* __restrict__ grad_xes, int L, int M, int N, int Bx, int Lx,
-                                                             int chunks, int xes_shared, int n_mixtures,
-                                                             bool covariance_form) {
+template <typename T, int D>
+__device__ __forceinline__ void bwd_epilogue_one(const T* __restrict__ g, const T* __restrict__ rs, T* __restrict__ o,
+                                                 bool covariance_form);
+
+// SOLE: the workgroup covers all points of its mixture (one chunk).  Its per-Gaussian sums are then final: they go
+// to `sums` with plain stores (no zero fill before the launch, no atomics) and the workgroup itself carries them on
+// to grad_mixture at the end, which saves the fill and the epilogue launch of small problems.
+template <typename T, int D, int P, bool NEED_GM, bool NEED_GX, bool SOLE>
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 3 : 1)))
+void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture, const T* __restrict__ xes,
+                        T* __restrict__ sums, T* __restrict__ grad_xes, T* __restrict__ grad_mixture, int L, int M, int N,
+                        int Bx, int Lx, int chunks, int xes_shared, int n_mixtures, bool covariance_form) {
     constexpr int G = 1 + D + D * D;
     constexpr int S = Rec<T, D>::kStride;
     constexpr int NR = Sums<D>::k;
@@ -314,7 +320,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
             __syncthreads();
             T* __restrict__ dst = sums + (size_t(bl) * M + g0) * NR;
             for (int i = threadIdx.x; i < cnt * NR; i += kBlock) {
-                atomic_add(&dst[i], block_sums[i]);
+                if (SOLE) dst[i] = block_sums[i]; else atomic_add(&dst[i], block_sums[i]);
                 block_sums[i] = T(0);
             }
         }
@@ -350,6 +356,13 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
             }
         }
     }
+    if (NEED_GM && SOLE) {
+        __syncthreads();            // the sums this workgroup stored are visible to all of its lanes
+        for (int i = threadIdx.x; i < M; i += kBlock) {
+            const size_t at = size_t(bl) * M + i;
+            bwd_epilogue_one<T, D>(mixture + at * G, sums + at * NR, grad_mixture + at * G, covariance_form);
+        }
+    }
 }
 
 // Epilogue, one lane per Gaussian: (R0, R1, R2) -> (dw, db, dC), written to grad_mixture in the reference's
@@ -361,17 +374,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T
 // carried on to S as the reference's Python layer does (transpose of pack_mixture's argument, then
 // MatrixInverse.backward, src/gmc/cpp/extensions/math/matrix_inverse.py:30-33):  dS = -S^-1 dC^T S^-1.
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void eval_bwd_epilogue_kernel(const T* __restrict__ mixture,
-                                                                   const T* __restrict__ sums,
-                                                                   T* __restrict__ grad_mixture, size_t n_gaussians,
-                                                                   bool covariance_form) {
-    constexpr int G = 1 + D + D * D;
-    constexpr int NR = Sums<D>::k;
-    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
-    if (i >= n_gaussians) return;
-    const T* g = mixture + i * G;
-    const T* rs = sums + i * NR;
-    T* o = grad_mixture + i * G;
+__device__ __forceinline__ void bwd_epilogue_one(const T* __restrict__ g, const T* __restrict__ rs, T* __restrict__ o,
+                                                 bool covariance_form) {
     const Derived<D> dv = derive<T, D>(g, covariance_form);
     double c[D][D];
     load_inverse_covariance<T, D>(g + 1 + D, covariance_form, c);
@@ -480,6 +484,18 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_epilogue_kernel(const T* __re
     }
 }
 
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void eval_bwd_epilogue_kernel(const T* __restrict__ mixture,
+                                                                   const T* __restrict__ sums,
+                                                                   T* __restrict__ grad_mixture, size_t n_gaussians,
+                                                                   bool covariance_form) {
+    constexpr int G = 1 + D + D * D;
+    constexpr int NR = Sums<D>::k;
+    const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n_gaussians) return;
+    bwd_epilogue_one<T, D>(mixture + i * G, sums + i * NR, grad_mixture + i * G, covariance_form);
+}
+
 // ---- host-side launchers ------------------------------------------------------------------------------
 
 static int pick_points_per_lane(int N, int BL) {
@@ -555,15 +571,14 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
-template <typename T, int D, bool GM, bool GX>
-static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T* sums, T* grad_xes, const gmc_shape& s,
-                            int xes_shared, bool cov, hipStream_t stream) {
+// Points per lane of the backward pair kernel.  A workgroup covers 4 wavefronts x 16 P points.  Larger P amortises
+// the per-Gaussian row reductions (about 4 (1 + D + D(D+1)/2) instructions per step and lane) over more pairs but
+// pads the last chunk more; pick the P with the least modelled work that still leaves enough workgroups for the
+// 256 CUs.  Every P from 2 to 16 (8 in double) has its instance: with powers of two only, 784 points (a 28 x 28
+// grid) ran as one chunk of 1024 with 23 % of the lanes' points padding; P = 13 covers them with 832.
+template <typename T, int D>
+static int bwd_points_per_lane(const gmc_shape& s) {
     const size_t BL = size_t(s.B) * s.L;
-    // A workgroup covers 4 wavefronts x 16 P points.  Larger P amortises the per-Gaussian row reductions (about
-    // 4 (1 + D + D(D+1)/2) instructions per step and lane) over more pairs but pads the last chunk more; pick the P
-    // with the least modelled work that still leaves enough workgroups for the 256 CUs.
-    // Every P from 2 to 16 (8 in double) has its instance: with powers of two only, 784 points (a 28 x 28 grid) ran
-    // as one chunk of 1024 with 23 % of the lanes' points padding; P = 13 covers them with 832.
     constexpr int p_max = sizeof(T) == 8 ? 8 : 16;
     const double pair_cost = D == 2 ? 18.0 : 30.0, reduce_cost = 5.0 * Sums<D>::k;
     int P = 2;
@@ -575,10 +590,18 @@ static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T
         const double cost = double(chunks) * span * (pair_cost + reduce_cost / cand);
         if (cost < best) { best = cost; P = cand; }
     }
+    return P;
+}
+
+template <typename T, int D, bool GM, bool GX, bool SOLE>
+static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T* sums, T* grad_xes, T* grad_mixture,
+                            const gmc_shape& s, int P, int xes_shared, bool cov, hipStream_t stream) {
+    const size_t BL = size_t(s.B) * s.L;
+    constexpr int p_max = sizeof(T) == 8 ? 8 : 16;
     const int span = 64 * P;
     const int chunks = (s.N + span - 1) / span;
     const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
-#define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL), cov)
+#define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX, SOLE><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL), cov)
     if constexpr (p_max > 8) {
         switch (P) {
             case 16: GMC_BWD(16); return;
@@ -618,12 +641,17 @@ static int launch_bwd(const T* grad_out, const T* mixture, const T* xes, T* grad
         if (need_gx) zero_async(grad_xes, n_x, stream);
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    if (need_gm) zero_async(sums, n_gauss * Sums<D>::k, stream);
+    const int P = bwd_points_per_lane<T, D>(s);
+    // one chunk per mixture: the pair kernel's workgroups finish the gradient of their mixture themselves
+    const bool sole = need_gm && s.N <= 64 * P;
+    if (need_gm && !sole) zero_async(sums, n_gauss * Sums<D>::k, stream);
     if (need_gx && xes_shared) zero_async(grad_xes, n_x, stream);
-    if (need_gm && need_gx) launch_bwd_main<T, D, true, true>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, cov, stream);
-    else if (need_gm) launch_bwd_main<T, D, true, false>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, cov, stream);
-    else if (need_gx) launch_bwd_main<T, D, false, true>(grad_out, mixture, xes, sums, grad_xes, s, xes_shared, cov, stream);
-    if (need_gm) {
+    if (sole && need_gx) launch_bwd_main<T, D, true, true, true>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
+    else if (sole) launch_bwd_main<T, D, true, false, true>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
+    else if (need_gm && need_gx) launch_bwd_main<T, D, true, true, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
+    else if (need_gm) launch_bwd_main<T, D, true, false, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
+    else if (need_gx) launch_bwd_main<T, D, false, true, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
+    if (need_gm && !sole) {
         const size_t blocks = (n_gauss + kBlock - 1) / kBlock;
         eval_bwd_epilogue_kernel<T, D><<<dim3(unsigned(blocks)), dim3(kBlock), 0, stream>>>(mixture, sums, grad_mixture, n_gauss, cov);
     }

@@ -104,6 +104,44 @@ def test_every_points_per_lane_instance(dtype):
         _check(mix, xes, gout, dtype, tag=f"points per lane {p}, D{D}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_one_chunk_per_mixture(dtype):
+    """When one chunk of points covers a mixture, the workgroups of the backward pair kernel finish grad_mixture
+    themselves (plain stores of the sums, no zero fill, no epilogue launch).  256 mixtures make a launch take one
+    chunk whenever that covers N.  Covered: two tiles of Gaussians, per-mixture and broadcast points, every
+    combination of the need flags, and the covariance form (gm.evaluate)."""
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    tol, fl = TOL[dtype], FLOOR[dtype]
+    for D, M, N, broadcast in ((2, 280, 150, False), (3, 270, 100, True)):
+        mix, xes, gout = _case(8, 32, M, N, D, 7100 + D, broadcast)
+        _check(mix, xes, gout, dtype, tag=f"one chunk D{D}")
+        mix, xes, gout = mix.astype(npdt), xes.astype(npdt), gout.astype(npdt)
+        rgm, rgx = o.evaluate_inversed_backward(gout, mix, xes)
+        _, gmix, gxes = _run(mix, xes, gout, dtype, need_m=True, need_x=False)
+        assert gxes is None and rel_l2(gmix, rgm, fl) <= tol
+        _, gmix, gxes = _run(mix, xes, gout, dtype, need_m=False, need_x=True)
+        assert gmix is None and rel_l2(gxes, rgx, fl) <= tol
+        # the same mixture given by its covariances
+        B, L = mix.shape[:2]
+        c = o.split(mix.astype(np.float64))[2]
+        cov_mix = np.concatenate([mix[..., :1 + D].astype(np.float64), np.linalg.inv(c).reshape(B, L, M, D * D)], axis=-1)
+        cov_mix = cov_mix.astype(npdt)
+        m = torch.tensor(cov_mix, device=DEV, requires_grad=True)
+        x = torch.tensor(xes, device=DEV, requires_grad=True)
+        out = gm.evaluate(m, x)
+        out.backward(torch.tensor(gout, device=DEV))
+        c64 = np.linalg.inv(o.split(cov_mix.astype(np.float64))[2])
+        inv_mix = np.concatenate([cov_mix[..., :1 + D].astype(np.float64), c64.reshape(B, L, M, D * D)], axis=-1)
+        ref = o.evaluate_inversed(inv_mix, xes.astype(np.float64))
+        rgm, rgx = o.evaluate_inversed_backward(gout.astype(np.float64), inv_mix, xes.astype(np.float64))
+        gs = -(c64 @ np.swapaxes(rgm[..., 1 + D:].reshape(B, L, M, D, D), -1, -2) @ c64)
+        gmix = m.grad.cpu().numpy()
+        assert rel_l2(out.detach().cpu().numpy(), ref, fl) <= tol
+        assert rel_l2(gmix[..., :1 + D], rgm[..., :1 + D], fl) <= tol
+        assert rel_l2(gmix[..., 1 + D:], gs.reshape(B, L, M, D * D), fl) <= tol * 2
+        assert rel_l2(x.grad.cpu().numpy(), rgx, fl) <= tol
+
+
 @pytest.mark.parametrize("D", [2, 3])
 def test_matrix_core_forward_shapes(D):
     """float32 shapes that take the wide matrix-core forward kernel (more than 128 components and either many
