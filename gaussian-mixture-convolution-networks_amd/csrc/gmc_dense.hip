@@ -157,6 +157,9 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_rc_kernel(const T* __restrict
 // row r works on Gaussian 4k + r of the tile in step k, column c on the points {c, c + 16, ..., c + 16 (P-1)} of
 // the wavefront's 16 P points.  The per-Gaussian sums are then reduced over one DPP row only (4 shifts, no
 // cross-row traffic) once per step and Gaussian, and dL/dx is reduced over the 4 rows once per kernel.
+// copies of a tile's per-Gaussian sums in LDS: one per wavefront in float, a shared one in double (80 KB otherwise)
+template <typename T> struct SumCopies { static constexpr int k = sizeof(T) == 4 ? 4 : 1; };
+
 template <typename T, int D, int P, bool NEED_GM, bool NEED_GX, bool CENTRED>
 __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __restrict__ block_sums, int begin, int end,
                                              int row, const T (&x)[P][D], const T (&go)[P], T (&gx)[P][D]) {
@@ -251,9 +254,13 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
             }
             if ((threadIdx.x & 7) == 7) {
                 if (idx >= 0) {
-                    T* dst = block_sums + idx * NR + (high ? 1 : 0);
+                    T* dst = block_sums + idx * NR + (high ? NR / 2 : 0);
 #pragma unroll
-                    for (int i = 0; i < NR / 2; ++i) atomic_add(&dst[2 * i], half[i]);
+                    for (int i = 0; i < NR / 2; ++i) {
+                        // float: every wavefront meets every Gaussian of a tile once and has its own copy of the sums,
+                        // so a plain store does (LDS float atomics are serialised lane by lane); double: one copy
+                        if constexpr (SumCopies<T>::k > 1) dst[i] = half[i]; else atomic_add(&dst[i], half[i]);
+                    }
                 }
             }
         }
@@ -277,7 +284,7 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
     constexpr int NR = Sums<D>::k;
     constexpr int kWavePoints = 16 * P;
     __shared__ __attribute__((aligned(16))) T lds[(kTile + 6) * S];
-    __shared__ T block_sums[NEED_GM ? kTile * NR : 1];
+    __shared__ __attribute__((aligned(16))) T block_sums[NEED_GM ? SumCopies<T>::k * kTile * NR : 1];
     __shared__ int counts[10];
 
     int bl, chunk;
@@ -307,21 +314,32 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
         go[p] = n < N ? grad_out[size_t(bl) * N + nc] : T(0);   // padding lanes contribute nothing
     }
     if (NEED_GM) {
-        for (int i = threadIdx.x; i < kTile * NR; i += kBlock) block_sums[i] = T(0);
+        // (the per-wavefront copies need no zero fill: a tile's entries are all written before they are read)
+        if constexpr (SumCopies<T>::k == 1)
+            for (int i = threadIdx.x; i < kTile * NR; i += kBlock) block_sums[i] = T(0);
     }
 
     for (int g0 = 0; g0 < M; g0 += kTile) {
         const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
         stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0 / kHalfLog2e, lds, counts, covariance_form);
         const int centred_start = counts[8], padded_total = counts[9];
-        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, false>(lds, block_sums, 0, centred_start, row, x, go, gx);
-        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, true>(lds, block_sums, centred_start, padded_total, row, x, go, gx);
+        T* wave_sums = block_sums + (NEED_GM && SumCopies<T>::k > 1 ? wave * kTile * NR : 0);
+        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, false>(lds, wave_sums, 0, centred_start, row, x, go, gx);
+        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, true>(lds, wave_sums, centred_start, padded_total, row, x, go, gx);
         if (NEED_GM) {
             __syncthreads();
             T* __restrict__ dst = sums + (size_t(bl) * M + g0) * NR;
             for (int i = threadIdx.x; i < cnt * NR; i += kBlock) {
-                if (SOLE) dst[i] = block_sums[i]; else atomic_add(&dst[i], block_sums[i]);
-                block_sums[i] = T(0);
+                // entry i holds sum k of Gaussian j at [j][k / 2 + (k odd ? NR / 2 : 0)] of every wavefront's copy
+                const int j = i / NR, k = i - j * NR;
+                const int at = j * NR + (k >> 1) + ((k & 1) ? NR / 2 : 0);
+                T v = block_sums[at];
+                if constexpr (SumCopies<T>::k > 1) {
+                    v = (v + block_sums[kTile * NR + at]) + (block_sums[2 * kTile * NR + at] + block_sums[3 * kTile * NR + at]);
+                } else {
+                    block_sums[at] = T(0);
+                }
+                if (SOLE) dst[i] = v; else atomic_add(&dst[i], v);
             }
         }
     }
