@@ -32,7 +32,7 @@ PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}     # MI355X vector peaks
 VALU_NOTE = ("compute-bound against the FP32 peak of 157.3 TFLOP/s (matrix = packed vector rate); the kernels issue "
              "unpacked FP32 vector instructions (measured issue rate: one wave64 FMA per 2.3 cycles and SIMD = 137 TFLOP/s), the float32 forward kernel takes y = u x - u b "
              "from the bf16 matrix cores")
-MEASURED_TRAFFIC_BYTES = {"C4": 158939 * 1024 * 2.0 + 567798 * 1024 * 1.0,
+MEASURED_TRAFFIC_BYTES = {"C4": 158833 * 1024 * 2.0 + 553648 * 1024 * 1.0,
                           # LBVH traversal kernels of C5 (aabb_mode "reference"): backward, forward
                           "C5": 18586.3 * 1024 * 2.0 + 18644.2 * 1024 * 1.0,
                           "C5_fwd": 21522.2 * 1024 * 2.0 + 4090.9 * 1024 * 1.0}
