@@ -282,6 +282,30 @@ def test_evaluate_covariance_form(golden_dir):
         assert rel_l2(got, ref) < 1e-5
 
 
+@pytest.mark.parametrize("D", [2, 3])
+def test_spatial_scale_invariance(D):
+    """Protocol of src/gmc/test_mixture.py:154-191 (a scaling per layer and dimension, then a uniform one per batch
+    entry and layer; points on a grid, shared by all mixtures, scaled along).  spatial_scale keeps the weights
+    (integrals), so the scaled mixture at the scaled points has the values of the original divided by the product
+    of the factors."""
+    g = torch.Generator().manual_seed(3100 + D)
+    torch.manual_seed(3100 + D)                 # generate_random_mixtures draws from the global generator
+    B, L, M = 10, 8, 3
+    mix = gm.generate_random_mixtures(B, L, M, D, pos_radius=1, cov_radius=1, weight_min=-0.5, weight_max=4)
+    mix = mix.double().to(DEV)                  # float64: the test pins the invariance, not float32 rounding
+    axis = torch.arange(-1, 1, 0.25, dtype=torch.float64)
+    xes = torch.stack(torch.meshgrid([axis] * D, indexing="ij"), -1).reshape(1, 1, -1, D).to(DEV)
+    ref = gm.evaluate(mix, xes)
+    for shape in ((1, L, D), (B, L, 1)):
+        factors = (torch.rand(shape, generator=g, dtype=torch.float64) * 19.5 + 0.5).to(DEV)
+        scaled = gm.spatial_scale(mix, factors)
+        per_dim = factors.expand(shape[0], L, D)
+        xes_scaled = (xes.expand(B, L, -1, D) * per_dim.unsqueeze(-2)).contiguous()
+        volume = per_dim.prod(-1).unsqueeze(-1)
+        got = gm.evaluate(scaled, xes_scaled) * volume
+        assert rel_l2(got.cpu().numpy(), ref.cpu().numpy(), FLOOR[torch.float64]) <= 1e-10
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("D", [2, 3])
 def test_evaluate_covariance_form_fused_inverse(dtype, D):
