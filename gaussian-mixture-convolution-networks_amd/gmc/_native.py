@@ -130,12 +130,40 @@ def check_input(mixture: torch.Tensor, xes: torch.Tensor) -> Shape:
     return Shape(B, L, M, N, d, Bx, Lx, GMC_F32 if mixture.dtype == torch.float32 else GMC_F64)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device) -> int:
+    """handle of torch's current HIP stream on `device` (the raw getter skips the construction of a Stream object)"""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
 
 
+class _on:
+    """Makes `device` the current HIP device for the duration of a call, like torch.cuda.device, but without its
+    bookkeeping when the device is current already (the usual case; these wrappers sit on launch-bound paths)."""
+    __slots__ = ("idx", "prev")
+
+    def __init__(self, device):
+        self.idx = device.index
+        self.prev = -1
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if self.idx is not None and cur != self.idx:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+
+    def __exit__(self, *exc):
+        if self.prev >= 0:
+            torch.cuda.set_device(self.prev)
+        return False
+
+
 def _p(t):
-    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else ctypes.c_void_p(0)
+    """device address as a plain int (ctypes converts it to void*); None (a null pointer) for absent or empty tensors"""
+    return t.data_ptr() if t is not None and t.numel() > 0 else None
 
 
 def eval_fwd(mixture: torch.Tensor, xes: torch.Tensor, covariance_form: bool = False) -> torch.Tensor:
@@ -143,7 +171,7 @@ def eval_fwd(mixture: torch.Tensor, xes: torch.Tensor, covariance_form: bool = F
     shape = check_input(mixture, xes)
     out = torch.empty((shape.B, shape.L, shape.N), dtype=mixture.dtype, device=mixture.device)
     fn = lib().gmc_eval_cov_fwd if covariance_form else lib().gmc_eval_fwd
-    with torch.cuda.device(mixture.device):
+    with _on(mixture.device):
         check(fn(_p(mixture), _p(xes), _p(out), ctypes.byref(shape), _stream(mixture.device)))
     return out
 
@@ -168,7 +196,7 @@ def eval_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool, cova
     grad_xes = torch.empty_like(xes) if need_xes else torch.zeros_like(xes)
     if not (need_mixture or need_xes):
         return grad_mixture, grad_xes
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
         ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
         fn = lib().gmc_eval_cov_bwd if covariance_form else lib().gmc_eval_bwd
@@ -181,7 +209,7 @@ def eval_componentwise_fwd(mixture: torch.Tensor, xes: torch.Tensor, covariance_
     """values [B, L, N, M] of every (point, component) pair"""
     shape = check_input(mixture, xes)
     out = torch.empty((shape.B, shape.L, shape.N, shape.M), dtype=mixture.dtype, device=mixture.device)
-    with torch.cuda.device(mixture.device):
+    with _on(mixture.device):
         check(lib().gmc_eval_componentwise_fwd(_p(mixture), _p(xes), _p(out), ctypes.byref(shape), int(covariance_form),
                                                _stream(mixture.device)))
     return out
@@ -200,7 +228,7 @@ def eval_componentwise_bwd(grad_output, mixture, xes, need_mixture: bool, need_x
     grad_xes = torch.empty_like(xes) if need_xes else torch.zeros_like(xes)
     if not (need_mixture or need_xes):
         return grad_mixture, grad_xes
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
         ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
         check(lib().gmc_eval_componentwise_bwd(_p(grad_output), _p(mixture), _p(xes), _p(grad_mixture), _p(grad_xes),
@@ -234,7 +262,7 @@ class Bvh:
         self.covariance_form = bool(covariance_form)
         cfg = _bvh_config(aabb_threshold, aabb_mode, covariance_form)
         dev = mixture.device
-        with torch.cuda.device(dev):
+        with _on(dev):
             nbytes = lib().gmc_bvh_bytes(ctypes.byref(self.shape))
             self.blob = torch.empty((max(nbytes, 8),), dtype=torch.uint8, device=dev)
             check(lib().gmc_bvh_build(_p(mixture), _p(xes), _p(self.blob), nbytes, ctypes.byref(self.shape),
@@ -246,7 +274,7 @@ class Bvh:
         s = self.shape
         lo = torch.empty((s.B, s.L, s.M, s.D), dtype=self.dtype, device=self.device)
         up = torch.empty_like(lo)
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             check(lib().gmc_bvh_export_boxes(_p(self.blob), _p(lo), _p(up), ctypes.byref(s), _stream(self.device)))
         return lo, up
 
@@ -256,14 +284,14 @@ class Bvh:
         n = max(2 * s.M - 1, 0)
         nodes = torch.empty((s.B, s.L, n, 4), dtype=torch.int32, device=self.device)
         nb = torch.empty((s.B, s.L, n, 2 * s.D), dtype=self.dtype, device=self.device)
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             check(lib().gmc_bvh_export_nodes(_p(self.blob), _p(nodes), _p(nb), ctypes.byref(s), _stream(self.device)))
         return nodes, nb
 
     def candidate_stats(self):
         """int32 [2]: pieces of long candidate lists published for the backward pass, pool ints in use"""
         stats = torch.empty((2,), dtype=torch.int32, device=self.device)
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             check(lib().gmc_bvh_export_candidate_stats(_p(self.blob), _p(stats), ctypes.byref(self.shape),
                                                        _stream(self.device)))
         return stats
@@ -281,7 +309,7 @@ def eval_bvh_fwd(mixture, xes, bvh: Bvh) -> torch.Tensor:
     shape = check_input(mixture, xes)
     _check_bvh_shape(shape, bvh)
     out = torch.empty((shape.B, shape.L, shape.N), dtype=mixture.dtype, device=mixture.device)
-    with torch.cuda.device(mixture.device):
+    with _on(mixture.device):
         check(lib().gmc_eval_bvh_fwd(_p(mixture), _p(xes), _p(bvh.blob), _p(out), ctypes.byref(shape),
                                      _stream(mixture.device)))
     return out
@@ -301,7 +329,7 @@ def eval_bvh_bwd(grad_output, mixture, xes, bvh: Bvh, need_mixture: bool, need_x
     grad_xes = torch.empty_like(xes) if need_xes else torch.zeros_like(xes)
     if not (need_mixture or need_xes):
         return grad_mixture, grad_xes
-    with torch.cuda.device(dev):
+    with _on(dev):
         ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
         ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
         fn = lib().gmc_eval_bvh_cov_bwd if bvh.covariance_form else lib().gmc_eval_bvh_bwd
@@ -341,7 +369,7 @@ def convolution_fwd(data: torch.Tensor, kernels: torch.Tensor) -> torch.Tensor:
     shape = check_convolution_input(data, kernels)
     out = torch.empty((shape.B, shape.Cout, shape.Nd * shape.Cin * shape.Nk, data.shape[-1]), dtype=data.dtype,
                       device=data.device)
-    with torch.cuda.device(data.device):
+    with _on(data.device):
         check(lib().gmc_convolution_fwd(_p(data), _p(kernels), _p(out), ctypes.byref(shape), _stream(data.device)))
     return out
 
@@ -357,7 +385,7 @@ def convolution_bwd(grad_out: torch.Tensor, data: torch.Tensor, kernels: torch.T
         raise RuntimeError("grad_output must be contiguous")
     grad_data = torch.empty_like(data) if need_data else torch.zeros_like(data)
     grad_kernels = torch.empty_like(kernels) if need_kernels else torch.zeros_like(kernels)
-    with torch.cuda.device(data.device):
+    with _on(data.device):
         check(lib().gmc_convolution_bwd(_p(grad_out), _p(data), _p(kernels), _p(grad_data), _p(grad_kernels),
                                         ctypes.byref(shape), int(need_data), int(need_kernels), _stream(data.device)))
     return grad_data, grad_kernels
