@@ -286,6 +286,9 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
     __shared__ __attribute__((aligned(16))) T lds[(kTile + 6) * S];
     __shared__ __attribute__((aligned(16))) T block_sums[NEED_GM ? SumCopies<T>::k * kTile * NR : 1];
     __shared__ int counts[10];
+    // three float workgroups share a compute unit's LDS; measured: three of 53.6 KB are resident together, three of
+    // 54.0 KB are not
+    static_assert(sizeof(T) == 8 || sizeof(lds) + sizeof(block_sums) + 64 <= 53760, "LDS of the backward pair kernel");
 
     int bl, chunk;
     map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
