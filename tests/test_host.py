@@ -38,6 +38,11 @@ def test_c_abi_rejects_bad_shapes_without_launching():
     assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(2, 3, 4, 5, 3, 2, 3, 7)), null) == -2
     assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(2, 3, 4, 5, 3, 3, 3, 0)), null) == -3
     assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(2, 3, 4, -5, 3, 2, 3, 0)), null) == -3
+    # sizes beyond what the 32-bit launch grids and per-mixture indices cover
+    assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(65536, 65536, 4, 5, 3, 65536, 65536, 0)), null) == -3
+    assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(1, 1, 2 ** 30, 5, 3, 1, 1, 0)), null) == -3
+    assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(S(4096, 4096, 4, 2 ** 20, 3, 1, 1, 0)), null) == -3
+    assert lib.gmc_eval_bwd_workspace_bytes(ctypes.byref(S(1, 1, 2 ** 30, 5, 3, 1, 1, 0))) == 0
     assert lib.gmc_eval_fwd(null, null, null, ctypes.byref(ok), null) == -4
     assert lib.gmc_eval_fwd(null, null, null, None, null) == -4
     assert lib.gmc_eval_bwd(null, null, null, null, null, null, 0, ctypes.byref(ok), 1, 1, null) == -4
