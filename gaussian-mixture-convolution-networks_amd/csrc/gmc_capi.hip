@@ -9,6 +9,8 @@ size_t dense_backward_workspace_bytes(const gmc_shape& s);
 int dense_backward(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
                    void* workspace, const gmc_shape& s, bool need_gm, bool need_gx, bool covariance_form,
                    hipStream_t stream);
+int dense_backward_static(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                          const gmc_shape& s, bool need_gm, bool need_gx, bool covariance_form, hipStream_t stream);
 
 int check_shape(const gmc_shape* s) {
     if (!s) return GMC_E_NULL;
@@ -30,7 +32,7 @@ int check_shape(const gmc_shape* s) {
 
 extern "C" {
 
-int gmc_abi_version(void) { return 5; }
+int gmc_abi_version(void) { return 6; }
 
 const char* gmc_error_string(int code) {
     switch (code) {
@@ -42,6 +44,7 @@ const char* gmc_error_string(int code) {
         case GMC_E_WORKSPACE: return "workspace too small";
         case GMC_E_LAUNCH: return "HIP launch failed";
         case GMC_E_CONFIG: return "invalid BVH configuration";
+        case GMC_E_TOO_LARGE: return "the per-Gaussian sums of this shape exceed the static scratch array (GMC_STATIC_SCRATCH_BYTES); use gmc_eval_bwd with a workspace";
         default: return "unknown error";
     }
 }
@@ -69,9 +72,10 @@ size_t gmc_eval_bwd_workspace_bytes(const gmc_shape* shape) {
     return gmc::dense_backward_workspace_bytes(*shape);
 }
 
+// use_static: the per-Gaussian sums go to the library's static device array instead of a caller's workspace
 static int eval_bwd_impl(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
                          void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
-                         int need_grad_xes, bool covariance_form, void* stream) {
+                         int need_grad_xes, bool covariance_form, void* stream, bool use_static = false) {
     const int rc = gmc::check_shape(shape);
     if (rc != GMC_OK) return rc;
     const bool gm = need_grad_mixture != 0, gx = need_grad_xes != 0;
@@ -81,6 +85,9 @@ static int eval_bwd_impl(const void* grad_out, const void* mixture, const void* 
     if (gm && n_g > 0 && !grad_mixture) return GMC_E_NULL;
     if (gx && n_x > 0 && !grad_xes) return GMC_E_NULL;
     if (n_g > 0 && n_x > 0 && (!grad_out || !mixture || !xes)) return GMC_E_NULL;
+    if (use_static)
+        return gmc::dense_backward_static(grad_out, mixture, xes, grad_mixture, grad_xes, *shape, gm, gx, covariance_form,
+                                          (hipStream_t)stream);
     if (gm && n_g > 0 && n_x > 0) {
         if (workspace_bytes < gmc::dense_backward_workspace_bytes(*shape)) return GMC_E_WORKSPACE;
         if (!workspace) return GMC_E_NULL;
@@ -101,6 +108,13 @@ int gmc_eval_cov_bwd(const void* grad_out, const void* mixture, const void* xes,
                      int need_grad_xes, void* stream) {
     return eval_bwd_impl(grad_out, mixture, xes, grad_mixture, grad_xes, workspace, workspace_bytes, shape,
                          need_grad_mixture, need_grad_xes, true, stream);
+}
+
+int gmc_eval_bwd_static(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                        const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, int covariance_form,
+                        void* stream) {
+    return eval_bwd_impl(grad_out, mixture, xes, grad_mixture, grad_xes, nullptr, 0, shape, need_grad_mixture,
+                         need_grad_xes, covariance_form != 0, stream, true);
 }
 
 }  // extern "C"

@@ -14,9 +14,18 @@
 //     into (dw, db, dC).
 #include "gmc_common.h"
 
+#include <atomic>
 #include <type_traits>
 
 namespace gmc {
+
+// Device memory of the allocation-free backward entry point: the per-Gaussian sums of dense_backward live here
+// instead of in a caller's workspace.  Every GPU the library runs on holds its own copy of the array at its own
+// address; host code never uses the array's name as an address, only what hipGetSymbolAddress returned for the
+// device that is current (kept per device below).
+static __device__ __align__(256) unsigned char scratch[GMC_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> scratch_address[kMaxDevices];
 
 // float32 forward pair kernel with y = u x - u b on the matrix cores (gmc_dense_mfma.hip)
 bool dense_forward_f32(const float* mixture, const float* xes, float* out, const gmc_shape& s, bool covariance_form,
@@ -712,6 +721,22 @@ int dense_backward(const void* grad_out, const void* mixture, const void* xes, v
     if (s.dtype == GMC_F32) return s.D == 2 ? GMC_CALL(float, 2) : GMC_CALL(float, 3);
     return s.D == 2 ? GMC_CALL(double, 2) : GMC_CALL(double, 3);
 #undef GMC_CALL
+}
+
+// The same launches with the sums in this library's own static device array: no allocation anywhere.  The address
+// of the array on the current device is looked up once per device (first call there) and kept.  All calls on one
+// GPU share the array: the launches clear the part they use themselves, and calls that overlap on one GPU race.
+int dense_backward_static(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                          const gmc_shape& s, bool need_gm, bool need_gx, bool covariance_form, hipStream_t stream) {
+    if (need_gm && dense_backward_workspace_bytes(s) > size_t(GMC_STATIC_SCRATCH_BYTES)) return GMC_E_TOO_LARGE;
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return GMC_E_LAUNCH;
+    void* ptr = scratch_address[device].load(std::memory_order_acquire);
+    if (!ptr) {
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return GMC_E_LAUNCH;
+        scratch_address[device].store(ptr, std::memory_order_release);
+    }
+    return dense_backward(grad_out, mixture, xes, grad_mixture, grad_xes, ptr, s, need_gm, need_gx, covariance_form, stream);
 }
 
 }  // namespace gmc

@@ -16,7 +16,8 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 5
+ABI_VERSION = 6
+STATIC_SCRATCH_BYTES = 64 << 20
 
 
 class Shape(ctypes.Structure):
@@ -61,6 +62,7 @@ def lib() -> ctypes.CDLL:
     l.gmc_eval_bwd_workspace_bytes.restype = sz
     l.gmc_eval_bwd_workspace_bytes.argtypes = [shp]
     l.gmc_eval_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
+    l.gmc_eval_bwd_static.argtypes = [vp, vp, vp, vp, vp, shp, ci, ci, ci, vp]
     l.gmc_eval_cov_fwd.argtypes = [vp, vp, vp, shp, vp]
     l.gmc_eval_cov_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
     l.gmc_eval_componentwise_fwd.argtypes = [vp, vp, vp, shp, ci, vp]

@@ -31,7 +31,8 @@ enum {
     GMC_E_NULL = -4,       /* a required pointer is NULL */
     GMC_E_WORKSPACE = -5,  /* workspace smaller than the matching *_workspace_bytes() */
     GMC_E_LAUNCH = -6,     /* the HIP runtime refused a launch (hipGetLastError) */
-    GMC_E_CONFIG = -7      /* unknown aabb mode / invalid threshold */
+    GMC_E_CONFIG = -7,     /* unknown aabb mode / invalid threshold */
+    GMC_E_TOO_LARGE = -8   /* gmc_eval_bwd_static: the shape needs more than GMC_STATIC_SCRATCH_BYTES of scratch */
 };
 
 /* shape of one call; replaces gpe::MixtureAndXesNs (src/gmc/cpp/extensions/util/mixture.h:9-17) */
@@ -74,6 +75,19 @@ int gmc_eval_cov_fwd(const void* mixture, const void* xes, void* out, const gmc_
 int gmc_eval_cov_bwd(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
                      void* workspace, size_t workspace_bytes, const gmc_shape* shape, int need_grad_mixture,
                      int need_grad_xes, void* stream);
+
+/* gmc_eval_bwd_static has no counterpart in the reference.  It is gmc_eval_bwd / gmc_eval_cov_bwd (covariance_form
+ * != 0) for callers that cannot allocate device memory or pass a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  The per-Gaussian partial sums live in a static device array
+ * of GMC_STATIC_SCRATCH_BYTES inside the library (every GPU the library runs on holds it until the process ends);
+ * the call allocates nothing.  Shapes with gmc_eval_bwd_workspace_bytes(shape) > GMC_STATIC_SCRATCH_BYTES return
+ * GMC_E_TOO_LARGE (need_grad_mixture == 0 needs no scratch and is never refused).  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two streams, two threads) race; stream-ordered calls are safe, each clears
+ * what it uses.  The address of the array is looked up at the first call on a device. */
+#define GMC_STATIC_SCRATCH_BYTES (64u << 20)
+int gmc_eval_bwd_static(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
+                        const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, int covariance_form,
+                        void* stream);
 
 /* ---- component-wise evaluation --------------------------------------------------------------------
  * Replaces evaluate_componentwise_inversed / evaluate_componentwise (src/gmc/mixture.py:152-185, pure torch in the
