@@ -25,17 +25,52 @@ FLOP_BWD = {2: 30, 3: 52}
 # util/gaussian.h:82-95); reported for transparency only, never as the headline
 FLOP_FWD_LITERAL = {2: 15, 3: 27}
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}     # MI355X vector peaks
-# HBM bytes per launch of the backward pair kernel, from rocprofv3 counter runs of this script (summary under
-# profiles/): FETCH_SIZE KiB x 2.0 + WRITE_SIZE KiB x 1.0, factors from a 1 GiB copy kernel in the same runs.
-# The dense kernels are compute-bound on FP32 arithmetic.  MI355X's FP32 matrix rate equals its (packed) FP32 vector
-# rate, 157.3 TFLOP/s, which is the peak the metric names; "mfma" below means "against that compute peak".
-VALU_NOTE = ("compute-bound against the FP32 peak of 157.3 TFLOP/s (matrix = packed vector rate); the kernels issue "
-             "unpacked FP32 vector instructions (measured issue rate: one wave64 FMA per 2.3 cycles and SIMD = 137 TFLOP/s), the float32 forward kernel takes y = u x - u b "
-             "from the bf16 matrix cores")
-MEASURED_TRAFFIC_BYTES = {"C4": 158833 * 1024 * 2.0 + 553648 * 1024 * 1.0,
-                          # LBVH traversal kernels of C5 (aabb_mode "reference"): backward, forward
-                          "C5": 18586.3 * 1024 * 2.0 + 18644.2 * 1024 * 1.0,
-                          "C5_fwd": 21522.2 * 1024 * 2.0 + 4090.9 * 1024 * 1.0}
+# The dense kernels are bound by FP32 arithmetic.  MI355X's FP32 matrix rate equals its (packed) FP32 vector rate,
+# 157.3 TFLOP/s, which is the peak the metric names.  `bound` says which unit issues the kernel's arithmetic: "valu"
+# for the all-vector kernels, "mfma" for the forward kernel that takes the affine part from the matrix cores, "hbm"
+# for the memory- and latency-bound paths.
+VALU_NOTE = ("bound by vector-instruction issue against the FP32 peak of 157.3 TFLOP/s (MI355X's FP32 matrix rate equals "
+             "its packed FP32 vector rate); the kernels issue unpacked FP32 vector instructions (measured: one wave64 FMA "
+             "per 2.3 cycles and SIMD = 137 TFLOP/s)")
+MFMA_NOTE = VALU_NOTE + "; this kernel takes y = u x - u b from the bf16 matrix cores and keeps |y|^2, exp2 and the sum on the vector ALU"
+PROFILES = {"C4": "eval_dense_fwd_bwd_C4.md", "C5": "eval_bvh_build_fwd_bwd_C5.md"}
+
+
+def profile_traffic(workload: str, kernel_prefix: str):
+    """HBM bytes per launch of the kernel whose name starts with `kernel_prefix`, read from the committed counter
+    summary of this script under profiles/: FETCH_SIZE and WRITE_SIZE (KiB per dispatch), each scaled by what the
+    same counter shows for the 1 GiB device copy in the same run.  None when the summary or the kernel is missing."""
+    path = os.path.join(ROOT, "profiles", PROFILES.get(workload, ""))
+    if not os.path.isfile(path):
+        return None
+    tables, header = {}, None
+    for line in open(path):
+        cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")] if line.startswith("|") else None
+        if not cells:
+            header = None
+        elif cells[0] == "kernel":
+            header = cells[1:]
+        elif header and not set(cells[0]) <= set("-: "):
+            for name, value in zip(header, cells[1:]):
+                try:
+                    tables.setdefault(name, {})[cells[0]] = float(value)
+                except ValueError:
+                    pass
+    total = 0.0
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        rows = tables.get(counter, {})
+        mine = [v for k, v in rows.items() if k.startswith(kernel_prefix)]
+        copy = [v for k, v in rows.items() if k.startswith("__amd_rocclr_copyBuffer")]
+        if not mine or not copy or copy[0] <= 0:
+            return None
+        total += mine[0] * 1024.0 * (1048576.0 / copy[0])            # the copy moves 1 GiB each way
+    return total
+
+
+def median(values):
+    v = sorted(values)
+    n = len(v)
+    return v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
 
 
 def cpu_baseline(name: str):
@@ -65,11 +100,11 @@ def cpu_baseline(name: str):
     }
 
 
-def bench_bvh(args):
+def measure_bvh(aabb_mode: str, steps: int, warmup: int, copy_calibration: bool = False):
     """LBVH-culled path on C5 (3-D, float64, one mixture of 16384 Gaussians, 100000 points).  A step builds the
-    tree (the mixture changes every training step), evaluates forward and backward.  Throughput is reported in
-    dense-equivalent pairs (B L M N per step); the roofline entry is against HBM with the compulsory bytes of the
-    step (Gaussians, node boxes and links, points in, values and gradients out)."""
+    tree (the mixture changes every training step), evaluates forward and backward.  Returns the timings (HIP events
+    on the launch stream, medians over the steps; the step time is the wall clock over all steps) and the number of
+    pairs actually evaluated."""
     import torch
     from gmc import _native, synthetic
     wl, mix, xes, gout = synthetic.make_workload("C5")
@@ -80,7 +115,7 @@ def bench_bvh(args):
     def step(ev=None):
         if ev:
             ev[0].record()
-        bvh = _native.Bvh(mix, xes, 0.001, args.aabb_mode)
+        bvh = _native.Bvh(mix, xes, 0.001, aabb_mode)
         if ev:
             ev[1].record()
         out = _native.eval_bvh_fwd(mix, xes, bvh)
@@ -91,32 +126,50 @@ def bench_bvh(args):
             ev[3].record()
         return out, g
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    if args.copy_calibration:
+    if copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
     t0 = time.perf_counter()
-    for k in range(args.steps):
+    for k in range(steps):
         step(events[k])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms_step = wall * 1e3 / args.steps
-    build_ms, fwd_ms, bwd_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(3))
+    build_ms, fwd_ms, bwd_ms = (median([e[i].elapsed_time(e[i + 1]) for e in events]) for i in range(3))
     # pairs actually evaluated: points inside the cutoff box of a Gaussian (counted outside the timed region)
-    lo, up = _native.Bvh(mix, xes, 0.001, args.aabb_mode).boxes()
+    bvh = _native.Bvh(mix, xes, 0.001, aabb_mode)
+    lo, up = bvh.boxes()
     hits = 0
     for n0 in range(0, wl.N, 2048):
         x = xes[0, 0, n0:n0 + 2048].unsqueeze(1)                       # [n, 1, D]
         hits += int(((x >= lo[0, 0].unsqueeze(0)) & (x <= up[0, 0].unsqueeze(0))).all(dim=-1).sum().item())
+    return {"wl": wl, "ms_step": wall * 1e3 / steps, "build_ms": build_ms, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "hits": hits}
+
+
+def bvh_summary(r, aabb_mode):
+    """the C5 numbers of one box rule as a compact object (entry of `other_workloads`)"""
+    wl = r["wl"]
+    return {"aabb_mode": aabb_mode, "ms_per_step": r["ms_step"], "build_ms": r["build_ms"], "fwd_ms": r["fwd_ms"],
+            "bwd_ms": r["bwd_ms"], "dense_equivalent_pairs_per_s": wl.pairs / (r["ms_step"] * 1e-3),
+            "evaluated_pairs": r["hits"], "evaluated_pairs_per_s": r["hits"] / (r["ms_step"] * 1e-3)}
+
+
+def bench_bvh(args):
+    """`--workload C5`: the LBVH-culled step (build + forward + backward).  Throughput is reported in dense-equivalent
+    pairs (B L M N per step); the roofline entries are against HBM with the compulsory bytes of the pass (Gaussians,
+    node boxes and links, points in, values and gradients out)."""
+    r = measure_bvh(args.aabb_mode, args.steps, args.warmup, args.copy_calibration)
+    wl, ms_step, build_ms, fwd_ms, bwd_ms, hits = r["wl"], r["ms_step"], r["build_ms"], r["fwd_ms"], r["bwd_ms"], r["hits"]
     s, M, N, D = 8, wl.M, wl.N, 3
     bytes_fwd = M * 13 * s + (2 * M - 1) * (2 * D * s + 8) + N * (D + 1) * s
     bytes_bwd = bytes_fwd + N * s + M * 13 * s + N * D * s
+    reference_rule = args.aabb_mode == "reference"
     line = {
         "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
         "value": wl.pairs / (ms_step * 1e-3), "unit": "dense-equivalent Gaussian-point pairs/s (LBVH build + forward + backward step)",
@@ -130,14 +183,14 @@ def bench_bvh(args):
         "roofline": {"kernel": "bvh_traverse_kernel (backward mode; event pair also holds its zero-fill and epilogue)",
                      "bound": "hbm", "achieved": bytes_bwd / (bwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
                      "frac": bytes_bwd / (bwd_ms * 1e-3) / 8e12,
-                     "traffic": MEASURED_TRAFFIC_BYTES["C5"] if args.aabb_mode == "reference" else None,
+                     "traffic": profile_traffic("C5", "bvh_traverse_kernel<double, 3, 1") if reference_rule else None,
                      "launch_ms": bwd_ms, "algorithmic_bytes": bytes_bwd,
                      "bound_detail": "latency-bound: dependent tree-node fetches and double-precision leaf "
                                      "evaluation; the tree (about 4 MB) is fetched once per XCD (8 L2 caches)"},
         "roofline_fwd": {"kernel": "bvh_traverse_kernel (forward mode)", "bound": "hbm",
                          "achieved": bytes_fwd / (fwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
                          "frac": bytes_fwd / (fwd_ms * 1e-3) / 8e12,
-                         "traffic": MEASURED_TRAFFIC_BYTES["C5_fwd"] if args.aabb_mode == "reference" else None,
+                         "traffic": profile_traffic("C5", "bvh_traverse_kernel<double, 3, 0") if reference_rule else None,
                          "launch_ms": fwd_ms, "algorithmic_bytes": bytes_fwd},
     }
     if not args.no_cpu_baseline:
@@ -219,7 +272,7 @@ def bench_convolution(args):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_step = wall * 1e3 / args.steps
-    fwd_ms, bwd_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(2))
+    fwd_ms, bwd_ms = (median([e[i].elapsed_time(e[i + 1]) for e in events]) for i in range(2))
     small = (data.numel() + kernels.numel()) * 4
     bytes_fwd = n_out * G * 4 + small
     bytes_bwd = n_out * G * 4 + 2 * small                    # grad_out once; operands in, gradients out
@@ -295,7 +348,7 @@ def bench_componentwise(args):
         step(events[k])
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    fwd_ms, bwd_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(2))
+    fwd_ms, bwd_ms = (median([e[i].elapsed_time(e[i + 1]) for e in events]) for i in range(2))
     small = (mix.numel() + xes.numel()) * 4
     bytes_fwd = wl.pairs * 4 + small
     bytes_bwd = wl.pairs * 4 + 2 * small
@@ -377,7 +430,7 @@ def bench_layer(args):
         step(events[k])
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    eval_ms, fit_ms, norm_ms = (sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i in range(3))
+    eval_ms, fit_ms, norm_ms = (median([e[i].elapsed_time(e[i + 1]) for e in events]) for i in range(3))
     mixtures = wl.B * wl.L
     pairs_eval = 2 * wl.pairs                                   # forward and backward
     pairs_fit = 2 * mixtures * wl.M * wl.M
@@ -393,7 +446,7 @@ def bench_layer(args):
         "evaluate_fwd_bwd": {"ms": eval_ms, "pairs": pairs_eval},
         "fixed_point_iteration_to_relu": {"ms": fit_ms, "pairs": pairs_fit},
         "batch_norm_forward": {"ms": norm_ms, "pairs": pairs_norm},
-        "roofline": {"kernel": "eval_bwd_rc_kernel (covariance form, inside evaluate_fwd_bwd)", "bound": "mfma",
+        "roofline": {"kernel": "eval_bwd_rc_kernel (covariance form, inside evaluate_fwd_bwd)", "bound": "valu",
                      "bound_detail": "launch-bound at this size: the step is a chain of small launches and "
                                      "element-wise torch operations; the fraction is that of the whole evaluate "
                                      "forward + backward against the FP32 peak at 12 + 30 flop per pair",
@@ -429,6 +482,8 @@ def main():
                          "fitting and BatchNorm on the C2 shape")
     ap.add_argument("--aabb-mode", default="reference", choices=["reference", "tight"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="C4 only: leave out the `other_workloads` object (C1, C2, C3 and C5 measured after C4)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (known HBM traffic) so that a counter run of "
                          "this command holds the calibration kernel next to the evaluation kernels")
@@ -449,7 +504,66 @@ def main():
         return bench_componentwise(args)
     if args.workload == "layer":
         return bench_layer(args)
-    wl, mix, xes, gout = synthetic.make_workload(args.workload)
+    r = measure_dense(args.workload, args.steps, args.warmup, args.copy_calibration)
+    wl, ms_step, fwd_ms, bwd_ms = r["wl"], r["ms_step"], r["fwd_ms"], r["bwd_ms"]
+    D = wl.dims
+    dt = "f32" if wl.dtype == torch.float32 else "f64"
+    peak = PEAK_TFLOPS[dt]
+    fwd_tf = FLOP_FWD[D] * wl.pairs / (fwd_ms * 1e-3) / 1e12
+    bwd_tf = FLOP_BWD[D] * wl.pairs / (bwd_ms * 1e-3) / 1e12
+    step_tf = (FLOP_FWD[D] + FLOP_BWD[D]) * wl.pairs / (ms_step * 1e-3) / 1e12
+    fwd_kernel = r["fwd_kernel"]
+
+    line = {
+        "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
+        "value": wl.pairs / (ms_step * 1e-3), "unit": "Gaussian-point pairs/s (forward + backward step)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
+        "config": {"workload": f"{wl.name}: D={D} {dt} B={wl.B} L={wl.L} M={wl.M} N={wl.N}, dense all-pairs, "
+                               f"{wl.pairs:.4g} pairs per step, forward + backward (grad mixture and grad xes)"},
+        "timing": "ms_per_step: wall clock over all steps / steps; fwd.ms, roofline launch_ms: medians of per-step HIP event pairs",
+        "fwd": {"ms": fwd_ms, "pairs_per_s": wl.pairs / (fwd_ms * 1e-3), "tflops": fwd_tf, "frac_of_peak": fwd_tf / peak,
+                "tflops_by_reference_literal_count": FLOP_FWD_LITERAL[D] * wl.pairs / (fwd_ms * 1e-3) / 1e12},
+        "fwd_bwd": {"ms": ms_step, "pairs_per_s": wl.pairs / (ms_step * 1e-3), "tflops": step_tf,
+                    "frac_of_peak": step_tf / peak},
+        "roofline": {"kernel": "eval_bwd_rc_kernel (backward pair kernel; its zero-fill and epilogue launches, <1% of "
+                               "the time, are inside the event pair)",
+                     "bound": "valu", "bound_detail": VALU_NOTE, "achieved": bwd_tf, "peak": peak, "unit": "TFLOP/s", "frac": bwd_tf / peak,
+                     "traffic": profile_traffic(args.workload, "eval_bwd_rc_kernel"), "launch_ms": bwd_ms,
+                     "flop_per_pair": FLOP_BWD[D]},
+        "roofline_fwd": {"kernel": fwd_kernel, "bound": "mfma" if fwd_kernel == "eval_fwd_mfma_kernel" else "valu",
+                         "bound_detail": MFMA_NOTE if fwd_kernel == "eval_fwd_mfma_kernel" else VALU_NOTE,
+                         "achieved": fwd_tf, "peak": peak,
+                         "unit": "TFLOP/s", "frac": fwd_tf / peak, "launch_ms": fwd_ms, "flop_per_pair": FLOP_FWD[D],
+                         "traffic": profile_traffic(args.workload, fwd_kernel)},
+    }
+    if args.workload == "C4" and not args.no_other_workloads:
+        # every other configuration of the baseline, measured in the same process after the timed region of C4
+        others = {}
+        for name in ("C1", "C2", "C3"):
+            o = measure_dense(name, 20, 3)
+            w, d = o["wl"], o["wl"].dims
+            others[name] = {
+                "config": f"D={d} f32 B={w.B} L={w.L} M={w.M} N={w.N}, dense, {w.pairs:.4g} pairs",
+                "fwd_ms": o["fwd_ms"], "bwd_ms": o["bwd_ms"], "ms_per_step": o["ms_step"],
+                "fwd_pairs_per_s": w.pairs / (o["fwd_ms"] * 1e-3), "fwd_bwd_pairs_per_s": w.pairs / (o["ms_step"] * 1e-3),
+                "fwd_frac_of_peak": FLOP_FWD[d] * w.pairs / (o["fwd_ms"] * 1e-3) / 1e12 / PEAK_TFLOPS["f32"],
+                "fwd_bwd_frac_of_peak": (FLOP_FWD[d] + FLOP_BWD[d]) * w.pairs / (o["ms_step"] * 1e-3) / 1e12 / PEAK_TFLOPS["f32"],
+                "fwd_kernel": o["fwd_kernel"]}
+        others["C5"] = {"config": "D=3 f64 B=1 L=1 M=16384 N=100000, LBVH-culled (threshold 0.001): build + forward + backward per step",
+                        "by_aabb_mode": [bvh_summary(measure_bvh(mode, 20, 3), mode) for mode in ("reference", "tight")]}
+        line["other_workloads"] = others
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(line))
+
+
+def measure_dense(name: str, steps: int, warmup: int, copy_calibration: bool = False):
+    """Forward + backward (both gradients) of the dense path on the named workload; timings from HIP events on the
+    launch stream (medians over the steps), the step time from the wall clock over all steps."""
+    import torch
+    from gmc import _native, synthetic
+    wl, mix, xes, gout = synthetic.make_workload(name)
     dev = torch.device("cuda:0")
     mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)
     torch.cuda.synchronize()
@@ -465,55 +579,27 @@ def main():
             ev[2].record()
         return out, gm_, gx_
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    if args.copy_calibration:
+    if copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
     t0 = time.perf_counter()
-    for k in range(args.steps):
+    for k in range(steps):
         step(events[k])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-
-    ms_step = wall * 1e3 / args.steps
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
-    D = wl.dims
-    dt = "f32" if wl.dtype == torch.float32 else "f64"
-    peak = PEAK_TFLOPS[dt]
-    fwd_tf = FLOP_FWD[D] * wl.pairs / (fwd_ms * 1e-3) / 1e12
-    bwd_tf = FLOP_BWD[D] * wl.pairs / (bwd_ms * 1e-3) / 1e12
-    step_tf = (FLOP_FWD[D] + FLOP_BWD[D]) * wl.pairs / (ms_step * 1e-3) / 1e12
-    traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
-
-    line = {
-        "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
-        "value": wl.pairs / (ms_step * 1e-3), "unit": "Gaussian-point pairs/s (forward + backward step)",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
-        "config": {"workload": f"{wl.name}: D={D} {dt} B={wl.B} L={wl.L} M={wl.M} N={wl.N}, dense all-pairs, "
-                               f"{wl.pairs:.4g} pairs per step, forward + backward (grad mixture and grad xes)"},
-        "fwd": {"ms": fwd_ms, "pairs_per_s": wl.pairs / (fwd_ms * 1e-3), "tflops": fwd_tf, "frac_of_peak": fwd_tf / peak,
-                "tflops_by_reference_literal_count": FLOP_FWD_LITERAL[D] * wl.pairs / (fwd_ms * 1e-3) / 1e12},
-        "fwd_bwd": {"ms": ms_step, "pairs_per_s": wl.pairs / (ms_step * 1e-3), "tflops": step_tf,
-                    "frac_of_peak": step_tf / peak},
-        "roofline": {"kernel": "eval_bwd_rc_kernel (backward pair kernel; its zero-fill and epilogue launches, <1% of "
-                               "the time, are inside the event pair)",
-                     "bound": "mfma", "bound_detail": VALU_NOTE, "achieved": bwd_tf, "peak": peak, "unit": "TFLOP/s", "frac": bwd_tf / peak,
-                     "traffic": traffic, "launch_ms": bwd_ms, "flop_per_pair": FLOP_BWD[D]},
-        "roofline_fwd": {"kernel": "eval_fwd_mfma_kernel" if dt == "f32" else "eval_fwd_kernel", "bound": "mfma",
-                         "bound_detail": VALU_NOTE, "achieved": fwd_tf, "peak": peak,
-                         "unit": "TFLOP/s", "frac": fwd_tf / peak, "launch_ms": fwd_ms, "flop_per_pair": FLOP_FWD[D]},
-    }
-    if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.workload)
-    print(json.dumps(line))
+    import ctypes
+    shape = _native.check_input(mix, xes)
+    return {"wl": wl, "ms_step": wall * 1e3 / steps,
+            "fwd_ms": median([e[0].elapsed_time(e[1]) for e in events]),
+            "bwd_ms": median([e[1].elapsed_time(e[2]) for e in events]),
+            "fwd_kernel": _native.lib().gmc_eval_fwd_kernel_name(ctypes.byref(shape)).decode()}
 
 
 if __name__ == "__main__":

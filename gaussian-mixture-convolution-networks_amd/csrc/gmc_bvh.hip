@@ -50,8 +50,9 @@ struct BvhLayout {
     size_t cand_count;          // int [BL][ceil(N/64)]    candidate leaves of every point group, -1: not known
     size_t cand_list;           // int [BL][ceil(N/64)][kLeafCap], then a pool of pool_cap ints for the lists of
                                 // later rounds (all empty when the lists would exceed kCandCacheBytes)
-    size_t cand_ctl;            // int [4]                 pieces published, pool ints handed out, address of the points
-                                //                         the object was built for (64 bits)
+    size_t cand_stamp;          // uint64 [BL][ceil(N/64)] content stamp of the 64 points a group's list was gathered for
+    size_t cand_pieces;         // int2 [BL][ceil(N/64)]   slots of the piece table that hold this group's pieces (first, count)
+    size_t cand_ctl;            // int [4]                 pieces published, pool ints handed out, error flags (kErr*), -
     size_t pieces;              // int4 [pieces_max]       (point group, offset into cand_list, leaves, -)
     size_t piece_gx;            // T [pieces_max][D][64]   dL/dx of the pieces, added to grad_xes by the epilogue
     bool cand_cache;
@@ -83,19 +84,21 @@ __host__ __device__ inline int own_share(int n) {
     return pieces > 1 ? (n + pieces - 1) / pieces : n;
 }
 
+// A list describes the 64 points it was gathered for.  A traversal may be given other points than the build (or the
+// same tensor after an in-place change): every list therefore carries a 64-bit stamp of the coordinates of its 64
+// points, and a traversal uses a list only when the points it has just loaded give the same stamp; otherwise it
+// descends the tree (the build's point order is then only a poor grouping, the result is still right).
 struct CandidateCache {
-    int* count;
+    int* count;                     // null: this object keeps no lists
     int* list;
-    int* ctl;
+    int* ctl;                       // always there (error flags)
     int4* pieces;
+    unsigned long long* stamp;
+    int2* piece_range;
     int pieces_max, pool_cap, pool_base;
-    // The lists describe the points the object was built for.  A traversal may be given other points (the order of
-    // the build is then only a poor grouping, the result is still right), so the lists are used and written only
-    // when the traversal's points live where the build's points lived.
-    __device__ bool built_for(const void* xes) const {
-        return count != nullptr && reinterpret_cast<const unsigned long long*>(ctl)[1] == (unsigned long long)(size_t)xes;
-    }
 };
+constexpr int kErrStack = 1;            // a traversal's node stack was full and a push was dropped (results incomplete)
+constexpr int kErrSort = 2;             // a radix pass computed an output slot outside its segment
 constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
 constexpr int kSortBlocksMax = 256;                 // radix blocks per segment (more items per lane beyond that)
 constexpr int kCoarseOrderMax = 8192;               // point segments up to this size are ordered by 8 Morton bits only
@@ -158,7 +161,9 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
         l.pool_cap = l.cand_cache ? int(65536 + point_groups * 16) : 0;
         l.cand_count = take(l.cand_cache ? point_groups * 4 : 0);
         l.cand_list = take(l.cand_cache ? (point_groups * kLeafCap + l.pool_cap) * 4 : 0);
-        l.cand_ctl = take(l.cand_cache ? 16 : 0);
+        l.cand_stamp = take(l.cand_cache ? point_groups * 8 : 0);
+        l.cand_pieces = take(l.cand_cache ? point_groups * 8 : 0);
+        l.cand_ctl = take(16);
         l.pieces = take(size_t(l.pieces_max) * 16);
         l.piece_gx = take(size_t(l.pieces_max) * D * kWave * e);
     }
@@ -168,11 +173,13 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
 
 static CandidateCache candidate_cache(char* bvh, const BvhLayout& lay) {
     CandidateCache c{};
+    c.ctl = (int*)(bvh + lay.cand_ctl);
     if (!lay.cand_cache) return c;
     c.count = (int*)(bvh + lay.cand_count);
     c.list = (int*)(bvh + lay.cand_list);
-    c.ctl = (int*)(bvh + lay.cand_ctl);
     c.pieces = (int4*)(bvh + lay.pieces);
+    c.stamp = (unsigned long long*)(bvh + lay.cand_stamp);
+    c.piece_range = (int2*)(bvh + lay.cand_pieces);
     c.pieces_max = lay.pieces_max;
     c.pool_cap = lay.pool_cap;
     c.pool_base = int(lay.point_groups * kLeafCap);
@@ -352,9 +359,11 @@ __device__ __forceinline__ T block_bounds(const T (&lo)[D], const T (&hi)[D], T 
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_bounds_kernel(const T* __restrict__ mixture, int M, int blocks_per_mixture,
                                                            T* __restrict__ parts_g, unsigned box_blocks, const T* __restrict__ xes, int N,
-                                                           int blocks_per_xseg, T* __restrict__ parts_p) {
+                                                           int blocks_per_xseg, T* __restrict__ parts_p, int* __restrict__ ctl) {
     constexpr int G = 1 + D + D * D;
     __shared__ T red[2 * D][kBlock];
+    // first launch of a build: a new tree has no published pieces, an empty pool and no error
+    if (blockIdx.x == 0 && threadIdx.x < 4) ctl[threadIdx.x] = 0;
     T lo[D], hi[D];
     for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
     if (blockIdx.x < box_blocks) {
@@ -399,16 +408,18 @@ __device__ __forceinline__ uint32_t expand_bits3(uint32_t v) {
     return v;
 }
 
-// 10 bits per axis of the position normalised by `bounds`; an axis of zero extent maps to cell 0
+// 10 bits per axis of the position normalised by `bounds`, in the arithmetic of the tensors' own precision as the
+// reference does it (lbvh/bvh.cu:281-287: p -= lower; p /= upper - lower; lbvh/morton_code.h:145-168: cell =
+// uint32(p * 1024) clamped to 1023); an axis of zero extent (0/0 in the reference) maps to cell 0
 template <typename T, int D>
 __device__ __forceinline__ uint32_t morton30(const T* __restrict__ p, const T* __restrict__ bounds) {
     uint32_t code = 0;
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-        const double lo = double(bounds[d]), ext = double(bounds[D + d]) - lo;
-        double q = ext > 0.0 ? (double(p[d]) - lo) / ext * 1024.0 : 0.0;
-        q = q < 0.0 ? 0.0 : (q > 1023.0 ? 1023.0 : q);
-        q = (q == q) ? q : 0.0;
+        const T lo = bounds[d], ext = bounds[D + d] - lo;
+        T q = ext > T(0) ? (p[d] - lo) / ext * T(1024)   /* hipcc divides with correct rounding by default */ : T(0);
+        q = q < T(0) ? T(0) : (q > T(1023) ? T(1023) : q);
+        q = (q == q) ? q : T(0);
         code |= expand_bits3(uint32_t(q)) << (2 - d);
     }
     return code;
@@ -460,6 +471,7 @@ struct SortJob {
     uint32_t* hist;                      // [segments][blocks_per_seg][256]
     int count, items, blocks_per_seg, shift;
     unsigned blocks;                     // workgroups of this job in the launch
+    int* err;                            // error flags of the BVH object
 };
 
 // block histograms of the pass's digit, for two jobs in one launch (job b behind job a)
@@ -565,6 +577,8 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJo
             if (slot < uint32_t(count)) {          // always true for a consistent histogram; keeps a bug from writing out of bounds
                 j.keys_out[seg_off + slot] = key;
                 j.vals_out[seg_off + slot] = val;
+            } else {
+                atomicOr(j.err, kErrSort);
             }
         }
         __syncthreads();
@@ -795,13 +809,10 @@ template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __restrict__ children,
                                                                 const long long* __restrict__ enc_box, T* node_box,
                                                                 T* __restrict__ child_box, int M, size_t total,
-                                                                CandidateCache cache, size_t point_groups,
-                                                                const void* xes) {
+                                                                CandidateCache cache, size_t point_groups) {
     const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
     if (cache.count) {                               // a new tree: no candidate list is known yet
         for (size_t j = t; j < point_groups; j += size_t(gridDim.x) * kBlock) cache.count[j] = -1;
-        if (t < 2) cache.ctl[t] = 0;
-        if (t == 2) reinterpret_cast<unsigned long long*>(cache.ctl)[1] = (unsigned long long)(size_t)xes;
     }
     if (t >= total) return;
     const size_t bl = t / (M - 1);
@@ -863,6 +874,25 @@ constexpr int kTravBlock = kTravWaves * kWave;
 constexpr int kGroupsMax = 4;           // 64-point groups per workgroup (each descends the tree with its own wavefront)
 constexpr int kStageBatch = 20;         // candidate leaves a wavefront stages in LDS at a time
 constexpr int kTravSlots = 2 * 256;     // workgroups resident at once: two per compute unit
+
+// 64-bit stamp of the coordinates of a group's 64 points (lanes beyond the last point count as absent): what a
+// candidate list is valid for.  Wave-uniform.
+template <typename T, int D>
+__device__ __forceinline__ unsigned long long points_stamp(const T (&x)[D], bool valid, int lane) {
+    unsigned long long h = 0x9E3779B97F4A7C15ull * (unsigned long long)(lane + 1);
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        unsigned long long bits;
+        if constexpr (sizeof(T) == 4) bits = __builtin_bit_cast(unsigned int, x[d]);
+        else bits = __builtin_bit_cast(unsigned long long, x[d]);
+        h = (h ^ bits) * 0xff51afd7ed558ccdull;
+        h ^= h >> 29;
+    }
+    h = valid ? h : 0ull;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) h += __shfl_xor(h, off, 64);
+    return h;
+}
 
 template <typename T>
 __device__ __forceinline__ T wave_min(T v) {
@@ -934,13 +964,13 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     // instruction, those of floats are serialised lane by lane
     __shared__ double rsum_mem[kTravWaves][NEED_GM ? kStageBatch * NR : 1];
     __shared__ int2 pend[kGroupsMax][kPendMax];             // pieces of a group's list that wait to be published
+    __shared__ int piece_valid;                             // helper workgroups: the piece still describes the group's points
     const int per_mixture = (N + kWave - 1) / kWave;        // point groups of one mixture
     // The last `helpers` workgroups of a backward launch each take one published piece of a long candidate list
     // (no descent: one group, its points, a slice of its list); all others own `groups_per_workgroup` groups.
     // (Last, because most of them find no piece: at the end of the grid they start when compute units run idle.)
     const int owners = int(gridDim.x) - (MODE == 1 ? helpers : 0);
     const int piece = int(blockIdx.x) >= owners ? int(blockIdx.x) - owners : -1;
-    if (!cache.built_for(xes)) cache.count = nullptr;       // other points than the build's: no lists, no pieces
     int4 piece_desc = make_int4(0, 0, 0, 0);
     if (piece >= 0) {
         if (!cache.count) return;
@@ -968,6 +998,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     int first_round_leaves = 0, n_pend = 0;
     bool publish = false;                                   // the group's descent has ended with all parts in place
     int piece_slot = 0, publish_slot = 0, publish_flags = 0;
+    unsigned long long my_stamp = 0ull;                     // of the points this wavefront has loaded
     if (wave < groups) {
         // The groups of a workgroup lie far apart in Morton order, one in every quarter of the range and at
         // different places within the quarters: point groups with long candidate lists come in clusters (dense
@@ -991,6 +1022,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
         }
         pts[wave][D][lane] = g;
         pids[wave][lane] = valid ? pid : -1;
+        if (cache.count) my_stamp = points_stamp<T, D>(x, valid, lane);
         const bool any = group * kWave < N;
         if (lane == 0) {
             // a single Gaussian is a tree without internal nodes: its leaf is the only candidate
@@ -1001,6 +1033,15 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
         }
         sp = (any && M > 1) ? 1 : 0;
         if (piece >= 0) {
+            // A piece is worked on only while it is one of the pieces its group has published last, for points with
+            // the stamp of the ones loaded here; the owner of the group applies the same test to the list and
+            // otherwise evaluates all of it itself.
+            const int slot = piece_desc.x;
+            const int known = cache.count[slot];
+            const int2 range = cache.piece_range[slot];
+            const bool ok = known >= 0 && (known & kCandSplit) != 0 && piece >= range.x && piece < range.x + range.y &&
+                            cache.stamp[slot] == my_stamp;
+            if (lane == 0) piece_valid = ok ? 1 : 0;
             for (int i = lane; i < piece_desc.z; i += kWave) leaves[0][i] = cache.list[piece_desc.y + i];
             if (lane == 0) state[0][0] = piece_desc.z;
             sp = 0;
@@ -1010,7 +1051,15 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             // takes a whole single-round list and descends again for a list of several rounds.
             cache_slot = bl * per_mixture + group;
             const int known = __builtin_amdgcn_readfirstlane(cache.count[cache_slot]);
-            if (known >= 0) {
+            if (known >= 0 && cache.stamp[cache_slot] != my_stamp) {
+                // a list for other points (another tensor, or this one changed in place): descend.  The forward pass
+                // then replaces the list; a backward launch leaves the group's entries alone, because helper
+                // workgroups of the same launch may be reading them.
+                if (MODE == 1) cache_slot = -1;
+                // the descent writes the new list over the old one before it is known whether all its parts find
+                // room: the group counts as unknown from here on
+                else if (lane == 0) cache.count[cache_slot] = -1;
+            } else if (known >= 0) {
                 const int all = known & kCandMask;
                 const int n = (MODE == 1 && (known & kCandSplit)) ? own_share(all) : all;
                 if (MODE == 1 || !(known & kCandRounds)) {
@@ -1192,6 +1241,11 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     };
 
     __syncthreads();
+    if (piece >= 0 && !piece_valid) {
+        // the epilogue adds the dL/dx of every published piece: a piece that is not worked on contributes zeros
+        if (NEED_GX && threadIdx.x < D * kWave) piece_gx[size_t(piece) * D * kWave + threadIdx.x] = T(0);
+        return;
+    }
     // every descent step retires at least one of the M-1 internal nodes, each of which is pushed at most once
     for (int round = 0; round < M; ++round) {
         if (sp > 0) {
@@ -1234,8 +1288,12 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                     const int c = side == 0 ? ch.x : ch.y;
                     const unsigned long long mp = __ballot(push[side]), mh = __ballot(hit[side]);
                     const int at = sp + __popcll(mp & below);
-                    if (push[side] && at < kStackCap + 128) stk[at] = c;       // always in range, see the pop rule
+                    if (push[side]) {
+                        if (at < kStackCap + 128) stk[at] = c;                 // always in range, see the pop rule
+                        else atomicOr(&cache.ctl[2], kErrStack);               // a dropped push is reported, never silent
+                    }
                     sp += __popcll(mp);
+                    sp = sp < kStackCap + 128 ? sp : kStackCap + 128;
                     if (hit[side]) cand[n_leaf + __popcll(mh & below)] = ~c;
                     n_leaf += __popcll(mh);
                 }
@@ -1306,8 +1364,8 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
         if (publish) {
             publish = false;
             bool fits = true;
+            const int slot = n_pend > 0 ? __builtin_amdgcn_readfirstlane(piece_slot) : 0;
             if (n_pend > 0) {
-                const int slot = __builtin_amdgcn_readfirstlane(piece_slot);
                 fits = slot + n_pend <= cache.pieces_max;
                 wave_lds_fence();
                 // slots in range are always filled: a helper must never read an unwritten piece
@@ -1315,7 +1373,11 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                     cache.pieces[slot + lane] = fits ? make_int4(publish_slot, pend[wave][lane].x, pend[wave][lane].y, 0)
                                                      : make_int4(0, 0, 0, 0);
             }
-            if (fits && lane == 0) cache.count[publish_slot] = publish_flags;
+            if (fits && lane == 0) {
+                cache.stamp[publish_slot] = my_stamp;
+                cache.piece_range[publish_slot] = make_int2(slot, n_pend);
+                cache.count[publish_slot] = publish_flags;
+            }
         }
         if (!left_on_stack) break;
         __syncthreads();                                                // every wavefront has read this round's state
@@ -1363,7 +1425,7 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
     // worked on, one wavefront per piece, added to what the owners of the point groups have stored (several
     // pieces of a group meet here, hence atomics).
     if (blockIdx.x >= gaussian_blocks) {
-        if (!cache.built_for(xes)) return;                  // the traversal had no helpers then
+        if (!cache.count) return;                           // the traversal had no helpers then
         const int published = cache.ctl[0] < cache.pieces_max ? cache.ctl[0] : cache.pieces_max;
         const int per_mixture = (N + kWave - 1) / kWave;
         const int lane = threadIdx.x & 63;
@@ -1484,8 +1546,9 @@ static unsigned grid_for(size_t n) { return unsigned((n + kBlock - 1) / kBlock);
 // `count` (key, value) pairs: input (ka, va) on even passes and (kb, vb) on odd ones, output the other pair, the
 // last pass writes to (keys_out, vals_out).  A job without workgroups stands for "nothing to do in this pass".
 static SortJob sort_job(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, uint32_t* keys_out, uint32_t* vals_out,
-                        uint32_t* hist, size_t segments, int count, int first_bit, int passes, int pass) {
+                        uint32_t* hist, size_t segments, int count, int first_bit, int passes, int pass, int* err) {
     SortJob j = {};
+    j.err = err;
     if (segments == 0 || count == 0 || pass >= passes) return j;
     const bool odd = pass & 1;
     j.keys_in = odd ? kb : ka; j.vals_in = odd ? vb : va;
@@ -1531,7 +1594,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     const unsigned box_blocks = have_g ? unsigned(BL * bpm) : 0u, bound_blocks = sort_p ? unsigned(XL * nbp) : 0u;
     if (box_blocks + bound_blocks > 0)
         bvh_bounds_kernel<T, D><<<dim3(box_blocks + bound_blocks), dim3(kBlock), 0, st>>>(
-            mixture, M, bpm, parts_g, box_blocks, xes, N, nbp, parts_p);
+            mixture, M, bpm, parts_g, box_blocks, xes, N, nbp, parts_p, (int*)(bvh + lay.cand_ctl));
     MortonJob<T> mg = {}, mp = {};
     if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm)};
     if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx)};
@@ -1542,9 +1605,10 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     // land in a spare buffer, which must not be the input of the last pass.
     const int p_passes = N > kCoarseOrderMax ? 2 : 1;
     for (int pass = 0; pass < 4; ++pass) {
-        const SortJob jg = sort_job(ka, va, kb, vb, g_keys, g_order, (uint32_t*)(bvh + lay.hist_g), have_g ? BL : 0, M, 0, 4, pass);
+        const SortJob jg = sort_job(ka, va, kb, vb, g_keys, g_order, (uint32_t*)(bvh + lay.hist_g), have_g ? BL : 0, M, 0, 4, pass, (int*)(bvh + lay.cand_ctl));
         const SortJob jp = sort_job(pka, pva, pkb, pvb, p_passes == 1 ? pkb : pka, (uint32_t*)p_order,
-                                    (uint32_t*)(bvh + lay.hist_p), sort_p ? XL : 0, N, 30 - 8 * p_passes, p_passes, pass);
+                                    (uint32_t*)(bvh + lay.hist_p), sort_p ? XL : 0, N, 30 - 8 * p_passes, p_passes, pass,
+                                    (int*)(bvh + lay.cand_ctl));
         if (jg.blocks + jp.blocks == 0) continue;
         radix_hist_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
         radix_scatter_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
@@ -1560,7 +1624,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
             bvh_merge_kernel<T, D><<<dim3(unsigned((n + kMergeBlock - 1) / kMergeBlock)), dim3(kMergeBlock), 0, st>>>(
                 parent, node_range, node_box, enc_box, M, n);
             bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(
-                children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups, xes);
+                children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups);
         }
     }
     if (have_p && !sort_p) iota_segments_kernel<<<dim3(grid_for(XL * N)), dim3(kBlock), 0, st>>>(p_order, N, XL * N);
@@ -1727,12 +1791,24 @@ int gmc_bvh_export_candidate_stats(const void* bvh, int32_t* stats, const gmc_sh
     if (rc != GMC_OK) return rc;
     if (!stats) return GMC_E_NULL;
     const gmc::BvhLayout lay = gmc::bvh_layout(*shape);
-    if (lay.cand_cache && !bvh) return GMC_E_NULL;
-    if (lay.cand_cache)
-        gmc::copy_kernel<int32_t><<<dim3(1), dim3(gmc::kBlock), 0, (hipStream_t)stream>>>(
-            (const int32_t*)((const char*)bvh + lay.cand_ctl), stats, 2);
-    else
-        gmc::fill_zero_kernel<int32_t><<<dim3(1), dim3(gmc::kBlock), 0, (hipStream_t)stream>>>(stats, 2);
+    if (!bvh) return GMC_E_NULL;
+    gmc::copy_kernel<int32_t><<<dim3(1), dim3(gmc::kBlock), 0, (hipStream_t)stream>>>(
+        (const int32_t*)((const char*)bvh + lay.cand_ctl), stats, 4);
+    return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
+
+int gmc_bvh_export_leaf_order(const void* bvh, uint32_t* keys, int32_t* components, const gmc_shape* shape, void* stream) {
+    const int rc = check_bvh_shape(shape);
+    if (rc != GMC_OK) return rc;
+    const size_t n = size_t(shape->B) * shape->L * shape->M;
+    if (n == 0) return GMC_OK;
+    if (!bvh || !keys || !components) return GMC_E_NULL;
+    const gmc::BvhLayout lay = gmc::bvh_layout(*shape);
+    const unsigned blocks = unsigned((n + gmc::kBlock - 1) / gmc::kBlock < 4096 ? (n + gmc::kBlock - 1) / gmc::kBlock : 4096);
+    gmc::copy_kernel<uint32_t><<<dim3(blocks), dim3(gmc::kBlock), 0, (hipStream_t)stream>>>(
+        (const uint32_t*)((const char*)bvh + lay.g_keys), keys, n);
+    gmc::copy_kernel<int32_t><<<dim3(blocks), dim3(gmc::kBlock), 0, (hipStream_t)stream>>>(
+        (const int32_t*)((const char*)bvh + lay.leaf_comp), components, n);
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 

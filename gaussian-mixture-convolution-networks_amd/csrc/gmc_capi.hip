@@ -12,6 +12,8 @@ int dense_backward(const void* grad_out, const void* mixture, const void* xes, v
 int dense_backward_static(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
                           const gmc_shape& s, bool need_gm, bool need_gx, bool covariance_form, hipStream_t stream);
 
+const char* dense_forward_kernel_name(const gmc_shape& s);
+
 int check_shape(const gmc_shape* s) {
     if (!s) return GMC_E_NULL;
     if (s->D != 2 && s->D != 3) return GMC_E_DIMS;
@@ -65,6 +67,11 @@ int gmc_eval_fwd(const void* mixture, const void* xes, void* out, const gmc_shap
 
 int gmc_eval_cov_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream) {
     return eval_fwd_impl(mixture, xes, out, shape, true, stream);
+}
+
+const char* gmc_eval_fwd_kernel_name(const gmc_shape* shape) {
+    if (gmc::check_shape(shape) != GMC_OK) return "";
+    return gmc::dense_forward_kernel_name(*shape);
 }
 
 size_t gmc_eval_bwd_workspace_bytes(const gmc_shape* shape) {

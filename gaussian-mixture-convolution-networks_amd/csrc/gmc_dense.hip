@@ -548,6 +548,29 @@ static int pick_points_per_lane(int N, int BL) {
     return best;
 }
 
+// Which all-vector forward kernel a shape takes: `rc` > 0: the 4 x 16 layout with that many points per lane,
+// otherwise the one-Gaussian-per-step layout with `P` points per lane.
+struct FwdPlan { int P, chunks, rc; };
+
+static FwdPlan plan_fwd(const gmc_shape& s, bool is_double) {
+    const size_t BL = size_t(s.B) * s.L;
+    FwdPlan plan;
+    plan.P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
+    plan.chunks = (s.N + kBlock * plan.P - 1) / (kBlock * plan.P);
+    // the 4 x 16 layout covers the points in steps of 64 q: taken when that pads the last chunk clearly less
+    const int q_max = is_double ? 8 : 16;
+    int q_best = 0;
+    size_t covered_best = size_t(plan.chunks) * kBlock * plan.P;
+    covered_best -= covered_best / 16;                              // the other layout has to win by 6 %
+    for (int q = q_max; q >= 2; --q) {
+        const size_t q_chunks = (size_t(s.N) + 64 * q - 1) / (64 * q);
+        if (q > 2 && q_chunks * BL < 256) continue;
+        if (q_chunks * 64 * q < covered_best) { covered_best = q_chunks * 64 * q; q_best = q; }
+    }
+    plan.rc = q_best;
+    return plan;
+}
+
 template <typename T, int D>
 static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s, bool cov, hipStream_t stream) {
     const size_t BL = size_t(s.B) * s.L;
@@ -556,19 +579,11 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
     if constexpr (std::is_same<T, float>::value) {
         if (dense_forward_f32(mixture, xes, out, s, cov, stream)) return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    const int P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
-    const int chunks = (s.N + kBlock * P - 1) / (kBlock * P);
+    const FwdPlan plan = plan_fwd(s, sizeof(T) == 8);
+    const int P = plan.P, chunks = plan.chunks;
     {
-        // the 4 x 16 layout covers the points in steps of 64 q: taken when that pads the last chunk clearly less
         constexpr int q_max = sizeof(T) == 8 ? 8 : 16;
-        int q_best = 0;
-        size_t covered_best = size_t(chunks) * kBlock * P;
-        covered_best -= covered_best / 16;                              // the other layout has to win by 6 %
-        for (int q = q_max; q >= 2; --q) {
-            const size_t q_chunks = (size_t(s.N) + 64 * q - 1) / (64 * q);
-            if (q > 2 && q_chunks * BL < 256) continue;
-            if (q_chunks * 64 * q < covered_best) { covered_best = q_chunks * 64 * q; q_best = q; }
-        }
+        const int q_best = plan.rc;
         if (q_best > 0) {
             const int q_chunks = (s.N + 64 * q_best - 1) / (64 * q_best);
             const dim3 q_grid(unsigned(grid_mixtures(BL) * q_chunks));
@@ -706,6 +721,14 @@ int dense_forward(const void* mixture, const void* xes, void* out, const gmc_sha
     }
     if (s.D == 2) return launch_fwd<double, 2>((const double*)mixture, (const double*)xes, (double*)out, s, cov, stream);
     return launch_fwd<double, 3>((const double*)mixture, (const double*)xes, (double*)out, s, cov, stream);
+}
+
+bool dense_forward_f32_takes(const gmc_shape& s);
+
+// Names of the kernels a call of this shape launches (the pair kernels; fills and epilogues aside), for reports.
+const char* dense_forward_kernel_name(const gmc_shape& s) {
+    if (s.dtype == GMC_F32 && dense_forward_f32_takes(s)) return "eval_fwd_mfma_kernel";
+    return plan_fwd(s, s.dtype == GMC_F64).rc > 0 ? "eval_fwd_rc_kernel" : "eval_fwd_kernel";
 }
 
 size_t dense_backward_workspace_bytes(const gmc_shape& s) {

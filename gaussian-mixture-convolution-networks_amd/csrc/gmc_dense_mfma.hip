@@ -359,10 +359,14 @@ static void launch_fwd_variant(const float* mixture, const float* xes, float* ou
 // true: the matrix-core kernel handles the shape (more than 128 components per mixture and enough points to fill
 // the machine with 512-component tiles and 1024-point blocks); false: the caller uses the all-vector kernel, which
 // is as fast or faster below that (measured: within +-10 % for 64..128 components).
+bool dense_forward_f32_takes(const gmc_shape& s) {
+    const size_t BL = size_t(s.B) * s.L;
+    return s.M > 128 && (BL * size_t((s.N + 1023) / 1024) >= 512 || s.N >= 8192);
+}
+
 bool dense_forward_f32(const float* mixture, const float* xes, float* out, const gmc_shape& s, bool covariance_form,
                        hipStream_t stream) {
-    const size_t BL = size_t(s.B) * s.L;
-    if (!(s.M > 128 && (BL * size_t((s.N + 1023) / 1024) >= 512 || s.N >= 8192))) return false;
+    if (!dense_forward_f32_takes(s)) return false;
     if (s.D == 2) launch_fwd_variant<2, 8, 512, 512>(mixture, xes, out, s, covariance_form, stream);
     else launch_fwd_variant<3, 8, 512, 512>(mixture, xes, out, s, covariance_form, stream);
     return true;

@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
     l.gmc_error_string.argtypes = [ci]
     l.gmc_abi_version.restype = ci
     l.gmc_eval_fwd.argtypes = [vp, vp, vp, shp, vp]
+    l.gmc_eval_fwd_kernel_name.restype = ctypes.c_char_p
+    l.gmc_eval_fwd_kernel_name.argtypes = [shp]
     l.gmc_eval_bwd_workspace_bytes.restype = sz
     l.gmc_eval_bwd_workspace_bytes.argtypes = [shp]
     l.gmc_eval_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
@@ -77,6 +79,7 @@ def lib() -> ctypes.CDLL:
         l.gmc_bvh_export_boxes.argtypes = [vp, vp, vp, shp, vp]
         l.gmc_bvh_export_nodes.argtypes = [vp, vp, vp, shp, vp]
         l.gmc_bvh_export_candidate_stats.argtypes = [vp, vp, shp, vp]
+        l.gmc_bvh_export_leaf_order.argtypes = [vp, vp, vp, shp, vp]
         l.gmc_eval_bvh_fwd.argtypes = [vp, vp, vp, vp, shp, vp]
         l.gmc_eval_bvh_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
         l.gmc_eval_bvh_cov_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
@@ -192,6 +195,7 @@ def eval_bwd(grad_output, mixture, xes, need_mixture: bool, need_xes: bool, cova
         raise RuntimeError("grad_output dtype does not match with mixture dtype")
     if not grad_output.is_contiguous():
         raise RuntimeError("grad_output must be contiguous")
+    _check_grad_output_device(grad_output, mixture)
     dev = mixture.device
     # both gradients are always returned, all-zero when not required (parallel_implementation.cu:120-121,175)
     grad_mixture = torch.empty_like(mixture) if need_mixture else torch.zeros_like(mixture)
@@ -221,6 +225,7 @@ def eval_componentwise_bwd(grad_output, mixture, xes, need_mixture: bool, need_x
     shape = check_input(mixture, xes)
     if tuple(grad_output.shape) != (shape.B, shape.L, shape.N, shape.M):
         raise RuntimeError("grad_output has wrong shape")
+    _check_grad_output_device(grad_output, mixture)
     if grad_output.dtype != mixture.dtype:
         raise RuntimeError("grad_output dtype does not match with mixture dtype")
     if not grad_output.is_contiguous():
@@ -262,14 +267,34 @@ class Bvh:
                  aabb_mode: str = "reference", covariance_form: bool = False):
         self.shape = check_input(mixture, xes)
         self.covariance_form = bool(covariance_form)
-        cfg = _bvh_config(aabb_threshold, aabb_mode, covariance_form)
+        self._cfg = _bvh_config(aabb_threshold, aabb_mode, covariance_form)
         dev = mixture.device
         with _on(dev):
-            nbytes = lib().gmc_bvh_bytes(ctypes.byref(self.shape))
-            self.blob = torch.empty((max(nbytes, 8),), dtype=torch.uint8, device=dev)
-            check(lib().gmc_bvh_build(_p(mixture), _p(xes), _p(self.blob), nbytes, ctypes.byref(self.shape),
-                                      ctypes.byref(cfg), _stream(dev)))
+            self._nbytes = lib().gmc_bvh_bytes(ctypes.byref(self.shape))
+            self.blob = torch.empty((max(self._nbytes, 8),), dtype=torch.uint8, device=dev)
         self.dtype, self.device = mixture.dtype, dev
+        self.rebuild(mixture, xes)
+
+    def rebuild(self, mixture: torch.Tensor, xes: torch.Tensor):
+        """Builds the trees of another mixture (same shape, dtype and device) into this object; all kept candidate
+        lists are forgotten."""
+        shape = check_input(mixture, xes)
+        _check_bvh_shape(shape, self)
+        if mixture.device != self.device:
+            raise RuntimeError("the BVH lives on another device than the mixture")
+        with _on(self.device):
+            check(lib().gmc_bvh_build(_p(mixture), _p(xes), _p(self.blob), self._nbytes, ctypes.byref(self.shape),
+                                      ctypes.byref(self._cfg), _stream(self.device)))
+        # The object holds the Gaussians as they were now (leaf records, boxes): the forward pass reads only those,
+        # the backward epilogue reads the mixture it is given.  Remember which values the tree belongs to.
+        self._mixture_key = (mixture.data_ptr(), mixture._version)
+
+    def check_mixture(self, mixture: torch.Tensor):
+        """A Bvh is bound to the mixture values it was built from: other storage, or the same storage after an
+        in-place update, needs a new Bvh (the forward pass would evaluate the old values otherwise)."""
+        if (mixture.data_ptr(), mixture._version) != self._mixture_key:
+            raise RuntimeError("the BVH was built from other mixture values (another tensor, or this one was modified "
+                               "in place since): build a new Bvh")
 
     def boxes(self):
         """(lower, upper), each [B, L, M, D], in component order"""
@@ -290,9 +315,20 @@ class Bvh:
             check(lib().gmc_bvh_export_nodes(_p(self.blob), _p(nodes), _p(nb), ctypes.byref(s), _stream(self.device)))
         return nodes, nb
 
+    def leaf_order(self):
+        """(keys [B, L, M] int64 holding the 30-bit Morton codes of the leaves in sorted order, components [B, L, M]
+        int32 = component id of every leaf)"""
+        s = self.shape
+        keys = torch.empty((s.B, s.L, s.M), dtype=torch.int32, device=self.device)
+        comps = torch.empty((s.B, s.L, s.M), dtype=torch.int32, device=self.device)
+        with _on(self.device):
+            check(lib().gmc_bvh_export_leaf_order(_p(self.blob), _p(keys), _p(comps), ctypes.byref(s), _stream(self.device)))
+        return keys.to(torch.int64) & 0xFFFFFFFF, comps
+
     def candidate_stats(self):
-        """int32 [2]: pieces of long candidate lists published for the backward pass, pool ints in use"""
-        stats = torch.empty((2,), dtype=torch.int32, device=self.device)
+        """int32 [4]: pieces of long candidate lists published for the backward pass, pool ints in use, error flags
+        (0 unless the library has a bug: 1 = a traversal dropped a node, 2 = a sort pass went out of range), 0"""
+        stats = torch.empty((4,), dtype=torch.int32, device=self.device)
         with _on(self.device):
             check(lib().gmc_bvh_export_candidate_stats(_p(self.blob), _p(stats), ctypes.byref(self.shape),
                                                        _stream(self.device)))
@@ -307,9 +343,23 @@ def _check_bvh_shape(shape: Shape, bvh: "Bvh"):
                                f"build, {getattr(shape, name)} now)")
 
 
-def eval_bvh_fwd(mixture, xes, bvh: Bvh) -> torch.Tensor:
-    shape = check_input(mixture, xes)
+def _check_bvh_use(mixture, bvh: "Bvh", shape: Shape):
     _check_bvh_shape(shape, bvh)
+    if bvh.device != mixture.device:
+        raise RuntimeError("the BVH lives on another device than the mixture")
+    bvh.check_mixture(mixture)
+
+
+def _check_grad_output_device(grad_output, mixture):
+    if grad_output.device != mixture.device:
+        raise RuntimeError("grad_output must live on the device of the mixture")
+
+
+def eval_bvh_fwd(mixture, xes, bvh: Bvh) -> torch.Tensor:
+    """The forward pass evaluates the Gaussians stored in `bvh` at its build; `mixture` must be the tensor (and the
+    values) the Bvh was built from."""
+    shape = check_input(mixture, xes)
+    _check_bvh_use(mixture, bvh, shape)
     out = torch.empty((shape.B, shape.L, shape.N), dtype=mixture.dtype, device=mixture.device)
     with _on(mixture.device):
         check(lib().gmc_eval_bvh_fwd(_p(mixture), _p(xes), _p(bvh.blob), _p(out), ctypes.byref(shape),
@@ -319,7 +369,8 @@ def eval_bvh_fwd(mixture, xes, bvh: Bvh) -> torch.Tensor:
 
 def eval_bvh_bwd(grad_output, mixture, xes, bvh: Bvh, need_mixture: bool, need_xes: bool):
     shape = check_input(mixture, xes)
-    _check_bvh_shape(shape, bvh)
+    _check_bvh_use(mixture, bvh, shape)
+    _check_grad_output_device(grad_output, mixture)
     if tuple(grad_output.shape) != (shape.B, shape.L, shape.N):
         raise RuntimeError("grad_output has wrong shape")
     if grad_output.dtype != mixture.dtype:

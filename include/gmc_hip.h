@@ -53,6 +53,11 @@ int gmc_abi_version(void);
  */
 int gmc_eval_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream);
 
+/* Name of the forward pair kernel a call of this shape launches (for benchmark reports; no counterpart in the
+ * reference): "eval_fwd_mfma_kernel" (float32, more than 128 components, enough work for 512-component tiles),
+ * "eval_fwd_rc_kernel" or "eval_fwd_kernel" (all vector ALU, two layouts); "" for an invalid shape. */
+const char* gmc_eval_fwd_kernel_name(const gmc_shape* shape);
+
 /* gmc_eval_bwd replaces evaluate_inversed::parallel_backward
  *   (evaluate_inversed.cpp:22-34, parallel_implementation.cu:102-176, parallel_implementation_optimised_backward.cu:111-169).
  *   grad_mixture [B][L][M][1+D+D*D] and grad_xes [Bx][Lx][N][D] (summed over broadcast dims) are fully
@@ -145,20 +150,31 @@ int gmc_bvh_export_boxes(const void* bvh, void* lower, void* upper, const gmc_sh
  * nodes first, and node boxes [B][L][2M-1][2*D] (lower, upper). */
 int gmc_bvh_export_nodes(const void* bvh, int32_t* nodes, void* node_boxes, const gmc_shape* shape, void* stream);
 
-/* Diagnostics for tests (no counterpart in the reference): stats[0] = pieces of long candidate lists that the
- * forward traversals since the last build have handed to helper workgroups of the backward pass, stats[1] = ints
- * of the pool of later rounds' lists in use; `stats` is device memory for two int32. */
+/* Diagnostics for tests (no counterpart in the reference): `stats` is device memory for four int32.
+ * stats[0] = pieces of long candidate lists that the forward traversals since the last build have handed to helper
+ * workgroups of the backward pass, stats[1] = ints of the pool of later rounds' lists in use, stats[2] = error
+ * flags raised since the last build (1: a traversal's node stack was full and a push was dropped, so results are
+ * incomplete; 2: a radix pass of the build computed an output slot outside its segment; both stay 0 unless the
+ * library has a bug), stats[3] = 0. */
 int gmc_bvh_export_candidate_stats(const void* bvh, int32_t* stats, const gmc_shape* shape, void* stream);
+/* The leaves of every tree in their sorted order, for bit-exact tests of the integer part of the build:
+ * keys [B][L][M] = the 30-bit Morton code of each leaf's centre (lbvh/morton_code.h:77-85,145-168; position
+ * normalised by the bounds of the mixture's centres as lbvh/bvh.cu:281-287 does, in the tensors' precision),
+ * ascending, ties in component order -- the order of the reference's 64-bit keys `morton << 16 | component`
+ * (lbvh/morton_code.h:254-263, sorted at lbvh/bvh.cu:108); components [B][L][M] = component id of each leaf. */
+int gmc_bvh_export_leaf_order(const void* bvh, uint32_t* keys, int32_t* components, const gmc_shape* shape, void* stream);
 
 /* The first traversal after a build leaves the candidate leaves of every 64-point group in the BVH object
  * (when they fit into 64 MiB) and later traversals of the same object skip the tree descent, so the object is
- * written to by these calls: calls that use one BVH object must be ordered (same stream, or events).  A forward
+ * written to by these calls: calls that use one BVH object must be ordered (same stream, or events); calls on
+ * two streams race on the object.  A forward
  * pass also cuts candidate lists of more than 240 leaves into pieces; the backward pass that follows gives every
  * piece but the first to a workgroup of its own, so that a few point groups in dense regions do not hold up the
- * launch.  The lists belong to the points the object was built for: a traversal whose `xes` is another address than
- * the build's neither uses nor writes them (it is correct, only slower); the points at that address must not be
- * changed between the build and the traversals that use it.  `shape` must be the shape the object was built for:
- * the layout of the object follows from it and is not stored inside. */
+ * launch.  Every kept list carries a 64-bit stamp of the coordinates of its 64 points and is used only for points
+ * with the same stamp: a traversal with other points than the build's (another tensor, or the same one changed in
+ * place) descends the tree again and is correct, only slower.  The forward pass reads the Gaussians as they were at
+ * the build (leaf records inside the object); `mixture` there is not read.  `shape` must be the shape the object was
+ * built for: the layout of the object follows from it and is not stored inside. */
 int gmc_eval_bvh_fwd(const void* mixture, const void* xes, void* bvh, void* out, const gmc_shape* shape,
                      void* stream);
 int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh,

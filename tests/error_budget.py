@@ -1,0 +1,118 @@
+"""Per-element error budgets for the evaluation path (test infrastructure; numpy float64 on top of the oracle).
+
+A relative L2 norm over a whole tensor cannot see a few wrong elements among millions, so the parity tests also bound
+every element: |got - ref| <= budget.  The budget of an element is a first-order propagation of rounding errors
+through the pairs (Gaussian m, point n) that enter it.  With u the upper Cholesky factor of A = 1/2 log2(e) sym(C),
+y = u (x - b), q = |y|^2 and the pair value f = w norm exp2(-q):
+
+  dy    absolute error of y.  Shifted form (y = u x - u b without forming x - b, taken when bound_m = max_i sum_j
+        |u_ij b_j| is at most `limit`): CY eps bound_m, whatever the distance of the point.  Explicit x - b:
+        CC eps ya with ya_i = sum_j |u_ij| |t_j| >= |y_i| (products of mixed sign cancel for rotated, anisotropic
+        Gaussians).  `direct_form` (t^T C t straight from the stored matrix, as the culled path's leaves and the
+        reference do): the same with sum_ij |C_ij| |t_i| |t_j| in place of ya^2.
+  rel   relative error of f:  C0 eps (amplitude, exponential, accumulation over the other index) + CQ eps q (rounding
+        of q = |y|^2 itself) + 2 ln2 |y| dy;  direct form: C0 eps + CD eps sum_ij |C_ij t_i t_j| / 2 (every product of
+        the quadratic form is rounded, and they cancel).
+  out, dL/dw                  sum of |f| rel                    (resp. |f / w| |g| rel)
+  dL/dx, dL/db = -+ f g C t   sum of |f g| (rel |C t| + |u| dy / (1/2 log2 e)),   |C t| <= sqrt(2 v lambda_max(C))
+  dL/dC = -1/2 f g t t^T + cofactor term
+                              sum of |f g| (rel |t|^2 + 2 |t| dy / sigma_min(u)) / 2 + |cof| |w kappa g e| rel / (2 sqrt det)
+The gradient budgets are norm-wise per Gaussian (one value for all components of a position or a matrix).  Measured on
+the device over the whole test suite, the worst element uses 0.76 of its budget in float32 (0.34 for the matrix-core
+forward kernel at the edge of its shifted-form limit) and, with ORACLE_SHARE, 0.7 in float64; a wrong element (a
+dropped pair, a swapped index, a mis-rounded split) exceeds the budget by orders of magnitude.  float64 results are
+compared with a float64 oracle (numpy: other formulas, another summation order) whose own rounding is of the size of
+the error under test, hence the factor ORACLE_SHARE on the float64 budgets."""
+import numpy as np
+
+import gm_oracle as o
+
+EPS = {np.dtype(np.float32): 2.0 ** -24, np.dtype(np.float64): 2.0 ** -53}
+HALF_LOG2E = 0.72134752044448170368
+C0, CQ, CY, CC, CD = 48.0, 3.0, 6.0, 8.0, 12.0
+ORACLE_SHARE = {np.dtype(np.float32): 1.0, np.dtype(np.float64): 8.0}
+
+
+def shifted_bounds(mixture: np.ndarray) -> np.ndarray:
+    """bound_m = max_i sum_j |u_ij b_j| with u the upper Cholesky factor of 1/2 log2(e) sym(C): [B, L, M]"""
+    _, b, c = o.split(np.asarray(mixture, dtype=np.float64))
+    a = HALF_LOG2E * 0.5 * (c + np.swapaxes(c, -1, -2))
+    u = np.swapaxes(np.linalg.cholesky(a), -1, -2)
+    return np.abs(u * b[..., None, :]).sum(-1).max(-1)
+
+
+def budgets(mixture, xes, grad_output, dtype, limit, chunk=32, mask=None, direct_form=False):
+    """-> dict(out [B,L,N], gw [B,L,M], gb [B,L,M], gc [B,L,M], gx [Bx,Lx,N]): absolute error budgets per element
+    (gb, gc, gx: one value for all components).  `limit`: largest bound_m the kernel under test evaluates in the
+    shifted form (0: every Gaussian takes the explicit x - b).  `mask` [B,L,M,N]: pairs that count (culled variant)."""
+    eps = EPS[np.dtype(dtype)] * ORACLE_SHARE[np.dtype(dtype)]
+    mixture = np.asarray(mixture, dtype=np.float64)
+    xes = np.asarray(xes, dtype=np.float64)
+    g = np.abs(np.asarray(grad_output, dtype=np.float64))
+    B, L, M, _ = mixture.shape
+    N, D = xes.shape[2], xes.shape[3]
+    bound = shifted_bounds(mixture)
+    shifted = bound <= limit * (1.0 + 1e-9)
+    _, _, c_all = o.split(mixture)
+    sym = 0.5 * (c_all + np.swapaxes(c_all, -1, -2))
+    lam = np.linalg.eigvalsh(sym)
+    lam_min, lam_max = lam[..., 0], lam[..., -1]
+    u_all = np.swapaxes(np.linalg.cholesky(HALF_LOG2E * sym), -1, -2)
+    u_norm, u_min = np.sqrt(HALF_LOG2E * lam_max), np.sqrt(HALF_LOG2E * lam_min)
+    out = np.zeros((B, L, N))
+    gx = np.zeros((B, L, N))
+    gw, gb, gc = np.zeros((B, L, M)), np.zeros((B, L, M)), np.zeros((B, L, M))
+    kap = o.kappa(D)
+    for m0 in range(0, M, chunk):
+        m1 = min(M, m0 + chunk)
+        sl = (slice(None), slice(None), slice(m0, m1))
+        w, c, t, u, e, norm = o._pair_terms(mixture, xes, m0, m1)
+        if mask is not None:
+            e = e * mask[sl]
+        v = np.maximum(0.5 * np.einsum('blmni,blmni->blmn', t, u), 0.0)
+        ynorm = np.sqrt(HALF_LOG2E * 2.0 * v)
+        if direct_form:
+            ya = np.sqrt(HALF_LOG2E * np.einsum('blmni,blmij,blmnj->blmn', np.abs(t), np.abs(c), np.abs(t)))
+        else:
+            ya = np.sqrt((np.einsum('blmij,blmnj->blmni', np.abs(u_all[sl]), np.abs(t)) ** 2).sum(-1))
+        dy = eps * np.where(shifted[sl][..., None], CY * bound[sl][..., None], CC * ya)
+        if direct_form:
+            rel = eps * C0 + CD * eps * ya * ya / (2.0 * HALF_LOG2E)
+        else:
+            rel = eps * (C0 + CQ * ynorm * ynorm) + 2.0 * np.log(2.0) * ynorm * dy
+        f = np.abs(w * norm)[..., None] * e
+        gg = g[:, :, None, :]
+        out += (f * rel).sum(2)
+        gw[sl] = (norm[..., None] * e * gg * rel).sum(3)
+        ct = np.sqrt(2.0 * v * lam_max[sl][..., None])
+        pos = f * gg * (rel * ct + u_norm[sl][..., None] * dy / HALF_LOG2E)
+        gx += pos.sum(2)
+        gb[sl] = pos.sum(3)
+        tn = ynorm / u_min[sl][..., None]
+        cof = np.abs(o.cofactor(c)).max(axis=(-1, -2))
+        root = np.sqrt(np.linalg.det(c))
+        gc[sl] = 0.5 * (f * gg * (rel * tn * tn + 2.0 * tn * dy / u_min[sl][..., None])).sum(3) + \
+            cof * (np.abs(w * kap / (2.0 * root))[..., None] * e * gg * rel).sum(3)
+    Bx, Lx = xes.shape[0], xes.shape[1]
+    if Bx == 1 and B > 1:
+        gx = gx.sum(0, keepdims=True)
+    if Lx == 1 and L > 1:
+        gx = gx.sum(1, keepdims=True)
+    return dict(out=out, gw=gw, gb=gb, gc=gc, gx=gx)
+
+
+def worst_ratio(got, ref, budget, floor):
+    """max over elements of |got - ref| / (budget + floor); `floor`: absolute magnitude below which the precision
+    under test flushes to zero"""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    while budget.ndim < got.ndim:
+        budget = budget[..., None]
+    return float(np.max(np.abs(got - ref) / (budget + floor))) if got.size else 0.0
+
+
+def are_similar(a, b, precision):
+    """the reference's own per-element criterion (unittests/support.h:15-19): |a - b| / max(|a + b| / 2, 1) < precision"""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return np.abs(a - b) / np.maximum(np.abs(a + b) / 2.0, 1.0) < precision

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import cpu_ref
+import error_budget as eb
 import gm_oracle as o
 from conftest import rel_l2
 from gmc import _native
@@ -19,6 +20,15 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 TOL = {torch.float32: 1e-5, torch.float64: 1e-12}
 FLOOR = {torch.float32: 1e-30, torch.float64: 1e-290}
+
+
+BUDGET_USE = {}          # worst |error| / budget seen per (precision, tensor); printed at the end of the module
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _report_budget_use():
+    yield
+    print("\nworst |error| / budget per tensor (culled path):", {k: round(v, 4) for k, v in sorted(BUDGET_USE.items())}, flush=True)
 
 
 def _case(B, L, M, N, D, seed, broadcast=False, spread=4.0, cov_radius=0.3):
@@ -61,6 +71,16 @@ def _check_culled(mix, xes, gout, dtype, mode, tag=""):
     assert rel_l2(gmix[..., 1:1 + D], rgm[..., 1:1 + D], fl) <= tol, f"grad positions {tag}"
     assert rel_l2(gmix[..., 1 + D:], rgm[..., 1 + D:], fl) <= tol, f"grad inverse covariances {tag}"
     assert rel_l2(gxes, rgx, fl) <= tol, f"grad xes {tag}"
+    # every element against its error budget (the leaves are evaluated with an explicit x - b: no shifted form)
+    bud = eb.budgets(m_np, x_np, g_np, npdt, 0.0, mask=o.inside_mask(lo, up, x_np.astype(np.float64)),
+                     direct_form=True)
+    for got, want, b, what in ((out, ref, bud["out"], "out"), (gmix[..., 0], rgm[..., 0], bud["gw"], "grad weights"),
+                               (gmix[..., 1:1 + D], rgm[..., 1:1 + D], bud["gb"], "grad positions"),
+                               (gmix[..., 1 + D:], rgm[..., 1 + D:], bud["gc"], "grad inverse covariances"),
+                               (gxes, rgx, bud["gx"], "grad xes")):
+        ratio = eb.worst_ratio(got, want, b, fl)
+        BUDGET_USE[(str(npdt.__name__), what)] = max(BUDGET_USE.get((str(npdt.__name__), what), 0.0), ratio)
+        assert ratio <= 1.0, f"{what} {tag}: an element is off by {ratio:.3g} times its error budget"
     return out, ref
 
 
@@ -227,7 +247,6 @@ def test_candidate_lists_kept_in_the_bvh_object():
     """The first traversal after a build leaves the candidate list of every point group in the BVH object and later
     ones skip the descent: a second forward pass is bit-identical to the first, a backward pass gives the same
     gradients with and without a forward pass before it, and a rebuild into the same object forgets the lists."""
-    import ctypes
     mix, xes, gout = _case(2, 2, 300, 3000, 3, 640, cov_radius=0.1)
     m, x, g = (t.to(DEV).contiguous() for t in (mix, xes, gout))
     bvh = _native.Bvh(m, x, 0.001, "tight")
@@ -242,10 +261,7 @@ def test_candidate_lists_kept_in_the_bvh_object():
     # another mixture built into the same object
     mix2, _, _ = _case(2, 2, 300, 3000, 3, 641, cov_radius=0.1)
     m2 = mix2.to(DEV).contiguous()
-    cfg = _native._bvh_config(0.001, "tight")
-    with torch.cuda.device(m2.device):
-        _native.check(_native.lib().gmc_bvh_build(_native._p(m2), _native._p(x), _native._p(bvh.blob), bvh.blob.numel(),
-                                                  ctypes.byref(bvh.shape), ctypes.byref(cfg), _native._stream(m2.device)))
+    bvh.rebuild(m2, x)
     again = _native.eval_bvh_fwd(m2, x, bvh)
     assert torch.equal(again, _native.eval_bvh_fwd(m2, x, _native.Bvh(m2, x, 0.001, "tight")))
     assert not torch.equal(again, first)
@@ -278,12 +294,12 @@ def test_long_candidate_lists_are_shared_between_workgroups(broadcast):
     for dtype in (torch.float64, torch.float32):
         m, x, g = (t.to(dtype).to(DEV).contiguous() for t in (mix, xes, gout))
         bvh = _native.Bvh(m, x, 0.001, "tight")
-        assert n(bvh.candidate_stats()).tolist() == [0, 0]
+        assert n(bvh.candidate_stats()).tolist() == [0, 0, 0, 0]
         first = _native.eval_bvh_fwd(m, x, bvh)
         stats = n(bvh.candidate_stats()).tolist()
         assert stats[0] > 20 and stats[1] > 0, "the case is meant to publish pieces, some from later rounds"
         assert torch.equal(first, _native.eval_bvh_fwd(m, x, bvh))
-        assert n(bvh.candidate_stats()).tolist() == stats
+        assert n(bvh.candidate_stats()).tolist() == stats and stats[2] == 0
         gm_a, gx_a = _native.eval_bvh_bwd(g, m, x, bvh, True, True)
         gm_b, gx_b = _native.eval_bvh_bwd(g, m, x, _native.Bvh(m, x, 0.001, "tight"), True, True)
         tol = 1e-13 if dtype == torch.float64 else 2e-6       # two summation orders of the same terms
@@ -298,9 +314,10 @@ def test_long_candidate_lists_are_shared_between_workgroups(broadcast):
 
 
 def test_traversal_with_other_points_than_the_build():
-    """The lists and pieces kept in the BVH object describe the points it was built for.  A traversal that is given
-    other points (at another address) must neither use nor overwrite them: it gives what a BVH built for those points
-    gives, and the first points still find their lists afterwards."""
+    """Every candidate list kept in the BVH object carries a stamp of the 64 points it was gathered for.  A traversal
+    that is given other points (another tensor) must not use the lists and pieces of the build's points: it gives
+    what a BVH built for those points gives, forward and backward (the backward launch has helper workgroups for the
+    published pieces, which must all stand back), and the first points get their own results again afterwards."""
     mix, xes, gout = _crowded_case(1, 670, False)
     n = lambda t: t.cpu().numpy()
     m, xa, g = (t.to(DEV).contiguous() for t in (mix, xes, gout))
@@ -310,16 +327,103 @@ def test_traversal_with_other_points_than_the_build():
     stats = n(bvh.candidate_stats()).tolist()
     assert stats[0] > 0
     fresh = _native.Bvh(m, xb, 0.001, "tight")
-    other = _native.eval_bvh_fwd(m, xb, bvh)
-    assert rel_l2(n(other), n(_native.eval_bvh_fwd(m, xb, fresh))) <= 1e-13
-    assert n(bvh.candidate_stats()).tolist() == stats
+    # backward first: the lists and pieces of xa are all in place and none of them may be used
     gm_a, gx_a = _native.eval_bvh_bwd(g, m, xb, bvh, True, True)
     gm_b, gx_b = _native.eval_bvh_bwd(g, m, xb, fresh, True, True)
+    assert rel_l2(n(gm_a), n(gm_b)) <= 1e-13 and rel_l2(n(gx_a), n(gx_b)) <= 1e-13
+    assert n(bvh.candidate_stats()).tolist() == stats, "a backward pass publishes nothing"
+    other = _native.eval_bvh_fwd(m, xb, bvh)
+    assert rel_l2(n(other), n(_native.eval_bvh_fwd(m, xb, fresh))) <= 1e-13
+    gm_a, gx_a = _native.eval_bvh_bwd(g, m, xb, bvh, True, True)           # now with xb's own lists where they fitted
     assert rel_l2(n(gm_a), n(gm_b)) <= 1e-13 and rel_l2(n(gx_a), n(gx_b)) <= 1e-13
     assert torch.equal(first, _native.eval_bvh_fwd(m, xa, bvh))
     gm_c, gx_c = _native.eval_bvh_bwd(g, m, xa, bvh, True, True)
     gm_d, gx_d = _native.eval_bvh_bwd(g, m, xa, _native.Bvh(m, xa, 0.001, "tight"), True, True)
     assert rel_l2(n(gm_c), n(gm_d)) <= 1e-13 and rel_l2(n(gx_c), n(gx_d)) <= 1e-13
+    assert n(bvh.candidate_stats())[2] == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_points_changed_in_place_or_replaced_at_the_same_address(dtype):
+    """The points tensor is modified in place between the build / first traversal and later traversals, and then freed
+    and replaced by another tensor that the allocator puts at the same address: the kept candidate lists describe
+    points that are gone, and every result must still be the masked sum over the device's boxes for the points
+    that are there now (long lists with published pieces included)."""
+    mix, xes, gout = _crowded_case(2, 680, False)
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    tol, fl = TOL[dtype], FLOOR[dtype]
+    n = lambda t: t.cpu().numpy()
+    m, x, g = (t.to(dtype).to(DEV).contiguous() for t in (mix, xes, gout))
+    bvh = _native.Bvh(m, x, 0.001, "tight")
+    lo, up = (n(t).astype(np.float64) for t in bvh.boxes())
+    m_np, g_np = n(m), n(g)
+
+    def check(points, tag):
+        out = _native.eval_bvh_fwd(m, points, bvh)
+        gmix, gxes = _native.eval_bvh_bwd(g, m, points, bvh, True, True)
+        x_np = n(points)
+        ref = o.evaluate_inversed_bvh(m_np, x_np, lo, up)
+        rgm, rgx = o.evaluate_inversed_bvh_backward(g_np, m_np, x_np, lo, up)
+        assert rel_l2(n(out), ref, fl) <= tol, f"forward {tag}"
+        assert rel_l2(n(gmix), rgm, fl) <= tol, f"grad mixture {tag}"
+        assert rel_l2(n(gxes), rgx, fl) <= tol, f"grad xes {tag}"
+
+    check(x, "as built")
+    assert n(bvh.candidate_stats())[0] > 0, "the case is meant to publish pieces"
+    # in place: the points of the crowded region move out, others move in
+    x.mul_(-0.7)
+    x[:, :, ::3] += 0.25
+    check(x, "changed in place")                       # forward first: descends, replaces lists
+    x.mul_(-1.3)
+    gmix, gxes = _native.eval_bvh_bwd(g, m, x, bvh, True, True)   # backward first: stale lists and pieces all around
+    rgm, rgx = o.evaluate_inversed_bvh_backward(g_np, m_np, n(x), lo, up)
+    assert rel_l2(n(gmix), rgm, fl) <= tol and rel_l2(n(gxes), rgx, fl) <= tol
+    # another tensor at the same address
+    address, shape = x.data_ptr(), x.shape
+    del x
+    x2 = (torch.rand(shape, dtype=torch.float64, generator=torch.Generator().manual_seed(681)) * 2 - 1).mul(3.0).to(dtype).to(DEV)
+    if x2.data_ptr() != address:
+        print("the allocator placed the new points elsewhere; the case then equals 'other points'", flush=True)
+    check(x2, "replaced")
+    assert n(bvh.candidate_stats())[2] == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_leaf_order_is_bit_exact(dtype, D):
+    """Integer part of the build: the 30-bit Morton codes of the centres (lbvh/morton_code.h:77-85,145-168, positions
+    normalised as lbvh/bvh.cu:281-287 in the tensors' precision) and the sorted leaf order, which must be the
+    ascending order of the reference's keys `morton << 16 | component` (morton_code.h:254-263), i.e. a stable sort of
+    the codes.  Compared bit for bit with the oracle, duplicate codes (identical and nearly identical centres),
+    clustered centres and several mixtures included."""
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    for M, seed, spread in ((1, 1, 4.0), (2, 2, 4.0), (37, 3, 4.0), (300, 4, 0.01), (1000, 5, 4.0), (5000, 6, 50.0)):
+        mix, xes, _ = _case(2, 3, M, 70, D, seed=1200 + seed, spread=spread)
+        if M >= 37:
+            mix[:, :, 5:25] = mix[:, :, 5:6]                       # identical centres: identical codes, tie order matters
+            mix[:, :, 25:30, 1:1 + D] = mix[:, :, 25:26, 1:1 + D] * (1 + 1e-7)
+        if M >= 300:
+            mix[:, 1, ::2, 1:1 + D] *= 1e-3                        # half the centres crowd into a few cells
+        m = mix.to(dtype).to(DEV).contiguous()
+        bvh = _native.Bvh(m, xes.to(dtype).to(DEV).contiguous(), 0.001, "tight")
+        keys, comps = bvh.leaf_order()
+        torch.cuda.synchronize()
+        keys, comps = keys.cpu().numpy(), comps.cpu().numpy()
+        pos = m.cpu().numpy()[..., 1:1 + D]                        # values as the device sees them
+        lower, upper = pos.min(axis=2, keepdims=True), pos.max(axis=2, keepdims=True)
+        ext = (upper - lower).astype(npdt)
+        with np.errstate(invalid="ignore", divide="ignore"):
+            p01 = np.where(ext > 0, ((pos - lower).astype(npdt) / ext).astype(npdt), npdt(0))
+        codes = o.morton30(p01.astype(npdt)).astype(np.int64)
+        assert codes.max() < 2 ** 30
+        order = np.argsort(codes, axis=2, kind="stable")
+        assert np.array_equal(comps, order), f"leaf order M{M} D{D}"
+        assert np.array_equal(keys, np.take_along_axis(codes, order, axis=2)), f"sorted Morton codes M{M} D{D}"
+        assert n_errors(bvh) == 0
+
+
+def n_errors(bvh):
+    return int(bvh.candidate_stats().cpu().numpy()[2])
 
 
 def test_points_outside_every_box_and_need_flags():

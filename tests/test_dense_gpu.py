@@ -10,6 +10,7 @@ import pytest
 import torch
 
 import cpu_ref
+import error_budget as eb
 import gm_oracle as o
 from conftest import rel_l2
 from gmc import mixture as gm
@@ -21,6 +22,28 @@ TOL = {torch.float32: 1e-5, torch.float64: 1e-12}
 # magnitudes below these count as zero (float32 flushes them, the float64 oracle does not)
 FLOOR = {torch.float32: 1e-30, torch.float64: 1e-290}
 DEV = "cuda:0"
+# per-element criteria next to the norms: the reference's own (unittests/evaluate_inversed.cpp:20-21 with
+# unittests/support.h:15-19) and the error budgets of tests/error_budget.py
+SIMILAR = {torch.float32: 4e-5, torch.float64: 1e-10}
+# largest `bound` a kernel evaluates without forming x - b (float32: matrix-core forward kernel 32, vector kernels 16)
+SHIFT_LIMIT = {torch.float32: 32.0, torch.float64: 256.0}
+BUDGET_USE = {}          # worst |error| / budget seen per (precision, tensor); printed at the end of the module
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _report_budget_use():
+    yield
+    print("\nworst |error| / budget per tensor:", {k: round(v, 4) for k, v in sorted(BUDGET_USE.items())}, flush=True)
+
+
+def _check_elements(got, ref, budget, dtype, what, tag, similar=True):
+    """every element: the reference's are_similar criterion and the error budget"""
+    if similar:
+        assert eb.are_similar(got, ref, SIMILAR[dtype]).all(), f"{what} {tag}: an element fails the reference's criterion"
+    ratio = eb.worst_ratio(got, ref, budget, FLOOR[dtype])
+    key = ("f32" if dtype == torch.float32 else "f64", what)
+    BUDGET_USE[key] = max(BUDGET_USE.get(key, 0.0), ratio)
+    assert ratio <= 1.0, f"{what} {tag}: an element is off by {ratio:.3g} times its error budget"
 
 
 def _run(mix_np, xes_np, gout_np, dtype, need_m=True, need_x=True):
@@ -58,6 +81,12 @@ def _check(mix, xes, gout, dtype, tag=""):
     assert rel_l2(gmix[..., 1:1 + D], rgm[..., 1:1 + D], fl) <= tol, f"grad positions {tag}"
     assert rel_l2(gmix[..., 1 + D:], rgm[..., 1 + D:], fl) <= tol, f"grad inverse covariances {tag}"
     assert rel_l2(gxes, rgx, fl) <= tol, f"grad xes {tag}"
+    bud = eb.budgets(mix, xes, gout, npdt, SHIFT_LIMIT[dtype])
+    _check_elements(out, ref, bud["out"], dtype, "out", tag)
+    _check_elements(gmix[..., 0], rgm[..., 0], bud["gw"], dtype, "grad weights", tag)
+    _check_elements(gmix[..., 1:1 + D], rgm[..., 1:1 + D], bud["gb"], dtype, "grad positions", tag)
+    _check_elements(gmix[..., 1 + D:], rgm[..., 1 + D:], bud["gc"], dtype, "grad inverse covariances", tag)
+    _check_elements(gxes, rgx, bud["gx"], dtype, "grad xes", tag)
 
 
 def test_known_answer(golden_dir):
@@ -196,6 +225,78 @@ def test_matrix_core_forward_random_shapes():
         worst = max(worst, err)
         assert err <= TOL[torch.float32], f"case {case}: B{B} L{L} M{M} N{N} D{D} pos {pos_radius} cov {cov_radius}: {err}"
     print("worst relative L2", worst, flush=True)
+
+
+def _adversarial_case(D, M, target_bounds, seed, per_gaussian=52):
+    """Gaussians placed so that the cancellation bound of the shifted form, max_i sum_j |u_ij b_j|, takes the given
+    values (two sides of the kernel's limit), with covariance eigenvalues between 1e-3 and 1 and random rotations; per
+    Gaussian one point exactly at the centre and others 1e-3 ... 4 widths away from it."""
+    g = torch.Generator().manual_seed(seed)
+    lam = torch.exp(torch.rand((1, 1, M, D), generator=g, dtype=torch.float64) * math.log(1e3)) * 1e-3
+    rot = synthetic.random_rotations((1, 1, M), D, g)
+    c = rot @ torch.diag_embed(1.0 / lam) @ rot.transpose(-1, -2)
+    c = 0.5 * (c + c.transpose(-1, -2))
+    u = torch.linalg.cholesky(eb.HALF_LOG2E * c).transpose(-1, -2)
+    direction = torch.randn((1, 1, M, D), generator=g, dtype=torch.float64)
+    bound0 = (u * direction.unsqueeze(-2)).abs().sum(-1).max(-1).values
+    targets = torch.tensor(target_bounds, dtype=torch.float64)[torch.arange(M) % len(target_bounds)].view(1, 1, M)
+    pos = direction * (targets / bound0).unsqueeze(-1)
+    w = torch.randn((1, 1, M), generator=g, dtype=torch.float64)
+    mix = torch.cat([w.unsqueeze(-1), pos, c.reshape(1, 1, M, D * D)], -1).to(torch.float32)
+    # points: offsets z (in widths) mapped through R diag(sqrt(lambda)); the first of every Gaussian is its centre
+    radii = torch.tensor([0.0, 1e-3, 0.1, 0.1, 1.0, 1.0, 2.0, 3.0, 4.0], dtype=torch.float64)
+    z = torch.randn((M, per_gaussian, D), generator=g, dtype=torch.float64)
+    z = z / z.norm(dim=-1, keepdim=True) * radii[torch.arange(per_gaussian) % len(radii)].view(1, -1, 1)
+    offs = torch.einsum('mij,mpj->mpi', rot[0, 0] @ torch.diag_embed(lam[0, 0].sqrt()), z)
+    xes = (mix[0, 0, :, None, 1:1 + D].double() + offs).reshape(1, 1, M * per_gaussian, D).to(torch.float32)
+    xes[0, 0, ::per_gaussian] = mix[0, 0, :, 1:1 + D]                   # bit-identical to the centres
+    return mix, xes
+
+
+@pytest.mark.parametrize("D", [2, 3])
+def test_matrix_core_forward_cancellation_edge(D):
+    """The float32 forward kernel for more than 128 components takes y = u x - u b from bf16 matrix products of
+    three-way split operands; its accuracy rests on how the partial products cancel, which is worst for Gaussians
+    whose bound is just below the kernel's limit of 32 (above it a Gaussian is evaluated with an explicit x - b) and
+    for points at and next to the centres.  Every element is held to the error budget against the float64 oracle
+    (not only the norm), through gm.evaluate_inversed and, in covariance form, gm.evaluate; a single Gaussian with
+    w * norm = 1 among zero-weight ones makes out = exp2(-|y|^2), which exposes the error of y itself."""
+    dtype = torch.float32
+    M = 160
+    for k, targets in enumerate(((30.5, 31.0, 31.9, 31.999), (32.001, 32.1, 33.0, 34.0), (5.0, 31.99, 32.01, 300.0))):
+        mix, xes = _adversarial_case(D, M, targets, 9100 + 10 * D + k)
+        assert xes.shape[2] >= 8192                                      # the shape takes the matrix-core kernel
+        bounds = eb.shifted_bounds(mix.numpy().astype(np.float64))[0, 0]
+        assert np.abs(bounds[:len(targets)] / np.array(targets) - 1).max() < 1e-5
+        m_np, x_np = mix.numpy(), xes.numpy()
+        ones = np.ones((1, 1, xes.shape[2]), dtype=np.float32)
+        out = gm.evaluate_inversed(mix.to(DEV), xes.to(DEV)).cpu().numpy()
+        ref = o.evaluate_inversed(m_np, x_np)
+        bud = eb.budgets(m_np, x_np, ones, np.float32, SHIFT_LIMIT[dtype])
+        assert rel_l2(out, ref, FLOOR[dtype]) <= TOL[dtype]
+        _check_elements(out, ref, bud["out"], dtype, "out (edge)", f"targets {targets}")
+        # the same Gaussians given by their covariances
+        cov = np.linalg.inv(m_np[..., 1 + D:].reshape(1, 1, M, D, D).astype(np.float64))
+        mc = np.concatenate([m_np[..., :1 + D], (0.5 * (cov + np.swapaxes(cov, -1, -2))).reshape(1, 1, M, D * D)], -1)
+        mc = mc.astype(np.float32)
+        out_c = gm.evaluate(torch.tensor(mc, device=DEV), xes.to(DEV)).cpu().numpy()
+        c64 = np.linalg.inv(mc[..., 1 + D:].reshape(1, 1, M, D, D).astype(np.float64))
+        inv = np.concatenate([mc[..., :1 + D].astype(np.float64), c64.reshape(1, 1, M, D * D)], -1)
+        ref_c = o.evaluate_inversed(inv, x_np)
+        bud_c = eb.budgets(inv, x_np, ones, np.float32, SHIFT_LIMIT[dtype])
+        assert rel_l2(out_c, ref_c, FLOOR[dtype]) <= TOL[dtype]
+        _check_elements(out_c, ref_c, bud_c["out"], dtype, "out (edge, covariance form)", f"targets {targets}")
+        # one Gaussian at a time with w * norm = 1, the others with weight 0: out = exp2(-|y|^2)
+        for j in range(len(targets)):
+            single = m_np.copy()
+            single[..., 0] = 0.0
+            c_j = single[0, 0, j, 1 + D:].reshape(D, D).astype(np.float64)
+            single[0, 0, j, 0] = 1.0 / (o.kappa(D) * math.sqrt(np.linalg.det(c_j)))
+            out_1 = gm.evaluate_inversed(torch.tensor(single, device=DEV), xes.to(DEV)).cpu().numpy()
+            ref_1 = o.evaluate_inversed(single, x_np)
+            assert abs(ref_1[0, 0, j * 52] - 1.0) < 1e-6                 # the centre itself
+            bud_1 = eb.budgets(single, x_np, ones, np.float32, SHIFT_LIMIT[dtype])
+            _check_elements(out_1, ref_1, bud_1["out"], dtype, "out (edge, single Gaussian)", f"bound {targets[j]}")
 
 
 @pytest.mark.parametrize("D", [2, 3])
@@ -407,6 +508,19 @@ def _workload_check(name, **kw):
                 gc=rel_l2(gmix[..., 1 + D:], rgm[..., 1 + D:]), gx=rel_l2(gxes, rgx))
     print(name, kw, errs, flush=True)
     assert all(v <= tol for v in errs.values()), errs
+    # Every element of the values by the reference's own criterion.  (Its gradients are not held to it here: the
+    # upstream gradients of these workloads have mixed signs, so single gradient elements cancel to a small fraction
+    # of their terms, and a relative 4e-5 on such an element is beyond any float32 summation, the reference's
+    # included.  They are held to their error budgets instead, which scale with the terms.)
+    assert eb.are_similar(out, ref, SIMILAR[wl.dtype]).all(), f"{name} out: an element fails the reference's criterion"
+    nb = min(2, m64.shape[0])
+    npdt = np.float32 if wl.dtype == torch.float32 else np.float64
+    bud = eb.budgets(m64[:nb], x64[:nb], g64[:nb], npdt, SHIFT_LIMIT[wl.dtype])
+    _check_elements(out[:nb], ref[:nb], bud["out"], wl.dtype, "out", name)
+    _check_elements(gmix[:nb, ..., 0], rgm[:nb, ..., 0], bud["gw"], wl.dtype, "grad weights", name, similar=False)
+    _check_elements(gmix[:nb, ..., 1:1 + D], rgm[:nb, ..., 1:1 + D], bud["gb"], wl.dtype, "grad positions", name, similar=False)
+    _check_elements(gmix[:nb, ..., 1 + D:], rgm[:nb, ..., 1 + D:], bud["gc"], wl.dtype, "grad inverse covariances", name, similar=False)
+    _check_elements(gxes[:nb], rgx[:nb], bud["gx"], wl.dtype, "grad xes", name, similar=False)
 
 
 def test_workload_c1():
@@ -414,11 +528,11 @@ def test_workload_c1():
 
 
 def test_workload_c2():
-    _workload_check("C2", B=20)
+    _workload_check("C2")            # full size: B=100, L=8, M=128, N=784
 
 
 def test_workload_c3():
-    _workload_check("C3", B=4)
+    _workload_check("C3")            # full size: B=21, L=16, M=64, N=4096
 
 
 def test_workload_c4_slice():
