@@ -190,7 +190,8 @@ __device__ __forceinline__ T quad_form(const T* __restrict__ r, const T* __restr
 // caller needs no barrier of its own.
 template <typename T, int D, int GROUP = 1>
 __device__ __forceinline__ void stage_tile(const T* __restrict__ gaussians, int cnt, double amp_scale, T* lds,
-                                           int* counts /* LDS int[10] */, bool covariance_form) {
+                                           int* counts /* LDS int[10] */, bool covariance_form,
+                                           const T* __restrict__ weight_override = nullptr) {
     constexpr int S = Rec<T, D>::kStride;
     constexpr int G = 1 + D + D * D;
     const int tid = threadIdx.x;
@@ -200,6 +201,8 @@ __device__ __forceinline__ void stage_tile(const T* __restrict__ gaussians, int 
     bool centred = false;
     if (active) {
         dv = derive<T, D>(gaussians + size_t(tid) * G, covariance_form);
+        // (the fixed-point fitting evaluates a mixture with other weights than it stores: |x| of the iteration)
+        if (weight_override) dv.w = fabs(double(weight_override[tid]));
         centred = !(dv.bound <= ShiftedBound<T>::v);
     }
     const unsigned long long mc = __ballot(active && centred);

@@ -69,6 +69,11 @@ def lib() -> ctypes.CDLL:
     l.gmc_eval_cov_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, vp]
     l.gmc_eval_componentwise_fwd.argtypes = [vp, vp, vp, shp, ci, vp]
     l.gmc_eval_componentwise_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, ci, vp]
+    l.gmc_relu_fit_goal.argtypes = [vp, vp, vp, vp, shp, vp]
+    l.gmc_relu_fit_step.argtypes = [vp, vp, vp, vp, shp, vp]
+    l.gmc_eval_cov_moments.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_double, shp, ci, vp]
+    l.gmc_batch_norm_sampling_positions.argtypes = [vp, vp, shp, vp]
+    l.gmc_validate_mixture.argtypes = [vp, vp, shp, vp]
     cshp = ctypes.POINTER(ConvShape)
     l.gmc_convolution_fwd.argtypes = [vp, vp, vp, cshp, vp]
     l.gmc_convolution_bwd.argtypes = [vp, vp, vp, vp, vp, cshp, ci, ci, vp]
@@ -242,6 +247,107 @@ def eval_componentwise_bwd(grad_output, mixture, xes, need_mixture: bool, need_x
                                                _p(ws), ws_bytes, ctypes.byref(shape), int(need_mixture), int(need_xes),
                                                int(covariance_form), _stream(dev)))
     return grad_mixture, grad_xes
+
+
+def _mixture_shape(mixture: torch.Tensor, n_points: int) -> Shape:
+    if mixture.dim() != 4:
+        raise RuntimeError("mixture must have 4 dimensions")
+    d = n_dimensions(mixture)
+    if not mixture.is_contiguous():
+        raise RuntimeError("mixture must be contiguous")
+    if mixture.dtype not in (torch.float32, torch.float64):
+        raise RuntimeError("unsupported datatype: float32 and float64 only")
+    if not mixture.is_cuda:
+        raise RuntimeError("gmc_hip evaluates on an AMD GPU only; this build has no CPU implementation")
+    B, L, M, _ = mixture.shape
+    return Shape(B, L, M, n_points, d, B, L, GMC_F32 if mixture.dtype == torch.float32 else GMC_F64)
+
+
+def _like(t: torch.Tensor, ref: torch.Tensor, shape, what: str) -> torch.Tensor:
+    if tuple(t.shape) != tuple(shape) or t.dtype != ref.dtype or t.device != ref.device:
+        raise RuntimeError(f"{what} must have shape {tuple(shape)} and the dtype and device of the mixture")
+    return t.contiguous()
+
+
+def validate_mixture(mixture: torch.Tensor, what: str = "mixture") -> None:
+    """The reference's check_mixture (src/gmc/cpp/extensions/util/mixture.h:85-93) as one small launch and one read of
+    a flag (this synchronises with the device, which is why it is optional everywhere): raises RuntimeError for NaNs,
+    infinities and matrices with a determinant <= 0."""
+    shape = _mixture_shape(mixture, 0)
+    flag = torch.empty((1,), dtype=torch.int32, device=mixture.device)
+    with _on(mixture.device):
+        check(lib().gmc_validate_mixture(_p(mixture), _p(flag), ctypes.byref(shape), _stream(mixture.device)))
+    bits = int(flag.item())
+    if bits & 1:
+        raise RuntimeError(f"{what} contains NaNs or infinities")
+    if bits & 2:
+        raise RuntimeError(f"{what} contains non positive definite covariances")
+
+
+def relu_fit_goal(target_mixture: torch.Tensor, constant: torch.Tensor, fitting_mixture: torch.Tensor) -> torch.Tensor:
+    """relu(evaluate(target, centres of fitting) + constant) - relu(constant), [B, L, n_fitting] (no gradients)"""
+    shape = _mixture_shape(target_mixture, fitting_mixture.shape[2])
+    B, L = shape.B, shape.L
+    if fitting_mixture.dim() != 4 or fitting_mixture.shape[:2] != target_mixture.shape[:2] or \
+            fitting_mixture.shape[3] != target_mixture.shape[3]:
+        raise RuntimeError("target and fitting mixture must agree in batch, layers and dimensions")
+    fitting_mixture = _like(fitting_mixture, target_mixture, fitting_mixture.shape, "fitting mixture")
+    constant = _like(constant.expand(B, L), target_mixture, (B, L), "constant")
+    goal = torch.empty((B, L, shape.N), dtype=target_mixture.dtype, device=target_mixture.device)
+    with _on(target_mixture.device):
+        check(lib().gmc_relu_fit_goal(_p(target_mixture), _p(constant), _p(fitting_mixture), _p(goal), ctypes.byref(shape),
+                                      _stream(target_mixture.device)))
+    return goal
+
+
+def relu_fit_step(fitting_mixture: torch.Tensor, x: torch.Tensor, goal: torch.Tensor) -> torch.Tensor:
+    """one multiplicative update |x| (goal + 0.05) / (evaluate(fitting with weights |x|, own centres) + 0.05)"""
+    shape = _mixture_shape(fitting_mixture, fitting_mixture.shape[2])
+    dims = (shape.B, shape.L, shape.M)
+    x = _like(x, fitting_mixture, dims, "x")
+    goal = _like(goal, fitting_mixture, dims, "goal")
+    out = torch.empty_like(x)
+    with _on(fitting_mixture.device):
+        check(lib().gmc_relu_fit_step(_p(fitting_mixture), _p(x), _p(goal), _p(out), ctypes.byref(shape),
+                                      _stream(fitting_mixture.device)))
+    return out
+
+
+def eval_cov_moments(mixture: torch.Tensor, constant: torch.Tensor, xes: torch.Tensor, per_sample: bool,
+                     running_sd: torch.Tensor = None, running_mean: torch.Tensor = None, alpha: float = 0.0,
+                     want_inverse: bool = False):
+    """torch.std_mean of (evaluate(mixture, xes) + constant) over batch and samples per channel ([L], per_sample False)
+    or over the samples of every (b, l) ([B, L]), without the values going to memory -> (sd, mean), or
+    (sd, mean, 1 / max(sd, 0.001)) with want_inverse.  running_sd / running_mean: updated in place to
+    (1 - alpha) * running + alpha * statistic and returned in place of the statistics."""
+    shape = check_input(mixture, xes)
+    if shape.Bx != shape.B or shape.Lx != shape.L:
+        raise RuntimeError("the sampling positions must have the batch and layer dimensions of the mixture")
+    B, L = shape.B, shape.L
+    constant = _like(constant.expand(B, L), mixture, (B, L), "constant")
+    dims = (B, L) if per_sample else (L,)
+    if running_sd is not None:
+        running_sd = _like(running_sd, mixture, dims, "running_sd")
+        running_mean = _like(running_mean, mixture, dims, "running_mean")
+    sd = torch.empty(dims, dtype=mixture.dtype, device=mixture.device)
+    mean = torch.empty_like(sd)
+    inv = torch.empty_like(sd) if want_inverse else None
+    moments = torch.empty(dims + (2,), dtype=torch.float64, device=mixture.device)
+    with _on(mixture.device):
+        check(lib().gmc_eval_cov_moments(_p(mixture), _p(constant), _p(xes), _p(moments), _p(sd), _p(mean), _p(inv),
+                                         _p(running_sd), _p(running_mean), float(alpha), ctypes.byref(shape),
+                                         int(per_sample), _stream(mixture.device)))
+    return (sd, mean, inv) if want_inverse else (sd, mean)
+
+
+def batch_norm_sampling_positions(mixture: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+    """turns uniform numbers [B, L, N, D] in place into positions inside the box of all centres of their batch entry"""
+    shape = check_input(mixture, uniform)
+    if shape.Bx != shape.B or shape.Lx != shape.L:
+        raise RuntimeError("the uniform numbers must have the batch and layer dimensions of the mixture")
+    with _on(mixture.device):
+        check(lib().gmc_batch_norm_sampling_positions(_p(mixture), _p(uniform), ctypes.byref(shape), _stream(mixture.device)))
+    return uniform
 
 
 # ---------------------------------------------------------------------------------------------------------------

@@ -1,14 +1,16 @@
 """ReLU transfer fitting on top of the evaluation path: the part of the reference's src/gmc/fitting.py that calls
 gm.evaluate with the mixture's own centres as query points (initial_approx_to_relu :279-284,
 fixed_point_iteration_to_relu :287-312, generate_random_sampling :315-322).  The evaluations run through the HIP
-kernels (covariance-form entry points); the element-wise updates around them are torch operations on the
-[batch, layers, components] weight tensors.  The tree-based reduction fitters of that file are not part of this
-package."""
+kernels: without gradients (inference, or inputs that require none) each evaluation and the element-wise update
+that follows it are one launch (gmc_relu_fit_goal / gmc_relu_fit_step); when gradients flow through the fitting, as in
+the reference's training, the evaluations are the differentiable gm.evaluate and the updates torch operations.  The
+tree-based reduction fitters of that file are not part of this package."""
 import typing
 
 import torch
 from torch import Tensor
 
+from . import _native
 from . import mixture as gm
 
 
@@ -25,22 +27,40 @@ def initial_approx_to_relu(mixture: Tensor, constant: Tensor) -> Tensor:
 
 
 def fixed_point_iteration_to_relu(target_mixture: Tensor, target_constant: Tensor, fitting_mixture: Tensor,
-                                  n_iter: int = 1) -> typing.Tuple[Tensor, Tensor]:
+                                  n_iter: int = 1, validate: bool = False) -> typing.Tuple[Tensor, Tensor]:
     """Weights for `fitting_mixture` (positions and covariances stay) such that it matches
     relu(target_mixture + target_constant) - relu(target_constant) at its own centres, by the multiplicative
-    update x <- |x| (b + 0.05) / (fit(centres) + 0.05).  Returns (mixture, relu(target_constant))."""
-    assert gm.is_valid_mixture_and_constant(target_mixture, target_constant)
-    assert gm.is_valid_mixture(fitting_mixture)
-    assert gm.n_batch(target_mixture) == gm.n_batch(fitting_mixture)
-    assert gm.n_layers(target_mixture) == gm.n_layers(fitting_mixture)
-    assert gm.n_dimensions(target_mixture) == gm.n_dimensions(fitting_mixture)
-    assert target_mixture.device == fitting_mixture.device
+    update x <- |x| (b + 0.05) / (fit(centres) + 0.05).  Returns (mixture, relu(target_constant)).
+
+    validate: run the reference's is_valid_mixture checks on both mixtures first (NaN, infinity, determinant <= 0;
+    they read a flag back from the device, i.e. synchronise with it, so they are off unless asked for)."""
+    if validate:
+        _native.validate_mixture(target_mixture.contiguous(), "target mixture")
+        _native.validate_mixture(fitting_mixture.contiguous(), "fitting mixture")
+    if target_constant.dim() != 2 or target_constant.shape[0] not in (1, gm.n_batch(target_mixture)) or \
+            target_constant.shape[1] not in (1, gm.n_layers(target_mixture)):
+        raise RuntimeError("the constant must have shape [batch or 1, layers or 1]")
+    if gm.n_batch(target_mixture) != gm.n_batch(fitting_mixture) or gm.n_layers(target_mixture) != gm.n_layers(fitting_mixture) \
+            or gm.n_dimensions(target_mixture) != gm.n_dimensions(fitting_mixture) \
+            or target_mixture.device != fitting_mixture.device:
+        raise RuntimeError("target and fitting mixture must agree in batch, layers, dimensions and device")
+
+    out_constant = _relu(target_constant)
+    differentiable = torch.is_grad_enabled() and (target_mixture.requires_grad or target_constant.requires_grad
+                                                  or fitting_mixture.requires_grad)
+    if not differentiable:
+        fit = fitting_mixture.contiguous()
+        goal = _native.relu_fit_goal(target_mixture.contiguous(), target_constant, fit)
+        x = gm.weights(fit).abs() + 0.1
+        for _ in range(n_iter):
+            x = _native.relu_fit_step(fit, x, goal)
+        out = fit.clone()
+        out[..., 0] = x
+        return out, out_constant
 
     centres = gm.positions(fitting_mixture).contiguous()
     covariances = gm.covariances(fitting_mixture)
-    out_constant = _relu(target_constant)
     goal = _relu(gm.evaluate(target_mixture, centres) + target_constant.unsqueeze(-1)) - out_constant.unsqueeze(-1)
-
     x = gm.weights(fitting_mixture).abs() + 0.1
     for _ in range(n_iter):
         x = x.abs()

@@ -20,7 +20,7 @@ _PLY_PROPERTIES = ("x", "y", "z", "covxx", "covxy", "covxz", "covyy", "covyz", "
 
 
 def save(mixture: Tensor, file_name: typing.Union[str, os.PathLike], meta_info=None) -> None:
-    assert gm.is_valid_mixture(mixture)
+    gm.check_valid_mixture(mixture)
     torch.save({"type": _TYPE_TAG, "version": 6, "data": mixture.detach().cpu(), "meta_info": meta_info}, file_name)
 
 
@@ -41,7 +41,7 @@ def load(file_name: typing.Union[str, os.PathLike]) -> typing.Tuple[Tensor, typi
         mixture = gm.convert_amplitudes_to_priors(gm.pack_mixture(w, p, c))
     else:
         raise RuntimeError(f"unknown mixture container version {version}")
-    assert gm.is_valid_mixture(mixture)
+    gm.check_valid_mixture(mixture)
     return mixture, container.get("meta_info")
 
 
@@ -53,10 +53,11 @@ def write_gm_to_ply(m_weights: Tensor, m_positions: Tensor, m_covariances: Tenso
     assert m_positions.shape[3] == 3 and tuple(m_covariances.shape[3:]) == (3, 3)
     n = m_weights.shape[2]
     assert m_positions.shape[2] == n and m_covariances.shape[2] == n
-    cov = m_covariances[index, 0].detach().cpu().double()
-    rows = torch.cat([m_positions[index, 0].detach().cpu().double(),
+    # the reference fills a float32 table (torch.zeros(n, 10)) and prints it with numpy's default '%.18e'
+    cov = m_covariances[index, 0].detach().cpu().float()
+    rows = torch.cat([m_positions[index, 0].detach().cpu().float(),
                       torch.stack([cov[:, 0, 0], cov[:, 0, 1], cov[:, 0, 2], cov[:, 1, 1], cov[:, 1, 2], cov[:, 2, 2]], -1),
-                      m_weights[index, 0].detach().cpu().double().unsqueeze(-1)], dim=-1).numpy()
+                      m_weights[index, 0].detach().cpu().float().unsqueeze(-1)], dim=-1).numpy()
     directory = os.path.dirname(filename)
     if directory:
         os.makedirs(directory, exist_ok=True)

@@ -72,6 +72,23 @@ def is_valid_mixture(mixture: Tensor) -> bool:
     return True
 
 
+def check_valid_mixture(mixture: Tensor, what: str = "mixture") -> None:
+    """the same conditions as is_valid_mixture (and the reference's check_mixture,
+    src/gmc/cpp/extensions/util/mixture.h:85-93), raised as RuntimeError; host tensors are checked with torch
+    operations, device tensors with one small launch and one flag read (a synchronisation)"""
+    if mixture.dim() != 4:
+        raise RuntimeError(f"{what} must have 4 dimensions")
+    n_dimensions(mixture)
+    if mixture.is_cuda:
+        from . import _native
+        _native.validate_mixture(mixture.detach().contiguous(), what)
+        return
+    if not bool(torch.isfinite(mixture).all()):
+        raise RuntimeError(f"{what} contains NaNs or infinities")
+    if not bool((covariances(mixture).det() > 0).all()):
+        raise RuntimeError(f"{what} contains non positive definite covariances")
+
+
 def is_valid_mixture_and_constant(mixture: Tensor, constant: Tensor) -> bool:
     """a per-(batch or 1, layer) constant that is added to the mixture's values (src/gmc/mixture.py:188-204)"""
     assert is_valid_mixture(mixture)
@@ -95,9 +112,15 @@ class BvhConfig:
     aabb_mode: str = "reference"
 
 
-def evaluate_inversed(mixture: Tensor, xes: Tensor, bvh: typing.Optional[BvhConfig] = None) -> Tensor:
+def evaluate_inversed(mixture: Tensor, xes: Tensor, bvh: typing.Optional[BvhConfig] = None,
+                      validate: bool = False) -> Tensor:
     """mixture holds inverse covariances; returns [batch, layers, n_points].  With `bvh` the sum runs only over
-    the Gaussians whose cutoff box contains the point (LBVH-culled variant)."""
+    the Gaussians whose cutoff box contains the point (LBVH-culled variant).
+    validate: first check the mixture as the reference's CUDA backward does (NaN, infinity, determinant <= 0 raise
+    RuntimeError; one small launch and a flag read, i.e. a synchronisation with the device: off by default.  Without
+    it a matrix that is not positive definite yields NaN results, not an error)."""
+    if validate:
+        check_valid_mixture(mixture)
     if bvh is None:
         return cppExtensionsEvaluateInversed.apply(mixture, xes)
     from .cpp.extensions.evaluate_inversed import evaluate_inversed_bvh
@@ -108,10 +131,13 @@ def evaluate_inversed_with_amplitude_mixture(mixture: Tensor, xes: Tensor) -> Te
     return evaluate_inversed(convert_amplitudes_to_priors(mixture), xes)
 
 
-def evaluate(mixture: Tensor, xes: Tensor, bvh: typing.Optional[BvhConfig] = None) -> Tensor:
+def evaluate(mixture: Tensor, xes: Tensor, bvh: typing.Optional[BvhConfig] = None, validate: bool = False) -> Tensor:
     """mixture holds covariances; returns [batch, layers, n_points].  Both paths invert the covariances inside
     their kernels (one read of the mixture, no intermediate tensors): the dense path while it stages the
-    Gaussians, the culled path while it builds the boxes and leaf records of the LBVH."""
+    Gaussians, the culled path while it builds the boxes and leaf records of the LBVH.
+    validate: as in evaluate_inversed."""
+    if validate:
+        check_valid_mixture(mixture)
     if bvh is None:
         return cppExtensionsEvaluateInversed.apply_covariance(mixture, xes)
     from .cpp.extensions.evaluate_inversed import evaluate_inversed_bvh

@@ -7,6 +7,7 @@ import typing
 import torch
 from torch import Tensor
 
+from . import _native
 from . import mixture as gm
 from .cpp.extensions.convolution import binding as cpp_convolution
 
@@ -31,43 +32,44 @@ class BatchNorm(torch.nn.Module):
         self.register_buffer("averaged_channel_mean", torch.ones(n_layers))
 
     def sampling_positions(self, x_gm: Tensor) -> Tensor:
+        """uniform positions in the box of all centres of a batch entry (widened in 2-D), one set per channel"""
         n_batch, n_channels, n_dim = gm.n_batch(x_gm), gm.n_layers(x_gm), gm.n_dimensions(x_gm)
         n_samples = 10000 // n_batch if self.batch_norm else 1000
-        centres = gm.positions(x_gm).detach().reshape(n_batch, -1, n_dim)
-        lo = centres.min(dim=1)[0].view(n_batch, 1, 1, n_dim)
-        hi = centres.max(dim=1)[0].view(n_batch, 1, 1, n_dim)
         u = torch.rand(n_batch, n_channels, n_samples, n_dim, device=x_gm.device, dtype=x_gm.dtype)
-        if n_dim == 2:
-            u = u * 1.3 - 0.15
-        return u * (hi - lo) + lo
+        return _native.batch_norm_sampling_positions(x_gm.detach().contiguous(), u)
 
     def forward(self, x: typing.Tuple[Tensor, typing.Optional[Tensor]],
-                sampling_positions: typing.Optional[Tensor] = None) -> typing.Tuple[Tensor, Tensor]:
+                sampling_positions: typing.Optional[Tensor] = None, validate: bool = False) -> typing.Tuple[Tensor, Tensor]:
+        """validate: run the reference's is_valid_mixture check on the input and the finiteness check on the scaling
+        (both read a flag back from the device, i.e. synchronise with it; off unless asked for)"""
         x_gm, x_constant = x
         if x_constant is None:
             x_constant = torch.zeros(gm.n_batch(x_gm), gm.n_layers(x_gm), device=x_gm.device, dtype=x_gm.dtype)
-        assert gm.is_valid_mixture_and_constant(x_gm, x_constant)
+        if validate:
+            _native.validate_mixture(x_gm.detach().contiguous())
         n_channels = gm.n_layers(x_gm)
-        if sampling_positions is None:
-            sampling_positions = self.sampling_positions(x_gm)
 
         with torch.no_grad():
-            values = gm.evaluate(x_gm.detach(), sampling_positions.contiguous()) + x_constant.detach().unsqueeze(-1)
-            if self.batch_norm:
-                sd, mean = torch.std_mean(values, dim=(0, 2))
-                if self.training:
-                    alpha = min(gm.n_batch(x_gm) / 1000, 0.1)
-                    self.averaged_channel_sd = (1.0 - alpha) * self.averaged_channel_sd + alpha * sd
-                    self.averaged_channel_mean = (1.0 - alpha) * self.averaged_channel_mean + alpha * mean
-                sd, mean = self.averaged_channel_sd, self.averaged_channel_mean
+            if self.batch_norm and not self.training:
+                # the running averages alone decide: nothing to sample
+                mean = self.averaged_channel_mean
+                scaling = 1 / torch.clamp(self.averaged_channel_sd, min=0.001)
             else:
-                sd, mean = torch.std_mean(values, dim=2)
-            sd = torch.clamp(sd, min=0.001)
+                if sampling_positions is None:
+                    sampling_positions = self.sampling_positions(x_gm)
+                running = self.batch_norm and self.training
+                alpha = min(gm.n_batch(x_gm) / 1000, 0.1)
+                # evaluation, torch.std_mean, the update of the running averages and 1 / max(sd, 0.001) in three small
+                # launches: the sampled values never go to memory
+                _, mean, scaling = _native.eval_cov_moments(
+                    x_gm.detach().contiguous(), x_constant.detach(), sampling_positions.contiguous(),
+                    per_sample=not self.batch_norm, running_sd=self.averaged_channel_sd if running else None,
+                    running_mean=self.averaged_channel_mean if running else None, alpha=alpha, want_inverse=True)
 
-        scaling = 1 / sd
         if self.learnable_scaling is not None:
             scaling = scaling * self.learnable_scaling
         scaling = scaling.view(-1, n_channels, 1)
-        assert torch.isfinite(scaling).all()
-        scaled = gm.pack_mixture(gm.weights(x_gm) * scaling, gm.positions(x_gm), gm.covariances(x_gm))
+        if validate and not bool(torch.isfinite(scaling).all()):
+            raise RuntimeError("BatchNorm: the scaling is not finite")
+        scaled = torch.cat((gm.weights(x_gm).unsqueeze(-1) * scaling.unsqueeze(-1), x_gm[..., 1:]), dim=-1)
         return scaled, x_constant - mean

@@ -106,6 +106,40 @@ int gmc_eval_componentwise_bwd(const void* grad_out, const void* mixture, const 
                                void* grad_xes, void* workspace, size_t workspace_bytes, const gmc_shape* shape,
                                int need_grad_mixture, int need_grad_xes, int covariance_form, void* stream);
 
+/* ---- evaluations fused with the reductions of their callers ------------------------------------------
+ * The two consumers of gm.evaluate that reduce the values at once.  All mixtures hold COVARIANCES; forward only (no
+ * gradients: callers that differentiate through these functions compose gmc_eval_cov_fwd / _bwd instead).  Points
+ * are per mixture (Bx == B, Lx == L).
+ *
+ * ReLU transfer fitting by fixed-point iteration, src/gmc/fitting.py:287-312:
+ *   gmc_relu_fit_goal   goal[b,l,n] = relu(v + c) - relu(c),  v = target mixture [B][L][M] evaluated at centre n of
+ *                       the fitting mixture [B][L][N], c = constant[b,l]        (fitting.py:301-303)
+ *   gmc_relu_fit_step   x_out[b,l,n] = |x_in| (goal + 0.05) / (v + 0.05),  v = fitting mixture with the weights |x_in|
+ *                       evaluated at its own centre n; shape M == N; x_out must not alias x_in   (fitting.py:307-310)
+ */
+int gmc_relu_fit_goal(const void* target_mixture, const void* constant, const void* fitting_mixture, void* goal,
+                      const gmc_shape* shape, void* stream);
+int gmc_relu_fit_step(const void* fitting_mixture, const void* x_in, const void* goal, void* x_out, const gmc_shape* shape,
+                      void* stream);
+/* Sampled moments of BatchNorm, src/gmc/modules.py:401-415: the mixture is evaluated at xes [B][L][N][D] and
+ * torch.std_mean of (value + constant[b,l]) is returned without the values going to memory: over batch and samples
+ * per channel (per_sample == 0: outputs [L]) or over the samples of every (b,l) (per_sample != 0: [B][L]); sd is the
+ * unbiased one.  `moments`: device scratch of 2 doubles per output element (sum, sum of squares; cleared inside).
+ * running_sd / running_mean (both or neither; may be NULL): the running averages of modules.py:405-410, updated in
+ * place to (1 - alpha) * running + alpha * statistic; sd and mean then return the averages.  inv_sd (may be NULL)
+ * receives 1 / max(sd, 0.001) (modules.py:414-415). */
+int gmc_eval_cov_moments(const void* mixture, const void* constant, const void* xes, double* moments, void* sd, void* mean,
+                         void* inv_sd, void* running_sd, void* running_mean, double alpha, const gmc_shape* shape,
+                         int per_sample, void* stream);
+/* Sampling positions of BatchNorm, src/gmc/modules.py:394-400: uniform numbers in [0, 1) [B][L][N][D] are turned, in
+ * place, into positions inside the box of all centres of their batch entry (2-D: widened by u * 1.3 - 0.15). */
+int gmc_batch_norm_sampling_positions(const void* mixture, void* uniform_in_positions_out, const gmc_shape* shape, void* stream);
+
+/* Optional input check, the reference's check_mixture (src/gmc/cpp/extensions/util/mixture.h:85-93, called by its CUDA
+ * backward): flags[0] (device int32, cleared inside) |= 1 if the mixture holds a NaN or an infinity, |= 2 if a
+ * matrix has a determinant <= 0.  One small launch; the caller decides when to read the flag back. */
+int gmc_validate_mixture(const void* mixture, int32_t* flags, const gmc_shape* shape, void* stream);
+
 /* ---- closed-form convolution of Gaussian mixtures ----------------------------------------------------
  * Replaces convolution::forward_impl / backward_impl (src/gmc/cpp/extensions/convolution/implementation_forward.h:27-103,
  * implementation_backward.h:27-128, bound to Python at convolution/binding.py:21-43), the step that produces the

@@ -29,7 +29,7 @@ import gm_oracle as o
 
 EPS = {np.dtype(np.float32): 2.0 ** -24, np.dtype(np.float64): 2.0 ** -53}
 HALF_LOG2E = 0.72134752044448170368
-C0, CQ, CY, CC, CD = 48.0, 3.0, 6.0, 8.0, 12.0
+C0, CQ, CY, CC, CD = 48.0, 3.0, 6.0, 8.0, 24.0
 ORACLE_SHARE = {np.dtype(np.float32): 1.0, np.dtype(np.float64): 8.0}
 
 

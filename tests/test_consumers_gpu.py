@@ -8,7 +8,7 @@ import torch
 
 import gm_oracle as o
 from conftest import rel_l2
-from gmc import fitting, modules
+from gmc import _native, fitting, inout, modules
 from gmc import mixture as gm
 from gmc.cpp.extensions.convolution import binding as cpp_convolution
 
@@ -171,3 +171,155 @@ def test_layer_pipeline_against_the_oracle_composition():
     assert rel_l2(pre.detach().cpu().numpy(), o.evaluate(onormed, grid.astype(np.float64))) <= 1e-5
     assert torch.isfinite(dt.grad).all() and torch.isfinite(kt.grad).all()
     assert dt.grad.abs().sum() > 0 and kt.grad.abs().sum() > 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("dims", [(2, 3, 70, 33, 2), (1, 2, 300, 200, 3), (2, 1, 40, 700, 2)])
+def test_fused_fitting_kernels_against_their_differentiable_composition(dims, dtype):
+    """(B, L, target components, fitting components, D).  Without gradients the fitting runs on gmc_relu_fit_goal /
+    gmc_relu_fit_step (evaluation and update in one launch each: 128-, 256- and 512-point workgroups, several chunks of
+    centres per mixture, two Gaussian tiles); with inputs that require gradients it composes gm.evaluate with torch
+    operations.  Both must agree with the oracle and with each other, and the gradients of the composition must be
+    finite."""
+    B, L, Mt, Mf, D = dims
+    rng = np.random.default_rng(sum(dims))
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    target = _cov_mixture(rng, B, L, Mt, D, cov=0.1).astype(npdt)
+    const = (rng.normal(size=(B, L)) * 0.3).astype(npdt)
+    fit = _cov_mixture(rng, B, L, Mf, D, cov=0.1).astype(npdt)
+    t, c, f = (torch.tensor(a, device=DEV) for a in (target, const, fit))
+    for n_iter in (1, 2):
+        ref, _ = o.fixed_point_iteration_to_relu(target.astype(np.float64), const.astype(np.float64), fit.astype(np.float64), n_iter)
+        fused, _ = fitting.fixed_point_iteration_to_relu(t, c, f, n_iter)
+        tg = t.clone().requires_grad_(True)
+        composed, _ = fitting.fixed_point_iteration_to_relu(tg, c, f, n_iter)
+        assert composed.requires_grad and not fused.requires_grad
+        assert rel_l2(fused.cpu().numpy(), ref) <= 10 * TOL[dtype]
+        assert rel_l2(composed.detach().cpu().numpy(), ref) <= 10 * TOL[dtype]
+        composed[..., 0].sum().backward()
+        assert torch.isfinite(tg.grad).all() and tg.grad.abs().sum() > 0
+    # a broadcast constant [1, L] and the raw goal
+    goal = _native.relu_fit_goal(t, c[:1], f).cpu().numpy()
+    c0 = const[:1].astype(np.float64)
+    want = np.maximum(o.evaluate(target.astype(np.float64), fit[..., 1:1 + D].astype(np.float64)) + c0[..., None], 0) - np.maximum(c0, 0)[..., None]
+    assert rel_l2(goal, want, 1e-30) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_fused_moments_are_std_mean_of_the_sampled_values(D, dtype):
+    """gmc_eval_cov_moments against torch.std_mean of the values that gm.evaluate returns and against numpy on the
+    oracle's values, per channel over batch and samples and per (b, l), for point counts that take the 128-, 256- and
+    512-point workgroups and several chunks"""
+    rng = np.random.default_rng(90 + D)
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    for B, L, M, N in ((3, 4, 30, 100), (2, 3, 270, 250), (2, 2, 17, 1300), (1, 5, 9, 1)):
+        m = _cov_mixture(rng, B, L, M, D, cov=0.1).astype(npdt)
+        const = rng.normal(size=(B, L)).astype(npdt)
+        xes = rng.uniform(-1.5, 1.5, (B, L, N, D)).astype(npdt)
+        mt, ct, xt = (torch.tensor(a, device=DEV) for a in (m, const, xes))
+        values = o.evaluate(m.astype(np.float64), xes.astype(np.float64)) + const.astype(np.float64)[..., None]
+        for per_sample in (False, True):
+            sd, mean = _native.eval_cov_moments(mt, ct, xt, per_sample)
+            if per_sample:
+                ref_sd, ref_mean = values.std(axis=2, ddof=1) if N > 1 else np.full((B, L), np.nan), values.mean(axis=2)
+            else:
+                flat = np.transpose(values, (1, 0, 2)).reshape(L, -1)
+                ref_sd, ref_mean = flat.std(axis=1, ddof=1) if B * N > 1 else np.full((L,), np.nan), flat.mean(axis=1)
+            assert sd.shape == ref_sd.shape and mean.shape == ref_mean.shape
+            assert rel_l2(mean.cpu().numpy(), ref_mean) <= TOL[dtype]
+            if np.isnan(ref_sd).any():
+                assert torch.isnan(sd).all()                  # one value: torch.std_mean returns nan as well
+            else:
+                assert rel_l2(sd.cpu().numpy(), ref_sd) <= 10 * TOL[dtype]
+
+
+def test_batch_norm_sampling_positions_and_running_averages():
+    """the sampling positions kernel against the torch formula of src/gmc/modules.py:394-400 on the same uniform
+    numbers, and the finishing kernel's running averages / clamped reciprocal against the same arithmetic in numpy"""
+    rng = np.random.default_rng(12)
+    for D in (2, 3):
+        m = torch.tensor(_cov_mixture(rng, 5, 3, 40, D).astype(np.float32), device=DEV)
+        u = torch.rand(5, 3, 77, D, device=DEV)
+        centres = gm.positions(m).reshape(5, -1, D)
+        lo = centres.min(dim=1)[0].view(5, 1, 1, D)
+        hi = centres.max(dim=1)[0].view(5, 1, 1, D)
+        want = (u * 1.3 - 0.15 if D == 2 else u) * (hi - lo) + lo
+        got = _native.batch_norm_sampling_positions(m, u.clone())
+        assert torch.allclose(got, want, rtol=1e-6, atol=1e-6)
+        const = torch.tensor(rng.normal(size=(5, 3)).astype(np.float32), device=DEV)
+        sd0, mean0 = _native.eval_cov_moments(m, const, got, False)
+        run_sd = torch.full((3,), 2.0, device=DEV)
+        run_mean = torch.full((3,), -1.0, device=DEV)
+        sd, mean, inv = _native.eval_cov_moments(m, const, got, False, running_sd=run_sd, running_mean=run_mean, alpha=0.25,
+                                                 want_inverse=True)
+        assert torch.allclose(sd, 0.75 * 2.0 + 0.25 * sd0, rtol=1e-6) and torch.allclose(mean, 0.75 * -1.0 + 0.25 * mean0, rtol=1e-6, atol=1e-7)
+        assert torch.equal(run_sd, sd) and torch.equal(run_mean, mean)
+        assert torch.allclose(inv, 1 / torch.clamp(sd, min=0.001), rtol=1e-6)
+    # a channel without spread: the reciprocal is clamped
+    flat = torch.tensor(_cov_mixture(rng, 2, 2, 3, 2).astype(np.float32), device=DEV)
+    flat[..., 0] = 0.0
+    _, _, inv = _native.eval_cov_moments(flat, torch.zeros(2, 2, device=DEV), torch.rand(2, 2, 50, 2, device=DEV), True, want_inverse=True)
+    assert torch.allclose(inv, torch.full((2, 2), 1000.0, device=DEV), rtol=1e-6)
+
+
+def test_validate_flag_raises_like_the_reference_check():
+    """util/mixture.h:85-93 (called by the reference's CUDA backward), off by default here: with validate=True NaNs,
+    infinities and matrices with a determinant <= 0 raise RuntimeError; without it nothing is checked (and nothing
+    synchronises)"""
+    rng = np.random.default_rng(5)
+    for D in (2, 3):
+        m = torch.tensor(_cov_mixture(rng, 2, 3, 7, D).astype(np.float32), device=DEV)
+        x = torch.zeros(2, 3, 4, D, device=DEV)
+        gm.evaluate(m, x, validate=True)
+        gm.check_valid_mixture(m)
+        bad = m.clone()
+        bad[1, 2, 3, 2] = float("inf")
+        with pytest.raises(RuntimeError, match="NaNs or infinities"):
+            gm.evaluate(bad, x, validate=True)
+        bad = m.clone()
+        bad[0, 0, 0, 1 + D:] = -bad[0, 0, 0, 1 + D:] if D == 3 else torch.tensor([1.0, 2.0, 2.0, 1.0], device=DEV)
+        with pytest.raises(RuntimeError, match="non positive definite"):
+            gm.evaluate_inversed(bad, x, validate=True)
+        with pytest.raises(RuntimeError, match="non positive definite"):
+            fitting.fixed_point_iteration_to_relu(bad, torch.zeros(2, 3, device=DEV), m, validate=True)
+        with pytest.raises(RuntimeError, match="non positive definite"):
+            modules.BatchNorm(3).to(DEV)((bad, None), validate=True)
+        gm.evaluate(bad, x)                                       # not checked: NaN values, no error
+        fitting.fixed_point_iteration_to_relu(m, torch.zeros(2, 3, device=DEV), m)
+
+
+def test_files_written_like_the_reference_replay_through_the_device_path(tmp_path, golden_dir):
+    """Containers of versions 3 to 6 as the reference's save/older writers lay them out (src/gmc/inout.py:12-49) and
+    PLY files (:52-141), the committed golden one included, are loaded with gmc.inout and evaluated on the device;
+    the values must be those of the oracle on the mixture that was written."""
+    rng = np.random.default_rng(66)
+    B, M, D = 3, 20, 3
+    m64 = _cov_mixture(rng, B, 1, M, D, cov=0.2)
+    m64[..., 0] = np.abs(m64[..., 0]) + 0.1
+    m = torch.tensor(m64, dtype=torch.float32)
+    xes = rng.uniform(-2, 2, (1, 1, 300, D)).astype(np.float32)
+    ref = o.evaluate(m.numpy().astype(np.float64), xes.astype(np.float64))
+    amp = gm.convert_priors_to_amplitudes(m)
+    w, p, c = gm.weights(amp), gm.positions(amp), gm.covariances(amp)
+    torch.save({"type": "gm.Mixture", "version": 6, "data": m, "meta_info": {"k": 1}}, tmp_path / "v6.torch")
+    torch.save({"type": "gm.Mixture", "version": 5, "data": amp, "meta_info": None}, tmp_path / "v5.torch")
+    torch.save({"type": "gm.Mixture", "version": 4, "weights": w, "positions": p, "covariances": c, "meta_info": None}, tmp_path / "v4.torch")
+    torch.save({"type": "gm.Mixture", "version": 3, "weights": w[:, 0], "positions": p[:, 0], "covariances": c[:, 0],
+                "meta_info": None}, tmp_path / "v3.torch")
+    xt = torch.tensor(xes, device=DEV)
+    for version in (6, 5, 4, 3):
+        loaded, _ = inout.load(tmp_path / f"v{version}.torch")
+        out = gm.evaluate(loaded.to(DEV), xt, validate=True)
+        assert rel_l2(out.cpu().numpy(), ref) <= 1e-5, f"container version {version}"
+    # PLY: one file per mixture, weights as they are (amplitudes when read back with ismodel=False)
+    inout.write_gm_to_ply2(m, str(tmp_path / "ply" / "gm"))
+    for b in range(B):
+        loaded = inout.read_gm_from_ply(str(tmp_path / "ply" / f"gm_b{b}_l0.ply"))
+        out = gm.evaluate(loaded.to(DEV), xt)
+        assert rel_l2(out.cpu().numpy(), ref[b:b + 1]) <= 1e-5
+    golden = inout.read_gm_from_ply(f"{golden_dir}/mixture_b0_l0.ply")
+    out = gm.evaluate(golden.to(DEV), xt, bvh=gm.BvhConfig(aabb_mode="tight"))
+    dense = o.evaluate(golden.numpy().astype(np.float64), xes.astype(np.float64))
+    assert rel_l2(gm.evaluate(golden.to(DEV), xt).cpu().numpy(), dense) <= 1e-5
+    assert rel_l2(out.cpu().numpy(), dense) <= 5e-3            # culled at the 0.001 threshold

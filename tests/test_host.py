@@ -142,3 +142,38 @@ def test_on_disk_formats_roundtrip(tmp_path):
     prior = inout.read_gm_from_ply(str(tmp_path / "ply" / "gm_b1_l0.ply"), ismodel=True)
     wn = w[1:2] / w[1:2].sum()
     assert torch.allclose(gm.weights(prior), gm.convert_priors_to_amplitudes2(wn, c[1:2]), atol=1e-6)
+
+
+def test_ply_text_matches_the_reference_writer_byte_for_byte(tmp_path, golden_dir):
+    """tests/golden/mixture_b0_l0.ply holds the text the reference's write_gm_to_ply (src/gmc/inout.py:52-98) produces for
+    the mixture of mixture_ply.json (written by tests/golden/make_ply_golden.py without this package): the writer here
+    must reproduce it byte for byte, also from a float64 mixture (the reference prints a float32 table), and the
+    reader must return the values."""
+    import json
+    from gmc import inout
+    data = json.load(open(os.path.join(golden_dir, "mixture_ply.json")))
+    w = torch.tensor(data["weights"], dtype=torch.float32).view(1, 1, -1)
+    p = torch.tensor(data["positions"], dtype=torch.float32).view(1, 1, -1, 3)
+    c = torch.tensor(data["covariances"], dtype=torch.float32).view(1, 1, -1, 3, 3)
+    golden = open(os.path.join(golden_dir, "mixture_b0_l0.ply"), "rb").read()
+    for dtype in (torch.float32, torch.float64):
+        m = gm.pack_mixture(w.to(dtype), p.to(dtype), c.to(dtype))
+        inout.write_gm_to_ply2(m, str(tmp_path / str(dtype) / "mixture"))
+        assert open(tmp_path / str(dtype) / "mixture_b0_l0.ply", "rb").read() == golden
+    back = inout.read_gm_from_ply(os.path.join(golden_dir, "mixture_b0_l0.ply"))
+    assert torch.equal(back, gm.pack_mixture(w, p, c))
+
+
+def test_check_valid_mixture_on_host_tensors():
+    g = torch.Generator().manual_seed(4)
+    a = torch.rand(2, 2, 3, 2, 2, generator=g)
+    m = gm.pack_mixture(torch.rand(2, 2, 3, generator=g), torch.rand(2, 2, 3, 2, generator=g), a @ a.transpose(-1, -2) + torch.eye(2))
+    gm.check_valid_mixture(m)
+    bad = m.clone()
+    bad[0, 1, 2, 1] = float("nan")
+    with pytest.raises(RuntimeError, match="NaNs or infinities"):
+        gm.check_valid_mixture(bad)
+    bad = m.clone()
+    bad[1, 0, 0, 3:] = torch.tensor([1.0, 2.0, 2.0, 1.0])
+    with pytest.raises(RuntimeError, match="non positive definite"):
+        gm.check_valid_mixture(bad)
