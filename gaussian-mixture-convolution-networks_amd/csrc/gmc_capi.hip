@@ -13,6 +13,7 @@ int dense_backward_static(const void* grad_out, const void* mixture, const void*
                           const gmc_shape& s, bool need_gm, bool need_gx, bool covariance_form, hipStream_t stream);
 
 const char* dense_forward_kernel_name(const gmc_shape& s);
+void set_tuning(int fwd_points_per_lane, int bwd_points_per_lane);
 
 int check_shape(const gmc_shape* s) {
     if (!s) return GMC_E_NULL;
@@ -68,6 +69,8 @@ int gmc_eval_fwd(const void* mixture, const void* xes, void* out, const gmc_shap
 int gmc_eval_cov_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream) {
     return eval_fwd_impl(mixture, xes, out, shape, true, stream);
 }
+
+void gmc_set_tuning(int fwd_points_per_lane, int bwd_points_per_lane) { gmc::set_tuning(fwd_points_per_lane, bwd_points_per_lane); }
 
 const char* gmc_eval_fwd_kernel_name(const gmc_shape* shape) {
     if (gmc::check_shape(shape) != GMC_OK) return "";

@@ -548,6 +548,13 @@ static int pick_points_per_lane(int N, int BL) {
     return best;
 }
 
+// Tuning overrides (gmc_set_tuning): 0 = automatic choice
+static std::atomic<int> forced_fwd_points{0}, forced_bwd_points{0};
+void set_tuning(int fwd_points_per_lane, int bwd_points_per_lane) {
+    forced_fwd_points.store(fwd_points_per_lane);
+    forced_bwd_points.store(bwd_points_per_lane);
+}
+
 // Which all-vector forward kernel a shape takes: `rc` > 0: the 4 x 16 layout with that many points per lane,
 // otherwise the one-Gaussian-per-step layout with `P` points per lane.
 struct FwdPlan { int P, chunks, rc; };
@@ -568,6 +575,8 @@ static FwdPlan plan_fwd(const gmc_shape& s, bool is_double) {
         if (q_chunks * 64 * q < covered_best) { covered_best = q_chunks * 64 * q; q_best = q; }
     }
     plan.rc = q_best;
+    const int forced = forced_fwd_points.load();
+    if (forced >= 2 && forced <= q_max) plan.rc = forced;
     return plan;
 }
 
@@ -628,6 +637,8 @@ static int bwd_points_per_lane(const gmc_shape& s) {
     const double pair_cost = D == 2 ? 18.0 : 30.0, reduce_cost = 5.0 * Sums<D>::k;
     int P = 2;
     double best = 1e300;
+    const int forced = forced_bwd_points.load();
+    if (forced >= 2 && forced <= p_max) return forced;
     for (int cand = p_max; cand >= 2; --cand) {
         const int span = 64 * cand;
         const size_t chunks = (size_t(s.N) + span - 1) / span;

@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
     l.gmc_error_string.argtypes = [ci]
     l.gmc_abi_version.restype = ci
     l.gmc_eval_fwd.argtypes = [vp, vp, vp, shp, vp]
+    l.gmc_set_tuning.restype = None
+    l.gmc_set_tuning.argtypes = [ci, ci]
     l.gmc_eval_fwd_kernel_name.restype = ctypes.c_char_p
     l.gmc_eval_fwd_kernel_name.argtypes = [shp]
     l.gmc_eval_bwd_workspace_bytes.restype = sz

@@ -53,6 +53,11 @@ int gmc_abi_version(void);
  */
 int gmc_eval_fwd(const void* mixture, const void* xes, void* out, const gmc_shape* shape, void* stream);
 
+/* Tuning and test knob (no counterpart in the reference; process-wide): forces the points per lane of the all-vector
+ * "4 x 16" kernels, forward and backward (2 ... 16, float64: 2 ... 8; a workgroup then covers 64 times as many points);
+ * 0 returns to the automatic choice.  Results do not depend on it beyond the order of additions. */
+void gmc_set_tuning(int fwd_points_per_lane, int bwd_points_per_lane);
+
 /* Name of the forward pair kernel a call of this shape launches (for benchmark reports; no counterpart in the
  * reference): "eval_fwd_mfma_kernel" (float32, more than 128 components, enough work for 512-component tiles),
  * "eval_fwd_rc_kernel" or "eval_fwd_kernel" (all vector ALU, two layouts); "" for an invalid shape. */
