@@ -53,6 +53,8 @@ struct BvhLayout {
     size_t cand_stamp;          // uint64 [BL][ceil(N/64)] content stamp of the 64 points a group's list was gathered for
     size_t cand_pieces;         // int2 [BL][ceil(N/64)]   slots of the piece table that hold this group's pieces (first, count)
     size_t cand_ctl;            // int [4]                 pieces published, pool ints handed out, error flags (kErr*), -
+    size_t sums;                // T [BL][M][1+D+D(D+1)/2]  per-Gaussian sums of the backward pass: all zero between calls (the
+                                //                          build clears them, the backward epilogue clears what it has read)
     size_t pieces;              // int4 [pieces_max]       (point group, offset into cand_list, leaves, -)
     size_t piece_gx;            // T [pieces_max][D][64]   dL/dx of the pieces, added to grad_xes by the epilogue
     bool cand_cache;
@@ -164,6 +166,7 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
         l.cand_stamp = take(l.cand_cache ? point_groups * 8 : 0);
         l.cand_pieces = take(l.cand_cache ? point_groups * 8 : 0);
         l.cand_ctl = take(16);
+        l.sums = take(BL * M * (D == 2 ? 6 : 10) * e);
         l.pieces = take(size_t(l.pieces_max) * 16);
         l.piece_gx = take(size_t(l.pieces_max) * D * kWave * e);
     }
@@ -661,9 +664,10 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
                                                            T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
                                                            int2* __restrict__ children, int* __restrict__ parent,
                                                            int2* __restrict__ node_range, int M, size_t total,
-                                                           bool covariance_form) {
+                                                           bool covariance_form, T* __restrict__ sums) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
+    constexpr int NS = 1 + D + D * (D + 1) / 2;
     // The records of the leaves and the internal nodes of the tree do not depend on each other, and both are
     // short chains of dependent memory reads: the first half of the grid writes the records, the second half
     // builds the nodes, side by side on different compute units.
@@ -678,6 +682,8 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         if (leaf < M - 1) build_internal_node(keys, children, parent, node_range, M, bl, leaf);
         return;
     }
+    // the per-Gaussian sums of the backward pass start from zero (and return to zero after every backward pass)
+    for (int k = 0; k < NS; ++k) sums[i * NS + k] = T(0);
     int comp = int(order[i]);
     comp = (comp >= 0 && comp < M) ? comp : 0;      // a permutation by construction; never index out of bounds
     const size_t gi = bl * M + comp;
@@ -1412,7 +1418,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
 // MatrixInverse.backward does (src/gmc/cpp/extensions/math/matrix_inverse.py:30-33: -S^-1 g S^-1 without transposes,
 // which is the derivative for symmetric matrices only): dS = -(C dC C)^T.
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __restrict__ mixture, const T* __restrict__ sums,
+__global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __restrict__ mixture, T* __restrict__ sums,
                                                                  T* __restrict__ grad_mixture, size_t n,
                                                                  bool covariance_form, CandidateCache cache,
                                                                  const T* __restrict__ piece_gx,
@@ -1447,7 +1453,8 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
     const size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x;
     if (i >= n) return;
     const T* g = mixture + i * G;
-    const T* rs = sums + i * NR;
+    T rs[NR];
+    for (int k = 0; k < NR; ++k) { rs[k] = sums[i * NR + k]; sums[i * NR + k] = T(0); }     // ready for the next backward pass
     T* o = grad_mixture + i * G;
     const double w = double(g[0]);
     double c[D][D];
@@ -1618,7 +1625,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         bvh_leaves_kernel<T, D><<<dim3(2 * grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi,
                                                                                   double(cfg.aabb_threshold), cfg.aabb_mode, g_order, g_keys,
                                                                            node_box, leaf_rec, enc_box, children, parent, node_range, M, n,
-                                                                           cfg.covariance_form != 0);
+                                                                           cfg.covariance_form != 0, (T*)(bvh + lay.sums));
         if (M > 1) {
             const size_t ni = BL * (M - 1);
             bvh_merge_kernel<T, D><<<dim3(unsigned((n + kMergeBlock - 1) / kMergeBlock)), dim3(kMergeBlock), 0, st>>>(
@@ -1665,7 +1672,6 @@ template <typename T, int D>
 static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bvh, T* grad_mixture, T* grad_xes,
                      T* sums, const gmc_shape& s, bool gm, bool gx, bool covariance_form, hipStream_t st) {
     constexpr int G = 1 + D + D * D;
-    constexpr int NR = BvhSums<D>::k;
     const BvhLayout lay = bvh_layout(s);
     const size_t BL = size_t(s.B) * s.L;
     const size_t n_g = BL * s.M, n_x = size_t(s.Bx) * s.Lx * s.N * D;
@@ -1679,7 +1685,7 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bv
         if (gx) zero(grad_xes, n_x);
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    if (gm) zero(sums, n_g * NR);
+    sums = (T*)(bvh + lay.sums);                   // inside the object and all zero here; the caller's workspace is not used
     if (gx && xes_shared) zero(grad_xes, n_x);
     const int groups = traversal_groups(BL, s.N);
     const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
@@ -1838,11 +1844,7 @@ static int eval_bvh_bwd_impl(const void* grad_out, const void* mixture, const vo
     if (gm && n_g > 0 && !grad_mixture) return GMC_E_NULL;
     if (gx && n_x > 0 && !grad_xes) return GMC_E_NULL;
     if (n_g > 0 && n_x > 0 && (!grad_out || !mixture || !xes || !bvh)) return GMC_E_NULL;
-    if (gm && n_g > 0 && n_x > 0) {
-        const size_t need = n_g * (shape->D == 2 ? 6 : 10) * (shape->dtype == GMC_F32 ? 4 : 8);
-        if (workspace_bytes < need) return GMC_E_WORKSPACE;
-        if (!workspace) return GMC_E_NULL;
-    }
+    (void)workspace_bytes;    // the per-Gaussian sums live inside the BVH object; a workspace is accepted and not used
 #define ARGS(T) (const T*)grad_out, (const T*)mixture, (const T*)xes, (char*)bvh, (T*)grad_mixture, (T*)grad_xes, (T*)workspace, *shape, gm, gx, covariance_form, (hipStream_t)stream
     if (shape->dtype == GMC_F32) return shape->D == 2 ? gmc::bvh_bwd_t<float, 2>(ARGS(float)) : gmc::bvh_bwd_t<float, 3>(ARGS(float));
     return shape->D == 2 ? gmc::bvh_bwd_t<double, 2>(ARGS(double)) : gmc::bvh_bwd_t<double, 3>(ARGS(double));

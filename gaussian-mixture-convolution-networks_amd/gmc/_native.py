@@ -491,10 +491,8 @@ def eval_bvh_bwd(grad_output, mixture, xes, bvh: Bvh, need_mixture: bool, need_x
     if not (need_mixture or need_xes):
         return grad_mixture, grad_xes
     with _on(dev):
-        ws_bytes = lib().gmc_eval_bwd_workspace_bytes(ctypes.byref(shape)) if need_mixture else 0
-        ws = torch.empty((max(ws_bytes, 8) // 8,), dtype=torch.float64, device=dev)
         fn = lib().gmc_eval_bvh_cov_bwd if bvh.covariance_form else lib().gmc_eval_bvh_bwd
-        check(fn(_p(grad_output), _p(mixture), _p(xes), _p(bvh.blob), _p(grad_mixture), _p(grad_xes), _p(ws), ws_bytes,
+        check(fn(_p(grad_output), _p(mixture), _p(xes), _p(bvh.blob), _p(grad_mixture), _p(grad_xes), None, 0,
                  ctypes.byref(shape), int(need_mixture), int(need_xes), _stream(dev)))
     return grad_mixture, grad_xes
 

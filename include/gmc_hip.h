@@ -216,6 +216,8 @@ int gmc_bvh_export_leaf_order(const void* bvh, uint32_t* keys, int32_t* componen
  * built for: the layout of the object follows from it and is not stored inside. */
 int gmc_eval_bvh_fwd(const void* mixture, const void* xes, void* bvh, void* out, const gmc_shape* shape,
                      void* stream);
+/* (`workspace` / `workspace_bytes` of the backward calls are accepted and not used: the per-Gaussian sums live inside
+ * the BVH object, cleared by the build and again by every backward pass; NULL and 0 are fine.) */
 int gmc_eval_bvh_bwd(const void* grad_out, const void* mixture, const void* xes, void* bvh,
                      void* grad_mixture, void* grad_xes, void* workspace, size_t workspace_bytes,
                      const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, void* stream);
