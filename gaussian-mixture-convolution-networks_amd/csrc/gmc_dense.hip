@@ -53,15 +53,20 @@ __device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, int begin, 
 template <typename T, int D, int P>
 __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ mixture, const T* __restrict__ xes,
                                                           T* __restrict__ out, int L, int M, int N, int Bx, int Lx,
-                                                          int chunks, int n_mixtures, bool covariance_form) {
+                                                          int chunks, int n_mixtures, bool covariance_form,
+                                                          TileSlices ts) {
     constexpr int G = 1 + D + D * D;
     constexpr int S = Rec<T, D>::kStride;
     __shared__ __attribute__((aligned(16))) T lds[kTile * S];
     __shared__ int counts[10];
 
     int bl, chunk;
-    map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
+    map_workgroup(blockIdx.x, chunks * ts.slices, n_mixtures, bl, chunk);
     if (bl >= n_mixtures) return;
+    const int slice = chunk / chunks;
+    chunk -= slice * chunks;
+    const int g_begin = slice * ts.tiles_per_slice * kTile;
+    const int g_end = (g_begin + ts.tiles_per_slice * kTile) < M ? (g_begin + ts.tiles_per_slice * kTile) : M;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const T* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
@@ -79,8 +84,8 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
         acc[p] = T(0);
     }
 
-    for (int g0 = 0; g0 < M; g0 += kTile) {
-        const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
+    for (int g0 = g_begin; g0 < g_end; g0 += kTile) {
+        const int cnt = (g_end - g0) < kTile ? (g_end - g0) : kTile;
         stage_tile<T, D>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts, covariance_form);
         const int n_shifted = counts[8];
         fwd_pairs<T, D, P, false>(lds, 0, n_shifted, x, acc);
@@ -89,7 +94,9 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
 #pragma unroll
     for (int p = 0; p < P; ++p) {
         const int n = n0 + p * kBlock;
-        if (n < N) out[size_t(bl) * N + n] = acc[p];
+        if (n < N) {
+            if (ts.slices > 1) atomic_add(&out[size_t(bl) * N + n], acc[p]); else out[size_t(bl) * N + n] = acc[p];
+        }
     }
 }
 
@@ -118,15 +125,20 @@ __device__ __forceinline__ void fwd_rc_pairs(const T* __restrict__ lds, int begi
 template <typename T, int D, int P>
 __global__ __launch_bounds__(kBlock) void eval_fwd_rc_kernel(const T* __restrict__ mixture, const T* __restrict__ xes,
                                                              T* __restrict__ out, int L, int M, int N, int Bx, int Lx,
-                                                             int chunks, int n_mixtures, bool covariance_form) {
+                                                             int chunks, int n_mixtures, bool covariance_form,
+                                                             TileSlices ts) {
     constexpr int G = 1 + D + D * D;
     constexpr int S = Rec<T, D>::kStride;
     __shared__ __attribute__((aligned(16))) T lds[(kTile + 6) * S];
     __shared__ int counts[10];
 
     int bl, chunk;
-    map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
+    map_workgroup(blockIdx.x, chunks * ts.slices, n_mixtures, bl, chunk);
     if (bl >= n_mixtures) return;
+    const int slice = chunk / chunks;
+    chunk -= slice * chunks;
+    const int g_begin = slice * ts.tiles_per_slice * kTile;
+    const int g_end = (g_begin + ts.tiles_per_slice * kTile) < M ? (g_begin + ts.tiles_per_slice * kTile) : M;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const T* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
@@ -145,8 +157,8 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_rc_kernel(const T* __restrict
         for (int d = 0; d < D; ++d) x[p][d] = x_bl[size_t(n) * D + d];
         acc[p] = T(0);
     }
-    for (int g0 = 0; g0 < M; g0 += kTile) {
-        const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
+    for (int g0 = g_begin; g0 < g_end; g0 += kTile) {
+        const int cnt = (g_end - g0) < kTile ? (g_end - g0) : kTile;
         stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts, covariance_form);
         const int centred_start = counts[8], padded_total = counts[9];
         fwd_rc_pairs<T, D, P, false>(lds, 0, centred_start, row, x, acc);
@@ -158,7 +170,9 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_rc_kernel(const T* __restrict
         v += __shfl_xor(v, 16, 64);
         v += __shfl_xor(v, 32, 64);
         const int n = n0 + p * 16;
-        if (row == 0 && n < N) out[size_t(bl) * N + n] = v;
+        if (row == 0 && n < N) {
+            if (ts.slices > 1) atomic_add(&out[size_t(bl) * N + n], v); else out[size_t(bl) * N + n] = v;
+        }
     }
 }
 
@@ -287,7 +301,7 @@ template <typename T, int D, int P, bool NEED_GM, bool NEED_GX, bool SOLE>
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 3 : 1)))
 void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mixture, const T* __restrict__ xes,
                         T* __restrict__ sums, T* __restrict__ grad_xes, T* __restrict__ grad_mixture, int L, int M, int N,
-                        int Bx, int Lx, int chunks, int xes_shared, int n_mixtures, bool covariance_form) {
+                        int Bx, int Lx, int chunks, int xes_shared, int n_mixtures, bool covariance_form, TileSlices ts) {
     constexpr int G = 1 + D + D * D;
     constexpr int S = Rec<T, D>::kStride;
     constexpr int NR = Sums<D>::k;
@@ -300,8 +314,13 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
     static_assert(sizeof(T) == 8 || sizeof(lds) + sizeof(block_sums) + 64 <= 53760, "LDS of the backward pair kernel");
 
     int bl, chunk;
-    map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
+    map_workgroup(blockIdx.x, chunks * ts.slices, n_mixtures, bl, chunk);
     if (bl >= n_mixtures) return;
+    // (with several slices the host passes xes_shared != 0: dL/dx of a point then comes from several workgroups)
+    const int slice = chunk / chunks;
+    chunk -= slice * chunks;
+    const int g_begin = slice * ts.tiles_per_slice * kTile;
+    const int g_end = (g_begin + ts.tiles_per_slice * kTile) < M ? (g_begin + ts.tiles_per_slice * kTile) : M;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const T* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
@@ -331,8 +350,8 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
             for (int i = threadIdx.x; i < kTile * NR; i += kBlock) block_sums[i] = T(0);
     }
 
-    for (int g0 = 0; g0 < M; g0 += kTile) {
-        const int cnt = (M - g0) < kTile ? (M - g0) : kTile;
+    for (int g0 = g_begin; g0 < g_end; g0 += kTile) {
+        const int cnt = (g_end - g0) < kTile ? (g_end - g0) : kTile;
         stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0 / kHalfLog2e, lds, counts, covariance_form);
         const int centred_start = counts[8], padded_total = counts[9];
         T* wave_sums = block_sums + (NEED_GM && SumCopies<T>::k > 1 ? wave * kTile * NR : 0);
@@ -595,8 +614,10 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
         const int q_best = plan.rc;
         if (q_best > 0) {
             const int q_chunks = (s.N + 64 * q_best - 1) / (64 * q_best);
-            const dim3 q_grid(unsigned(grid_mixtures(BL) * q_chunks));
-#define GMC_FWD_RC(QQ) case QQ: eval_fwd_rc_kernel<T, D, QQ><<<q_grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, q_chunks, int(BL), cov); break
+            const TileSlices ts = plan_tile_slices(grid_mixtures(BL) * q_chunks, s.M, kTile);
+            if (ts.slices > 1) zero_async(out, BL * s.N, stream);
+            const dim3 q_grid(unsigned(grid_mixtures(BL) * q_chunks * ts.slices));
+#define GMC_FWD_RC(QQ) case QQ: eval_fwd_rc_kernel<T, D, QQ><<<q_grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, q_chunks, int(BL), cov, ts); break
             switch (q_best) {
                 GMC_FWD_RC(2); GMC_FWD_RC(3); GMC_FWD_RC(4); GMC_FWD_RC(5); GMC_FWD_RC(6); GMC_FWD_RC(7); GMC_FWD_RC(8);
                 default:
@@ -613,8 +634,10 @@ static int launch_fwd(const T* mixture, const T* xes, T* out, const gmc_shape& s
             return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
         }
     }
-    const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
-#define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks, int(BL), cov)
+    const TileSlices ts = plan_tile_slices(grid_mixtures(BL) * chunks, s.M, kTile);
+    if (ts.slices > 1) zero_async(out, BL * s.N, stream);
+    const dim3 grid(unsigned(grid_mixtures(BL) * chunks * ts.slices));
+#define GMC_FWD(PP) eval_fwd_kernel<T, D, PP><<<grid, dim3(kBlock), 0, stream>>>(mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, chunks, int(BL), cov, ts)
     switch (P) {
         case 8: GMC_FWD(8); break;
         case 4: GMC_FWD(4); break;
@@ -651,13 +674,13 @@ static int bwd_points_per_lane(const gmc_shape& s) {
 
 template <typename T, int D, bool GM, bool GX, bool SOLE>
 static void launch_bwd_main(const T* grad_out, const T* mixture, const T* xes, T* sums, T* grad_xes, T* grad_mixture,
-                            const gmc_shape& s, int P, int xes_shared, bool cov, hipStream_t stream) {
+                            const gmc_shape& s, int P, int xes_shared, bool cov, TileSlices ts, hipStream_t stream) {
     const size_t BL = size_t(s.B) * s.L;
     constexpr int p_max = sizeof(T) == 8 ? 8 : 16;
     const int span = 64 * P;
     const int chunks = (s.N + span - 1) / span;
-    const dim3 grid(unsigned(grid_mixtures(BL) * chunks));
-#define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX, SOLE><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL), cov)
+    const dim3 grid(unsigned(grid_mixtures(BL) * chunks * ts.slices));
+#define GMC_BWD(PP) eval_bwd_rc_kernel<T, D, PP, GM, GX, SOLE><<<grid, dim3(kBlock), 0, stream>>>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s.L, s.M, s.N, s.Bx, s.Lx, chunks, xes_shared, int(BL), cov, ts)
     if constexpr (p_max > 8) {
         switch (P) {
             case 16: GMC_BWD(16); return;
@@ -698,15 +721,19 @@ static int launch_bwd(const T* grad_out, const T* mixture, const T* xes, T* grad
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
     const int P = bwd_points_per_lane<T, D>(s);
+    const size_t chunks = (size_t(s.N) + 64 * P - 1) / (64 * P);
+    const TileSlices ts = plan_tile_slices(grid_mixtures(BL) * chunks, s.M, kTile);
+    // several slices of Gaussian tiles per point chunk: dL/dx of a point is then added up over workgroups
+    const int gx_shared = (xes_shared || ts.slices > 1) ? 1 : 0;
     // one chunk per mixture: the pair kernel's workgroups finish the gradient of their mixture themselves
-    const bool sole = need_gm && s.N <= 64 * P;
+    const bool sole = need_gm && s.N <= 64 * P && ts.slices == 1;
     if (need_gm && !sole) zero_async(sums, n_gauss * Sums<D>::k, stream);
-    if (need_gx && xes_shared) zero_async(grad_xes, n_x, stream);
-    if (sole && need_gx) launch_bwd_main<T, D, true, true, true>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
-    else if (sole) launch_bwd_main<T, D, true, false, true>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
-    else if (need_gm && need_gx) launch_bwd_main<T, D, true, true, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
-    else if (need_gm) launch_bwd_main<T, D, true, false, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
-    else if (need_gx) launch_bwd_main<T, D, false, true, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, xes_shared, cov, stream);
+    if (need_gx && gx_shared) zero_async(grad_xes, n_x, stream);
+    if (sole && need_gx) launch_bwd_main<T, D, true, true, true>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, gx_shared, cov, ts, stream);
+    else if (sole) launch_bwd_main<T, D, true, false, true>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, gx_shared, cov, ts, stream);
+    else if (need_gm && need_gx) launch_bwd_main<T, D, true, true, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, gx_shared, cov, ts, stream);
+    else if (need_gm) launch_bwd_main<T, D, true, false, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, gx_shared, cov, ts, stream);
+    else if (need_gx) launch_bwd_main<T, D, false, true, false>(grad_out, mixture, xes, sums, grad_xes, grad_mixture, s, P, gx_shared, cov, ts, stream);
     if (need_gm && !sole) {
         const size_t blocks = (n_gauss + kBlock - 1) / kBlock;
         eval_bwd_epilogue_kernel<T, D><<<dim3(unsigned(blocks)), dim3(kBlock), 0, stream>>>(mixture, sums, grad_mixture, n_gauss, cov);

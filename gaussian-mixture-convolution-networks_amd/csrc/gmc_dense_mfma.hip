@@ -236,7 +236,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4))) vo
                                                                 const float* __restrict__ xes, float* __restrict__ out,
                                                                 int L, int M, int N, int Bx, int Lx, int chunks,
                                                                 int blocks_per_chunk, int n_mixtures,
-                                                                bool covariance_form) {
+                                                                bool covariance_form, TileSlices ts) {
     constexpr int G = 1 + D + D * D;
     constexpr int kWaves = THREADS / 64;
     using Tile = MTile<D, D, T>;
@@ -244,8 +244,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4))) vo
     __shared__ Tile t;
 
     int bl, chunk;
-    map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
+    map_workgroup(blockIdx.x, chunks * ts.slices, n_mixtures, bl, chunk);
     if (bl >= n_mixtures) return;
+    // several slices of tiles per point chunk (launches that would leave compute units idle): `out` was cleared and
+    // every partial result is added
+    const int slice = chunk / chunks;
+    chunk -= slice * chunks;
+    const int g_begin = slice * ts.tiles_per_slice * T;
+    const int g_end = (g_begin + ts.tiles_per_slice * T) < M ? (g_begin + ts.tiles_per_slice * T) : M;
     const int b = bl / L, l = bl - b * L;
     const int xb = b < Bx ? b : Bx - 1, xl = l < Lx ? l : Lx - 1;
     const float* __restrict__ mix_bl = mixture + size_t(bl) * M * G;
@@ -256,8 +262,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4))) vo
     const int j = lane & 15, g = lane >> 4;
     if (threadIdx.x == 0) t.rows[Tile::kZero] = make_uint4(0u, 0u, 0u, 0u);
 
-    for (int g0 = 0; g0 < M; g0 += T) {
-        const int cnt = (M - g0) < T ? (M - g0) : T;
+    for (int g0 = g_begin; g0 < g_end; g0 += T) {
+        const int cnt = (g_end - g0) < T ? (g_end - g0) : T;
         stage_mtile<D, D, T, 4, THREADS>(t, mix_bl + size_t(g0) * G, cnt, 1.0, covariance_form);
         const int centred_start = t.counts[16], padded_total = t.counts[17];
         for (int blk = 0; blk < blocks_per_chunk; ++blk) {
@@ -318,7 +324,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4))) vo
                 const int n = n_base + p * 16 + j;
                 if (g == (p & 3) && n < N) {
                     // later tiles add to what this lane stored for the first one; an atomic needs no round trip
-                    if (g0 == 0) out_bl[n] = v; else atomic_add(&out_bl[n], v);
+                    if (g0 == 0 && ts.slices == 1) out_bl[n] = v; else atomic_add(&out_bl[n], v);
                 }
             }
         }
@@ -351,9 +357,12 @@ static void launch_fwd_variant(const float* mixture, const float* xes, float* ou
                                hipStream_t stream) {
     const size_t BL = size_t(s.B) * s.L;
     const PointPlan plan = plan_points(s.N, BL, THREADS / 64 * 16 * P, 4096);
-    const dim3 grid(unsigned(grid_mixtures(BL) * plan.chunks));
+    // a workgroup here has twice the wavefronts of the all-vector kernels' workgroups
+    const TileSlices ts = plan_tile_slices(2 * grid_mixtures(BL) * plan.chunks, s.M, T);
+    if (ts.slices > 1) zero_async(out, BL * size_t(s.N), stream);
+    const dim3 grid(unsigned(grid_mixtures(BL) * plan.chunks * ts.slices));
     eval_fwd_mfma_kernel<D, P, T, THREADS><<<grid, dim3(THREADS), 0, stream>>>(
-        mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, plan.chunks, plan.blocks_per_chunk, int(BL), cov);
+        mixture, xes, out, s.L, s.M, s.N, s.Bx, s.Lx, plan.chunks, plan.blocks_per_chunk, int(BL), cov, ts);
 }
 
 // true: the matrix-core kernel handles the shape (more than 128 components per mixture and enough points to fill

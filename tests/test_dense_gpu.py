@@ -123,6 +123,25 @@ def test_tile_and_chunk_boundaries(dtype, D):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_few_large_mixtures_split_their_gaussians_over_workgroups(dtype, D):
+    """One or two mixtures with many components make launches of few workgroups; the tiles of Gaussians are then dealt
+    to several workgroups per chunk of points, which add their partial values and dL/dx with atomics into cleared
+    outputs (all-vector forward kernels in both layouts, backward kernel, and in float32 the matrix-core forward
+    kernel from 8192 points on): ragged last tile and last slice, per-mixture and broadcast points, every need flag."""
+    for B, M, N, broadcast in ((1, 1500, 700, False), (2, 2100, 1300, True), (1, 777, 8200, False)):
+        mix, xes, gout = _case(B, 1, M, N, D, 8800 + M, broadcast)
+        _check(mix, xes, gout, dtype, tag=f"sliced B{B} M{M} N{N} D{D}")
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    mix, xes, gout = (a.astype(npdt) for a in _case(1, 1, 1300, 900, D, 8899, False))
+    rgm, rgx = o.evaluate_inversed_backward(gout, mix, xes)
+    _, gmix, _ = _run(mix, xes, gout, dtype, need_m=True, need_x=False)
+    assert rel_l2(gmix, rgm, FLOOR[dtype]) <= TOL[dtype]
+    _, _, gxes = _run(mix, xes, gout, dtype, need_m=False, need_x=True)
+    assert rel_l2(gxes, rgx, FLOOR[dtype]) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_every_points_per_lane_instance(dtype):
     """The backward pair kernel has one instance per number of points per lane, 2 to 16 (8 in float64), chosen from
     the point count: with 256 mixtures a launch takes one chunk of 64 p points whenever that covers N, so N = 64 p - 3
