@@ -33,7 +33,7 @@ VALU_NOTE = ("bound by vector-instruction issue against the FP32 peak of 157.3 T
              "its packed FP32 vector rate); the kernels issue unpacked FP32 vector instructions (measured: one wave64 FMA "
              "per 2.3 cycles and SIMD = 137 TFLOP/s)")
 MFMA_NOTE = VALU_NOTE + "; this kernel takes y = u x - u b from the bf16 matrix cores and keeps |y|^2, exp2 and the sum on the vector ALU"
-PROFILES = {"C4": "eval_dense_fwd_bwd_C4.md", "C5": "eval_bvh_build_fwd_bwd_C5.md"}
+PROFILES = {"C4": "eval_dense_fwd_bwd_C4.md", "C5": "eval_bvh_build_fwd_bwd_C5.md", "C5dense": "eval_dense_fwd_bwd_C5_f64.md"}
 
 
 def profile_traffic(workload: str, kernel_prefix: str):
@@ -475,8 +475,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5", "conv", "cw", "layer"],
-                    help="C1..C4: dense all-pairs path; C5: LBVH-culled path (build + forward + backward per step); "
+    ap.add_argument("--workload", default="C4", choices=["C1", "C2", "C3", "C4", "C5", "C5dense", "conv", "cw", "layer"],
+                    help="C1..C4: dense all-pairs path; C5: LBVH-culled path (build + forward + backward per step); C5dense: the C5 "
+                         "inputs (float64, one mixture) through the dense path; "
                          "conv: closed-form convolution; cw: component-wise evaluation on the C2 shape (forward + "
                          "backward per step); layer: gm.evaluate on covariances forward + backward, the ReLU fixed-point "
                          "fitting and BatchNorm on the C2 shape")
@@ -504,7 +505,8 @@ def main():
         return bench_componentwise(args)
     if args.workload == "layer":
         return bench_layer(args)
-    r = measure_dense(args.workload, args.steps, args.warmup, args.copy_calibration)
+    dense_name = "C5" if args.workload == "C5dense" else args.workload
+    r = measure_dense(dense_name, args.steps, args.warmup, args.copy_calibration)
     wl, ms_step, fwd_ms, bwd_ms = r["wl"], r["ms_step"], r["fwd_ms"], r["bwd_ms"]
     D = wl.dims
     dt = "f32" if wl.dtype == torch.float32 else "f64"
@@ -519,7 +521,7 @@ def main():
         "value": wl.pairs / (ms_step * 1e-3), "unit": "Gaussian-point pairs/s (forward + backward step)",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
-        "config": {"workload": f"{wl.name}: D={D} {dt} B={wl.B} L={wl.L} M={wl.M} N={wl.N}, dense all-pairs, "
+        "config": {"workload": f"{args.workload}: D={D} {dt} B={wl.B} L={wl.L} M={wl.M} N={wl.N}, dense all-pairs, "
                                f"{wl.pairs:.4g} pairs per step, forward + backward (grad mixture and grad xes)"},
         "timing": "ms_per_step: wall clock over all steps / steps; fwd.ms, roofline launch_ms: medians of per-step HIP event pairs",
         "fwd": {"ms": fwd_ms, "pairs_per_s": wl.pairs / (fwd_ms * 1e-3), "tflops": fwd_tf, "frac_of_peak": fwd_tf / peak,
@@ -550,20 +552,35 @@ def main():
                 "fwd_frac_of_peak": FLOP_FWD[d] * w.pairs / (o["fwd_ms"] * 1e-3) / 1e12 / PEAK_TFLOPS["f32"],
                 "fwd_bwd_frac_of_peak": (FLOP_FWD[d] + FLOP_BWD[d]) * w.pairs / (o["ms_step"] * 1e-3) / 1e12 / PEAK_TFLOPS["f32"],
                 "fwd_kernel": o["fwd_kernel"]}
+        o = measure_dense("C2", 20, 3, broadcast_xes=True)
+        others["C2_broadcast_xes"] = {
+            "config": "C2 with the points of the first mixture shared by all 800 ([1, 1, 784, 2]): grad_xes is summed over the mixtures",
+            "fwd_ms": o["fwd_ms"], "bwd_ms": o["bwd_ms"], "ms_per_step": o["ms_step"]}
+        o = measure_dense("C5", 10, 2)
+        w = o["wl"]
+        others["C5_dense_f64"] = {
+            "config": f"the C5 inputs through the dense path: D=3 f64 B=1 L=1 M={w.M} N={w.N}, {w.pairs:.4g} pairs",
+            "fwd_ms": o["fwd_ms"], "bwd_ms": o["bwd_ms"], "ms_per_step": o["ms_step"],
+            "fwd_frac_of_f64_peak": FLOP_FWD[3] * w.pairs / (o["fwd_ms"] * 1e-3) / 1e12 / PEAK_TFLOPS["f64"],
+            "bwd_frac_of_f64_peak": FLOP_BWD[3] * w.pairs / (o["bwd_ms"] * 1e-3) / 1e12 / PEAK_TFLOPS["f64"],
+            "fwd_kernel": o["fwd_kernel"]}
         others["C5"] = {"config": "D=3 f64 B=1 L=1 M=16384 N=100000, LBVH-culled (threshold 0.001): build + forward + backward per step",
                         "by_aabb_mode": [bvh_summary(measure_bvh(mode, 20, 3), mode) for mode in ("reference", "tight")]}
         line["other_workloads"] = others
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.workload)
+        line["cpu_baseline"] = cpu_baseline(dense_name)
     print(json.dumps(line))
 
 
-def measure_dense(name: str, steps: int, warmup: int, copy_calibration: bool = False):
+def measure_dense(name: str, steps: int, warmup: int, copy_calibration: bool = False, broadcast_xes: bool = False):
     """Forward + backward (both gradients) of the dense path on the named workload; timings from HIP events on the
-    launch stream (medians over the steps), the step time from the wall clock over all steps."""
+    launch stream (medians over the steps), the step time from the wall clock over all steps.  broadcast_xes: all
+    mixtures share the points of the first one ([1, 1, N, D]; grad_xes is then summed over the mixtures)."""
     import torch
     from gmc import _native, synthetic
     wl, mix, xes, gout = synthetic.make_workload(name)
+    if broadcast_xes:
+        xes = xes[:1, :1].contiguous()
     dev = torch.device("cuda:0")
     mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)
     torch.cuda.synchronize()

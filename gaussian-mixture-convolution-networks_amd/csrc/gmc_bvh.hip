@@ -897,7 +897,9 @@ __device__ __forceinline__ unsigned long long points_stamp(const T (&x)[D], bool
     h = valid ? h : 0ull;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) h += __shfl_xor(h, off, 64);
-    return h;
+    // the same value in every lane: kept in scalar registers (it stays alive until the list is published)
+    const unsigned lo = __builtin_amdgcn_readfirstlane(unsigned(h)), hi = __builtin_amdgcn_readfirstlane(unsigned(h >> 32));
+    return ((unsigned long long)hi << 32) | lo;
 }
 
 template <typename T>
