@@ -547,14 +547,15 @@ __global__ __launch_bounds__(kBlock) void eval_bwd_epilogue_kernel(const T* __re
 
 // ---- host-side launchers ------------------------------------------------------------------------------
 
-static int pick_points_per_lane(int N, int BL) {
-    // keep the padding of the last chunk small and leave enough workgroups for 256 CUs
+static int pick_points_per_lane(int N, int BL, int tiles) {
+    // keep the padding of the last chunk small and leave enough workgroups for 256 CUs (the tiles of Gaussians of a
+    // mixture can be dealt to several workgroups per chunk, see plan_tile_slices)
     const int cands[4] = {8, 4, 2, 1};
     for (int c : cands) {
         const int span = kBlock * c;
         const int chunks = (N + span - 1) / span;
         const double waste = double(chunks) * span / double(N > 0 ? N : 1);
-        if (waste <= 1.15 && (size_t(chunks) * BL >= 1024 || c == 1)) return c;
+        if (waste <= 1.15 && (size_t(chunks) * BL * tiles >= 1024 || c == 1)) return c;
     }
     int best = 1;
     double best_waste = 1e30;
@@ -581,7 +582,8 @@ struct FwdPlan { int P, chunks, rc; };
 static FwdPlan plan_fwd(const gmc_shape& s, bool is_double) {
     const size_t BL = size_t(s.B) * s.L;
     FwdPlan plan;
-    plan.P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000));
+    const int tiles = (s.M + kTile - 1) / kTile > 0 ? (s.M + kTile - 1) / kTile : 1;
+    plan.P = pick_points_per_lane(s.N, int(BL < 1000000 ? BL : 1000000), tiles);
     plan.chunks = (s.N + kBlock * plan.P - 1) / (kBlock * plan.P);
     // the 4 x 16 layout covers the points in steps of 64 q: taken when that pads the last chunk clearly less
     const int q_max = is_double ? 8 : 16;
@@ -590,7 +592,7 @@ static FwdPlan plan_fwd(const gmc_shape& s, bool is_double) {
     covered_best -= covered_best / 16;                              // the other layout has to win by 6 %
     for (int q = q_max; q >= 2; --q) {
         const size_t q_chunks = (size_t(s.N) + 64 * q - 1) / (64 * q);
-        if (q > 2 && q_chunks * BL < 256) continue;
+        if (q > 2 && q_chunks * BL * tiles < 256) continue;
         if (q_chunks * 64 * q < covered_best) { covered_best = q_chunks * 64 * q; q_best = q; }
     }
     plan.rc = q_best;
@@ -665,7 +667,8 @@ static int bwd_points_per_lane(const gmc_shape& s) {
     for (int cand = p_max; cand >= 2; --cand) {
         const int span = 64 * cand;
         const size_t chunks = (size_t(s.N) + span - 1) / span;
-        if (cand > 2 && chunks * BL < 256) continue;
+        const size_t tiles = (size_t(s.M) + kTile - 1) / kTile > 0 ? (size_t(s.M) + kTile - 1) / kTile : 1;
+        if (cand > 2 && chunks * BL * tiles < 256) continue;
         const double cost = double(chunks) * span * (pair_cost + reduce_cost / cand);
         if (cost < best) { best = cost; P = cand; }
     }
