@@ -44,7 +44,9 @@ struct BvhLayout {
     size_t parts_g, parts_p;    // T [segments][blocks][2D] per-block partial bounds of the centres / the query points
     size_t keys_a, keys_b, vals_a, vals_b;       // uint32 [BL*M]   radix ping-pong of the leaves
     size_t pkeys_a, pkeys_b, pvals_a, pvals_b;   // uint32 [BxLx*N] radix ping-pong of the query points
-    size_t hist_g, hist_p;      // uint32 [segments][blocks][256] block histograms of one radix pass
+    size_t hist_g, hist_p;      // uint32 [4 | 2][segments][blocks][256] block histograms of every radix pass (leaves: 4
+                                // passes, points: 2), adjacent; all zero when the build starts to count
+    size_t hist_words;          // uint32 words from hist_g to the end of hist_p
     size_t p_order;             // int [BxLx][N]           Morton order of the query points
     size_t g_keys;              // uint32 [BL][M]          sorted Morton codes of the leaves
     size_t cand_count;          // int [BL][ceil(N/64)]    candidate leaves of every point group, -1: not known
@@ -151,8 +153,9 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.pkeys_b = take(XL * N * 4);
     l.pvals_a = take(XL * N * 4);
     l.pvals_b = take(XL * N * 4);
-    l.hist_g = take(BL * sort_blocks(M) * 256 * 4);
-    l.hist_p = take(XL * sort_blocks(N) * 256 * 4);
+    l.hist_g = take(4 * BL * sort_blocks(M) * 256 * 4);
+    l.hist_p = take(2 * XL * sort_blocks(N) * 256 * 4);
+    l.hist_words = (o - l.hist_g) / 4;
     l.p_order = take(XL * N * 4);
     l.g_keys = take(BL * M * 4);
     {
@@ -362,11 +365,14 @@ __device__ __forceinline__ T block_bounds(const T (&lo)[D], const T (&hi)[D], T 
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_bounds_kernel(const T* __restrict__ mixture, int M, int blocks_per_mixture,
                                                            T* __restrict__ parts_g, unsigned box_blocks, const T* __restrict__ xes, int N,
-                                                           int blocks_per_xseg, T* __restrict__ parts_p, int* __restrict__ ctl) {
+                                                           int blocks_per_xseg, T* __restrict__ parts_p, int* __restrict__ ctl,
+                                                           uint32_t* __restrict__ hist, size_t hist_words) {
     constexpr int G = 1 + D + D * D;
     __shared__ T red[2 * D][kBlock];
     // first launch of a build: a new tree has no published pieces, an empty pool and no error
     if (blockIdx.x == 0 && threadIdx.x < 4) ctl[threadIdx.x] = 0;
+    // the block histograms of all radix passes are counted with atomics by the kernels that follow
+    for (size_t i = size_t(blockIdx.x) * kBlock + threadIdx.x; i < hist_words; i += size_t(gridDim.x) * kBlock) hist[i] = 0u;
     T lo[D], hi[D];
     for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
     if (blockIdx.x < box_blocks) {
@@ -434,6 +440,7 @@ template <typename T> struct MortonJob {
     const T* parts; int n_parts;                                   // partial bounds of every segment
     uint32_t* keys; uint32_t* vals;
     unsigned blocks;                                               // workgroups of this job in the launch
+    uint32_t* hist; int sort_blocks_per_seg, sort_chunk_shift, shift;   // block histograms of the first radix pass
 };
 
 // Morton keys and index payload for two jobs in one launch (job b behind job a); every workgroup first combines
@@ -461,8 +468,10 @@ __global__ __launch_bounds__(kBlock) void morton_kernel(MortonJob<T> a, MortonJo
     const int i = blk * kBlock + threadIdx.x;
     if (i >= j.count) return;
     const size_t at = size_t(seg) * j.count + i;
-    j.keys[at] = morton30<T, D>(j.pts + at * j.stride + j.offset, bounds);
+    const uint32_t key = morton30<T, D>(j.pts + at * j.stride + j.offset, bounds);
+    j.keys[at] = key;
     j.vals[at] = uint32_t(i);
+    atomicAdd(&j.hist[(size_t(seg) * j.sort_blocks_per_seg + (i >> j.sort_chunk_shift)) * 256 + ((key >> j.shift) & 255u)], 1u);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -471,30 +480,16 @@ __global__ __launch_bounds__(kBlock) void morton_kernel(MortonJob<T> a, MortonJo
 // one pass over one set of segments
 struct SortJob {
     const uint32_t* keys_in; const uint32_t* vals_in; uint32_t* keys_out; uint32_t* vals_out;
-    uint32_t* hist;                      // [segments][blocks_per_seg][256]
-    int count, items, blocks_per_seg, shift;
+    const uint32_t* hist;                // [segments][blocks_per_seg][256] of this pass
+    uint32_t* hist_next;                 // the same for the next pass, counted here; null in the last pass
+    int count, items, blocks_per_seg, shift, chunk_shift;
     unsigned blocks;                     // workgroups of this job in the launch
     int* err;                            // error flags of the BVH object
 };
 
-// block histograms of the pass's digit, for two jobs in one launch (job b behind job a)
-__global__ __launch_bounds__(kBlock) void radix_hist_kernel(SortJob a, SortJob b) {
-    __shared__ uint32_t h[256];
-    const bool first = blockIdx.x < a.blocks;
-    const SortJob& j = first ? a : b;
-    const unsigned id = first ? blockIdx.x : blockIdx.x - a.blocks;
-    const int seg = id / j.blocks_per_seg, blk = id - seg * j.blocks_per_seg;
-    h[threadIdx.x] = 0;
-    __syncthreads();
-    const uint32_t* k = j.keys_in + size_t(seg) * j.count;
-    const int chunk = j.items * kBlock;
-    const int begin = blk * chunk;
-    const int end = begin + chunk < j.count ? begin + chunk : j.count;
-    for (int i = begin + threadIdx.x; i < end; i += kBlock) atomicAdd(&h[(k[i] >> j.shift) & 255u], 1u);
-    __syncthreads();
-    j.hist[size_t(id) * 256 + threadIdx.x] = h[threadIdx.x];
-}
-
+// One pass of the sort for two jobs in one launch (job b behind job a).  The block histograms of a pass are counted
+// by the kernel that writes the pass's input (the Morton kernel, or the pass before) with one atomic per key, which
+// saves a histogram launch per pass: the passes are short kernels, bound by launch latency.
 __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJob b) {
     __shared__ uint32_t running[256];        // next output slot of every digit for this block
     __shared__ uint32_t wave_count[4][256];
@@ -580,6 +575,8 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJo
             if (slot < uint32_t(count)) {          // always true for a consistent histogram; keeps a bug from writing out of bounds
                 j.keys_out[seg_off + slot] = key;
                 j.vals_out[seg_off + slot] = val;
+                if (j.hist_next)
+                    atomicAdd(&j.hist_next[(size_t(seg) * blocks_per_seg + (slot >> j.chunk_shift)) * 256 + ((key >> (shift + 8)) & 255u)], 1u);
             } else {
                 atomicOr(j.err, kErrSort);
             }
@@ -1563,10 +1560,14 @@ static SortJob sort_job(uint32_t* ka, uint32_t* va, uint32_t* kb, uint32_t* vb, 
     j.keys_in = odd ? kb : ka; j.vals_in = odd ? vb : va;
     j.keys_out = odd ? ka : kb; j.vals_out = odd ? va : vb;
     if (pass == passes - 1) { j.keys_out = keys_out; j.vals_out = vals_out; }
-    j.hist = hist;
     j.count = count;
     j.items = sort_items(size_t(count));
     j.blocks_per_seg = int(sort_blocks(size_t(count)));
+    const size_t pass_words = segments * size_t(j.blocks_per_seg) * 256;
+    j.hist = hist + size_t(pass) * pass_words;
+    j.hist_next = pass + 1 < passes ? hist + size_t(pass + 1) * pass_words : nullptr;
+    j.chunk_shift = 8;
+    for (int it = j.items; it > 1; it >>= 1) ++j.chunk_shift;
     j.shift = first_bit + 8 * pass;
     j.blocks = unsigned(segments * size_t(j.blocks_per_seg));
     return j;
@@ -1603,23 +1604,31 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     const unsigned box_blocks = have_g ? unsigned(BL * bpm) : 0u, bound_blocks = sort_p ? unsigned(XL * nbp) : 0u;
     if (box_blocks + bound_blocks > 0)
         bvh_bounds_kernel<T, D><<<dim3(box_blocks + bound_blocks), dim3(kBlock), 0, st>>>(
-            mixture, M, bpm, parts_g, box_blocks, xes, N, nbp, parts_p, (int*)(bvh + lay.cand_ctl));
+            mixture, M, bpm, parts_g, box_blocks, xes, N, nbp, parts_p, (int*)(bvh + lay.cand_ctl),
+            (uint32_t*)(bvh + lay.hist_g), lay.hist_words);
+    const int p_passes = N > kCoarseOrderMax ? 2 : 1;
+    auto jobs_of_pass = [&](int pass, SortJob& jg, SortJob& jp) {
+        jg = sort_job(ka, va, kb, vb, g_keys, g_order, (uint32_t*)(bvh + lay.hist_g), have_g ? BL : 0, M, 0, 4, pass, (int*)(bvh + lay.cand_ctl));
+        jp = sort_job(pka, pva, pkb, pvb, p_passes == 1 ? pkb : pka, (uint32_t*)p_order,
+                      (uint32_t*)(bvh + lay.hist_p), sort_p ? XL : 0, N, 30 - 8 * p_passes, p_passes, pass,
+                      (int*)(bvh + lay.cand_ctl));
+    };
+    SortJob jg0, jp0;
+    jobs_of_pass(0, jg0, jp0);
     MortonJob<T> mg = {}, mp = {};
-    if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm)};
-    if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx)};
+    if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm),
+                                  (uint32_t*)jg0.hist, jg0.blocks_per_seg, jg0.chunk_shift, jg0.shift};
+    if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx),
+                                  (uint32_t*)jp0.hist, jp0.blocks_per_seg, jp0.chunk_shift, jp0.shift};
     if (mg.blocks + mp.blocks > 0) morton_kernel<T, D><<<dim3(mg.blocks + mp.blocks), dim3(kBlock), 0, st>>>(mg, mp);
     // leaves: all 30 key bits; points: the top 16 Morton bits (65536 cells) are enough to make 64 consecutive
     // points neighbours, the top 8 bits for segments of at most kCoarseOrderMax points (32 points per cell; measured:
     // same traversal times, one sort pass less).  The sorted keys of the points are not needed afterwards: they
     // land in a spare buffer, which must not be the input of the last pass.
-    const int p_passes = N > kCoarseOrderMax ? 2 : 1;
     for (int pass = 0; pass < 4; ++pass) {
-        const SortJob jg = sort_job(ka, va, kb, vb, g_keys, g_order, (uint32_t*)(bvh + lay.hist_g), have_g ? BL : 0, M, 0, 4, pass, (int*)(bvh + lay.cand_ctl));
-        const SortJob jp = sort_job(pka, pva, pkb, pvb, p_passes == 1 ? pkb : pka, (uint32_t*)p_order,
-                                    (uint32_t*)(bvh + lay.hist_p), sort_p ? XL : 0, N, 30 - 8 * p_passes, p_passes, pass,
-                                    (int*)(bvh + lay.cand_ctl));
+        SortJob jg, jp;
+        jobs_of_pass(pass, jg, jp);
         if (jg.blocks + jp.blocks == 0) continue;
-        radix_hist_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
         radix_scatter_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
     }
     if (have_g) {
