@@ -1012,6 +1012,28 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                                      : wave * chunks + (chunk + wave * (chunks / (groups + 1))) % chunks;
         const int j = group * kWave + lane;
         const bool valid = j < N;
+        // What an earlier traversal has left for this group is fetched together with the points, not after them: each
+        // of these reads is a round trip through memory, and in a chain they add up to more than the evaluation of
+        // a short list.  (The group's fixed slot of the list exists whatever its state; a backward owner works on at
+        // most kPieceLeaves entries of it, a piece has at most as many.)
+        constexpr int kAhead = (kPieceLeaves + kWave - 1) / kWave;
+        int known_ahead = -1, list_ahead[kAhead];
+        unsigned long long stamp_ahead = 0ull;
+        int2 range_ahead = make_int2(0, 0);
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) list_ahead[k] = 0;
+        const bool look = cache.count && group * kWave < N && (piece >= 0 || M > 1);
+        if (look) {
+            const size_t slot = piece >= 0 ? size_t(piece_desc.x) : size_t(bl) * per_mixture + group;
+            known_ahead = cache.count[slot];
+            stamp_ahead = cache.stamp[slot];
+            if (piece >= 0) range_ahead = cache.piece_range[slot];
+            const int* src = piece >= 0 ? cache.list + piece_desc.y : cache.list + slot * kLeafCap;
+            const int n_ahead = piece >= 0 ? piece_desc.z : kLeafCap;
+#pragma unroll
+            for (int k = 0; k < kAhead; ++k)
+                if (lane + k * kWave < n_ahead) list_ahead[k] = src[lane + k * kWave];
+        }
         int pid = valid ? p_order[xseg * N + j] : 0;
         pid = unsigned(pid) < unsigned(N) ? pid : 0;        // a permutation by construction; never index out of bounds
         T x[D];
@@ -1041,13 +1063,15 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             // A piece is worked on only while it is one of the pieces its group has published last, for points with
             // the stamp of the ones loaded here; the owner of the group applies the same test to the list and
             // otherwise evaluates all of it itself.
-            const int slot = piece_desc.x;
-            const int known = cache.count[slot];
-            const int2 range = cache.piece_range[slot];
+            const int known = look ? known_ahead : -1;
+            const int2 range = range_ahead;
             const bool ok = known >= 0 && (known & kCandSplit) != 0 && piece >= range.x && piece < range.x + range.y &&
-                            cache.stamp[slot] == my_stamp;
+                            stamp_ahead == my_stamp;
             if (lane == 0) piece_valid = ok ? 1 : 0;
-            for (int i = lane; i < piece_desc.z; i += kWave) leaves[0][i] = cache.list[piece_desc.y + i];
+#pragma unroll
+            for (int k = 0; k < kAhead; ++k)
+                if (lane + k * kWave < piece_desc.z) leaves[0][lane + k * kWave] = list_ahead[k];
+            for (int i = lane + kAhead * kWave; i < piece_desc.z; i += kWave) leaves[0][i] = cache.list[piece_desc.y + i];
             if (lane == 0) state[0][0] = piece_desc.z;
             sp = 0;
         } else if (cache.count && sp > 0) {
@@ -1055,8 +1079,8 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             // published pieces of a long list to the helper workgroups; the forward pass has no helpers, so it
             // takes a whole single-round list and descends again for a list of several rounds.
             cache_slot = bl * per_mixture + group;
-            const int known = __builtin_amdgcn_readfirstlane(cache.count[cache_slot]);
-            if (known >= 0 && cache.stamp[cache_slot] != my_stamp) {
+            const int known = __builtin_amdgcn_readfirstlane(known_ahead);
+            if (known >= 0 && stamp_ahead != my_stamp) {
                 // a list for other points (another tensor, or this one changed in place): descend.  The forward pass
                 // then replaces the list; a backward launch leaves the group's entries alone, because helper
                 // workgroups of the same launch may be reading them.
@@ -1068,7 +1092,10 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                 const int all = known & kCandMask;
                 const int n = (MODE == 1 && (known & kCandSplit)) ? own_share(all) : all;
                 if (MODE == 1 || !(known & kCandRounds)) {
-                    for (int i = lane; i < n; i += kWave) leaves[wave][i] = cache.list[size_t(cache_slot) * kLeafCap + i];
+#pragma unroll
+                    for (int k = 0; k < kAhead; ++k)
+                        if (lane + k * kWave < n) leaves[wave][lane + k * kWave] = list_ahead[k];
+                    for (int i = lane + kAhead * kWave; i < n; i += kWave) leaves[wave][i] = cache.list[size_t(cache_slot) * kLeafCap + i];
                     if (lane == 0) state[wave][0] = n;
                     sp = 0;
                 }
