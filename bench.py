@@ -25,6 +25,7 @@ FLOP_BWD = {2: 30, 3: 52}
 # util/gaussian.h:82-95); reported for transparency only, never as the headline
 FLOP_FWD_LITERAL = {2: 15, 3: 27}
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}     # MI355X vector peaks
+PEAK_CLOCK_MHZ = 2400.0                        # the engine clock those peaks are quoted at (256 CUs x 256 flop/cycle x 2.4 GHz)
 # The dense kernels are bound by FP32 arithmetic.  MI355X's FP32 matrix rate equals its (packed) FP32 vector rate,
 # 157.3 TFLOP/s, which is the peak the metric names.  `bound` says which unit issues the kernel's arithmetic: "valu"
 # for the all-vector kernels, "mfma" for the forward kernel that takes the affine part from the matrix cores, "hbm"
@@ -515,6 +516,11 @@ def main():
     bwd_tf = FLOP_BWD[D] * wl.pairs / (bwd_ms * 1e-3) / 1e12
     step_tf = (FLOP_FWD[D] + FLOP_BWD[D]) * wl.pairs / (ms_step * 1e-3) / 1e12
     fwd_kernel = r["fwd_kernel"]
+    fwd_mhz, bwd_mhz = r["clocks_mhz"]
+
+    def at_measured_clock(frac, mhz):
+        """what the fraction of the published peak (quoted at PEAK_CLOCK_MHZ) is against the clock the launch ran at"""
+        return {"shader_clock_mhz": mhz, "frac_at_that_clock": frac * PEAK_CLOCK_MHZ / mhz} if mhz > 0 else {}
 
     line = {
         "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
@@ -532,12 +538,13 @@ def main():
                                "the time, are inside the event pair)",
                      "bound": "valu", "bound_detail": VALU_NOTE, "achieved": bwd_tf, "peak": peak, "unit": "TFLOP/s", "frac": bwd_tf / peak,
                      "traffic": profile_traffic(args.workload, "eval_bwd_rc_kernel"), "launch_ms": bwd_ms,
-                     "flop_per_pair": FLOP_BWD[D]},
+                     "flop_per_pair": FLOP_BWD[D], **at_measured_clock(bwd_tf / peak, bwd_mhz)},
         "roofline_fwd": {"kernel": fwd_kernel, "bound": "mfma" if fwd_kernel == "eval_fwd_mfma_kernel" else "valu",
                          "bound_detail": MFMA_NOTE if fwd_kernel == "eval_fwd_mfma_kernel" else VALU_NOTE,
                          "achieved": fwd_tf, "peak": peak,
                          "unit": "TFLOP/s", "frac": fwd_tf / peak, "launch_ms": fwd_ms, "flop_per_pair": FLOP_FWD[D],
-                         "traffic": profile_traffic(args.workload, fwd_kernel)},
+                         "traffic": profile_traffic(args.workload, fwd_kernel),
+                         **(at_measured_clock(fwd_tf / peak, fwd_mhz) if fwd_kernel == "eval_fwd_mfma_kernel" else {})},
     }
     if args.workload == "C4" and not args.no_other_workloads:
         # every other configuration of the baseline, measured in the same process after the timed region of C4
@@ -551,7 +558,9 @@ def main():
                 "fwd_pairs_per_s": w.pairs / (o["fwd_ms"] * 1e-3), "fwd_bwd_pairs_per_s": w.pairs / (o["ms_step"] * 1e-3),
                 "fwd_frac_of_peak": FLOP_FWD[d] * w.pairs / (o["fwd_ms"] * 1e-3) / 1e12 / PEAK_TFLOPS["f32"],
                 "fwd_bwd_frac_of_peak": (FLOP_FWD[d] + FLOP_BWD[d]) * w.pairs / (o["ms_step"] * 1e-3) / 1e12 / PEAK_TFLOPS["f32"],
-                "fwd_kernel": o["fwd_kernel"]}
+                "fwd_kernel": o["fwd_kernel"],
+                # short launches with gaps between them do not bring the clock up to what the long ones of C4 reach
+                "bwd_shader_clock_mhz": o["clocks_mhz"][1]}
         o = measure_dense("C2", 20, 3, broadcast_xes=True)
         others["C2_broadcast_xes"] = {
             "config": "C2 with the points of the first mixture shared by all 800 ([1, 1, 784, 2]): grad_xes is summed over the mixtures",
@@ -613,7 +622,11 @@ def measure_dense(name: str, steps: int, warmup: int, copy_calibration: bool = F
     wall = time.perf_counter() - t0
     import ctypes
     shape = _native.check_input(mix, xes)
-    return {"wl": wl, "ms_step": wall * 1e3 / steps,
+    # shader clock that one workgroup in the middle of the last forward (float32 matrix-core kernel) and backward
+    # launch saw: under this load the clock settles below the 2400 MHz that the published peak assumes
+    mhz = (ctypes.c_double * 2)()
+    clocks = (mhz[0], mhz[1]) if _native.lib().gmc_export_launch_clocks(mhz) == 0 else (0.0, 0.0)
+    return {"wl": wl, "ms_step": wall * 1e3 / steps, "clocks_mhz": clocks,
             "fwd_ms": median([e[0].elapsed_time(e[1]) for e in events]),
             "bwd_ms": median([e[1].elapsed_time(e[2]) for e in events]),
             "fwd_kernel": _native.lib().gmc_eval_fwd_kernel_name(ctypes.byref(shape)).decode()}

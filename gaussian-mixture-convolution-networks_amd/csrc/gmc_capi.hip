@@ -13,6 +13,8 @@ int dense_backward_static(const void* grad_out, const void* mixture, const void*
                           const gmc_shape& s, bool need_gm, bool need_gx, bool covariance_form, hipStream_t stream);
 
 const char* dense_forward_kernel_name(const gmc_shape& s);
+int dense_forward_f32_clocks(long long* ticks);
+int dense_backward_clocks(long long* ticks);
 void set_tuning(int fwd_points_per_lane, int bwd_points_per_lane);
 
 int check_shape(const gmc_shape* s) {
@@ -35,7 +37,7 @@ int check_shape(const gmc_shape* s) {
 
 extern "C" {
 
-int gmc_abi_version(void) { return 6; }
+int gmc_abi_version(void) { return 7; }
 
 const char* gmc_error_string(int code) {
     switch (code) {
@@ -71,6 +73,19 @@ int gmc_eval_cov_fwd(const void* mixture, const void* xes, void* out, const gmc_
 }
 
 void gmc_set_tuning(int fwd_points_per_lane, int bwd_points_per_lane) { gmc::set_tuning(fwd_points_per_lane, bwd_points_per_lane); }
+
+int gmc_export_launch_clocks(double* shader_mhz) {
+    if (!shader_mhz) return GMC_E_NULL;
+    int device = 0, wall_khz = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, device) != hipSuccess || wall_khz <= 0)
+        return GMC_E_LAUNCH;
+    long long f[2] = {0, 0}, b[2] = {0, 0};
+    if (gmc::dense_forward_f32_clocks(f) != GMC_OK || gmc::dense_backward_clocks(b) != GMC_OK) return GMC_E_LAUNCH;
+    shader_mhz[0] = f[1] > 0 ? double(f[0]) / double(f[1]) * wall_khz * 1e-3 : 0.0;
+    shader_mhz[1] = b[1] > 0 ? double(b[0]) / double(b[1]) * wall_khz * 1e-3 : 0.0;
+    return GMC_OK;
+}
 
 const char* gmc_eval_fwd_kernel_name(const gmc_shape* shape) {
     if (gmc::check_shape(shape) != GMC_OK) return "";

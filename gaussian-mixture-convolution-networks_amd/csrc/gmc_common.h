@@ -346,6 +346,26 @@ inline TileSlices plan_tile_slices(size_t workgroups, int M, int tile) {
     return t;
 }
 
+// Shader clock under the load of a launch, for benchmark reports.  The clock of the vector ALUs is not a constant
+// of the device: with all of them busy it settles well below the peak engine clock, which bounds what a
+// compute-bound kernel can reach.  One workgroup in the middle of the grid reads the shader-clock counter and the
+// constant-rate counter when it starts and when it ends and leaves the two differences; the counters are scalar
+// reads, the values live in scalar registers.
+struct ClockProbe {
+    long long shader0, wall0;
+    bool on;
+};
+__device__ __forceinline__ ClockProbe clock_probe_begin() {
+    ClockProbe c;
+    c.on = blockIdx.x == gridDim.x / 2;
+    c.shader0 = c.on ? clock64() : 0;
+    c.wall0 = c.on ? wall_clock64() : 0;
+    return c;
+}
+__device__ __forceinline__ void clock_probe_end(const ClockProbe& c, long long* __restrict__ out) {
+    if (c.on && threadIdx.x == 0) { out[0] = clock64() - c.shader0; out[1] = wall_clock64() - c.wall0; }
+}
+
 // Per-Gaussian partial sums of the backward pass, in the transformed coordinates y = u (x - b):
 //   R0 = sum_n e g,  R1_i = sum_n e g y_i,  R2_ij = sum_n e g y_i y_j (i <= j)     with e = exp2(-|y|^2)
 template <int D> struct Sums { static constexpr int k = 1 + D + D * (D + 1) / 2; };   // 6 / 10

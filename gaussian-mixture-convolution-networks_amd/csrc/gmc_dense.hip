@@ -24,6 +24,8 @@ namespace gmc {
 // address; host code never uses the array's name as an address, only what hipGetSymbolAddress returned for the
 // device that is current (kept per device below).
 static __device__ __align__(256) unsigned char scratch[GMC_STATIC_SCRATCH_BYTES];
+// (shader-clock ticks, constant-rate ticks) of one workgroup of the last backward pair launch (ClockProbe)
+static __device__ long long backward_clocks[2];
 constexpr int kMaxDevices = 64;
 static std::atomic<void*> scratch_address[kMaxDevices];
 
@@ -313,6 +315,7 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
     // 54.0 KB are not
     static_assert(sizeof(T) == 8 || sizeof(lds) + sizeof(block_sums) + 64 <= 53760, "LDS of the backward pair kernel");
 
+    const ClockProbe probe = clock_probe_begin();
     int bl, chunk;
     map_workgroup(blockIdx.x, chunks * ts.slices, n_mixtures, bl, chunk);
     if (bl >= n_mixtures) return;
@@ -412,6 +415,7 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
             bwd_epilogue_one<T, D>(mixture + at * G, sums + at * NR, grad_mixture + at * G, covariance_form);
         }
     }
+    clock_probe_end(probe, backward_clocks);
 }
 
 // Epilogue, one lane per Gaussian: (R0, R1, R2) -> (dw, db, dC), written to grad_mixture in the reference's
@@ -770,6 +774,12 @@ bool dense_forward_f32_takes(const gmc_shape& s);
 const char* dense_forward_kernel_name(const gmc_shape& s) {
     if (s.dtype == GMC_F32 && dense_forward_f32_takes(s)) return "eval_fwd_mfma_kernel";
     return plan_fwd(s, s.dtype == GMC_F64).rc > 0 ? "eval_fwd_rc_kernel" : "eval_fwd_kernel";
+}
+
+// (shader-clock ticks, constant-rate ticks) left by the last backward pair launch on the current device; waits for
+// the device's work on the null stream like any plain copy from a device symbol
+int dense_backward_clocks(long long* ticks) {
+    return hipMemcpyFromSymbol(ticks, HIP_SYMBOL(backward_clocks), sizeof(long long) * 2) == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
 size_t dense_backward_workspace_bytes(const gmc_shape& s) {

@@ -231,6 +231,9 @@ __device__ __forceinline__ void load_centred_record(const uint4* rows, int slot,
 // walks over `blocks_per_chunk` blocks of (THREADS / 64) * 16 P points for every staged tile, so the per-Gaussian
 // preparation is shared by that many points; partial results of tiles after the first are added to `out` by the
 // lane that stored the first.
+// (shader-clock ticks, constant-rate ticks) of one workgroup of the last launch of the kernel below (ClockProbe)
+static __device__ long long forward_clocks[2];
+
 template <int D, int P, int T, int THREADS>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4))) void eval_fwd_mfma_kernel(const float* __restrict__ mixture,
                                                                 const float* __restrict__ xes, float* __restrict__ out,
@@ -243,6 +246,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4))) vo
     constexpr int kSlots = Tile::kSlots;
     __shared__ Tile t;
 
+    const ClockProbe probe = clock_probe_begin();
     int bl, chunk;
     map_workgroup(blockIdx.x, chunks * ts.slices, n_mixtures, bl, chunk);
     if (bl >= n_mixtures) return;
@@ -329,9 +333,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4))) vo
             }
         }
     }
+    clock_probe_end(probe, forward_clocks);
 }
 
 // ---- host side -------------------------------------------------------------------------------------------
+
+int dense_forward_f32_clocks(long long* ticks) {
+    return hipMemcpyFromSymbol(ticks, HIP_SYMBOL(forward_clocks), sizeof(long long) * 2) == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+}
 
 struct PointPlan {
     int chunks;             // workgroups per mixture

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 6
+ABI_VERSION = 7
 STATIC_SCRATCH_BYTES = 64 << 20
 
 
@@ -61,6 +61,7 @@ def lib() -> ctypes.CDLL:
     l.gmc_eval_fwd.argtypes = [vp, vp, vp, shp, vp]
     l.gmc_set_tuning.restype = None
     l.gmc_set_tuning.argtypes = [ci, ci]
+    l.gmc_export_launch_clocks.argtypes = [ctypes.POINTER(ctypes.c_double)]
     l.gmc_eval_fwd_kernel_name.restype = ctypes.c_char_p
     l.gmc_eval_fwd_kernel_name.argtypes = [shp]
     l.gmc_eval_bwd_workspace_bytes.restype = sz

@@ -62,6 +62,13 @@ void gmc_set_tuning(int fwd_points_per_lane, int bwd_points_per_lane);
  * reference): "eval_fwd_mfma_kernel" (float32, more than 128 components, enough work for 512-component tiles),
  * "eval_fwd_rc_kernel" or "eval_fwd_kernel" (all vector ALU, two layouts); "" for an invalid shape. */
 const char* gmc_eval_fwd_kernel_name(const gmc_shape* shape);
+/* Shader clock in MHz that one workgroup in the middle of the grid saw during the last launch of the float32
+ * matrix-core forward kernel (shader_mhz[0]) and of the backward pair kernel (shader_mhz[1]) on the current device; 0
+ * before the first such launch.  For benchmark reports (no counterpart in the reference): with the vector ALUs busy
+ * the clock settles below the peak engine clock that published peak rates assume.  `shader_mhz` is host memory
+ * for two doubles; the call waits for the device like a plain copy from device memory (do not call it under graph
+ * capture). */
+int gmc_export_launch_clocks(double* shader_mhz);
 
 /* gmc_eval_bwd replaces evaluate_inversed::parallel_backward
  *   (evaluate_inversed.cpp:22-34, parallel_implementation.cu:102-176, parallel_implementation_optimised_backward.cu:111-169).
