@@ -594,3 +594,10 @@ def test_c4_full_size_properties():
                                     xes[b:b + 1, l:l + 1].cpu().numpy().astype(np.float64), n_threads=16)
         assert rel_l2(g1m[b:b + 1, l:l + 1].cpu().numpy(), rgm) < 1e-5
         assert rel_l2(g1x[b:b + 1, l:l + 1].cpu().numpy(), rgx) < 1e-5
+    # the two headline kernels have just run at full size: the clocks they left are those of a busy device
+    import ctypes
+    mhz = (ctypes.c_double * 2)()
+    torch.cuda.synchronize()
+    assert _native.lib().gmc_export_launch_clocks(mhz) == 0
+    assert 800.0 < mhz[0] < 3500.0 and 800.0 < mhz[1] < 3500.0, (mhz[0], mhz[1])
+    assert _native.lib().gmc_export_launch_clocks(None) != 0
