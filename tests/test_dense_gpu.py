@@ -13,6 +13,7 @@ import cpu_ref
 import error_budget as eb
 import gm_oracle as o
 from conftest import rel_l2
+from gmc import _native
 from gmc import mixture as gm
 from gmc import synthetic
 
