@@ -1,9 +1,10 @@
 """ReLU transfer fitting on top of the evaluation path: the part of the reference's src/gmc/fitting.py that calls
 gm.evaluate with the mixture's own centres as query points (initial_approx_to_relu :279-284,
 fixed_point_iteration_to_relu :287-312, generate_random_sampling :315-322).  The evaluations run through the HIP
-kernels: without gradients (inference, or inputs that require none) each evaluation and the element-wise update
-that follows it are one launch (gmc_relu_fit_goal / gmc_relu_fit_step); when gradients flow through the fitting, as in
-the reference's training, the evaluations are the differentiable gm.evaluate and the updates torch operations.  The
+kernels: each evaluation and the element-wise update that follows it are one launch (gmc_relu_fit_goal /
+gmc_relu_fit_step); when gradients flow through the fitting, as in the reference's training, one iteration (the
+reference's default) keeps those launches and differentiates by hand around the backward kernels of the evaluation
+(_FusedReluFit), several iterations are composed of the differentiable gm.evaluate and torch operations.  The
 tree-based reduction fitters of that file are not part of this package."""
 import typing
 
@@ -24,6 +25,63 @@ def initial_approx_to_relu(mixture: Tensor, constant: Tensor) -> Tensor:
     c = constant.unsqueeze(-1)
     new_w = torch.where(w + c > 0, w, -_relu(c).expand_as(w))
     return gm.pack_mixture(new_w, gm.positions(mixture), gm.covariances(mixture))
+
+
+class _FusedReluFit(torch.autograd.Function):
+    """One fixed-point iteration with gradients: the forward pass is the two fused launches of the inference path;
+    the backward pass differentiates  x1 = x0 (b + 0.05) / (cur + 0.05),  x0 = |w| + 0.1,
+    b = relu(v + c) - relu(c),  v = evaluate(target, centres),  cur = evaluate(fit with weights x0, centres)
+    by hand and sends the two upstream gradients d v and d cur through the backward kernels of the evaluation
+    (covariance form), whose gradients with respect to the query points come back to the centres."""
+
+    @staticmethod
+    def forward(ctx, target_mixture: Tensor, target_constant: Tensor, fitting_mixture: Tensor) -> Tensor:
+        target, fit = target_mixture.contiguous(), fitting_mixture.contiguous()
+        goal = _native.relu_fit_goal(target, target_constant, fit)
+        x0 = gm.weights(fit).abs() + 0.1
+        x1 = _native.relu_fit_step(fit, x0, goal)
+        out = fit.clone()
+        out[..., 0] = x1
+        ctx.save_for_backward(target, target_constant, fit, goal)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out: Tensor):
+        target, constant, fit, b = ctx.saved_tensors
+        D = gm.n_dimensions(fit)
+        need_target, need_constant, need_fit = ctx.needs_input_grad
+        grad_out = grad_out.contiguous()
+        w = fit[..., 0]
+        x0 = w.abs() + 0.1
+        centres = fit[..., 1:1 + D].contiguous()
+        fit_abs = fit.clone()
+        fit_abs[..., 0] = x0
+        cur = _native.eval_fwd(fit_abs, centres, covariance_form=True) + 0.05
+        d_x1 = grad_out[..., 0]
+        ratio = (b + 0.05) / cur
+        d_b = d_x1 * x0 / cur
+        d_cur = -d_x1 * x0 * ratio / cur
+        c = constant.expand(b.shape[0], b.shape[1]).unsqueeze(-1)
+        relu_c = torch.clamp(c, min=0)
+        lifted = (b + relu_c) > 0                                    # v + c > 0
+        d_v = (d_b * lifted).contiguous()
+        grad_target = grad_constant = grad_fit = None
+        g_target, g_centres = _native.eval_bwd(d_v, target, centres, need_target, need_fit, covariance_form=True)
+        if need_target:
+            grad_target = g_target
+        if need_constant:
+            g = (d_b * (lifted.to(d_b.dtype) - (c > 0).to(d_b.dtype))).sum(-1)
+            for dim in (0, 1):
+                if constant.shape[dim] == 1 and g.shape[dim] != 1:
+                    g = g.sum(dim, keepdim=True)
+            grad_constant = g
+        if need_fit:
+            g_abs, g_centres2 = _native.eval_bwd(d_cur.contiguous(), fit_abs, centres, True, True, covariance_form=True)
+            grad_fit = grad_out.clone()
+            grad_fit[..., 0] = torch.sign(w) * (d_x1 * ratio + g_abs[..., 0])
+            grad_fit[..., 1:1 + D] += g_abs[..., 1:1 + D] + g_centres + g_centres2
+            grad_fit[..., 1 + D:] += g_abs[..., 1 + D:]
+        return grad_target, grad_constant, grad_fit
 
 
 def fixed_point_iteration_to_relu(target_mixture: Tensor, target_constant: Tensor, fitting_mixture: Tensor,
@@ -58,15 +116,22 @@ def fixed_point_iteration_to_relu(target_mixture: Tensor, target_constant: Tenso
         out[..., 0] = x
         return out, out_constant
 
+    if n_iter == 1:
+        return _FusedReluFit.apply(target_mixture, target_constant, fitting_mixture), out_constant
+    return _composed_fixed_point(target_mixture, target_constant, fitting_mixture, n_iter), out_constant
+
+
+def _composed_fixed_point(target_mixture: Tensor, target_constant: Tensor, fitting_mixture: Tensor, n_iter: int) -> Tensor:
+    """the iteration as the reference writes it (fitting.py:296-311): differentiable evaluations, torch operations"""
     centres = gm.positions(fitting_mixture).contiguous()
     covariances = gm.covariances(fitting_mixture)
-    goal = _relu(gm.evaluate(target_mixture, centres) + target_constant.unsqueeze(-1)) - out_constant.unsqueeze(-1)
+    goal = _relu(gm.evaluate(target_mixture, centres) + target_constant.unsqueeze(-1)) - _relu(target_constant).unsqueeze(-1)
     x = gm.weights(fitting_mixture).abs() + 0.1
     for _ in range(n_iter):
         x = x.abs()
         current = gm.evaluate(gm.pack_mixture(x, centres, covariances), centres)
         x = x * (goal + 0.05) / (current + 0.05)
-    return gm.pack_mixture(x, centres, covariances), out_constant
+    return gm.pack_mixture(x, centres, covariances)
 
 
 def generate_random_sampling(m: Tensor, n: int) -> Tensor:

@@ -206,6 +206,42 @@ def test_fused_fitting_kernels_against_their_differentiable_composition(dims, dt
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("dims", [(2, 3, 70, 33, 2), (1, 2, 300, 200, 3)])
+@pytest.mark.parametrize("broadcast_constant", [False, True])
+def test_fused_fitting_gradients(dims, dtype, broadcast_constant):
+    """One iteration with gradients keeps the fused launches and differentiates by hand around the evaluation's
+    backward kernels: values and all three gradients must equal those of the reference's formulation (differentiable
+    evaluations and torch operations, fitting.py:296-311), also with constants on both sides of zero, negative fitting
+    weights and an upstream gradient on every entry of the returned mixture."""
+    B, L, Mt, Mf, D = dims
+    rng = np.random.default_rng(sum(dims) + 7)
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    target = _cov_mixture(rng, B, L, Mt, D, cov=0.1).astype(npdt)
+    const = (rng.normal(size=(1 if broadcast_constant else B, L)) * 0.3).astype(npdt)
+    fit = _cov_mixture(rng, B, L, Mf, D, cov=0.1).astype(npdt)
+    fit[..., 0] *= np.where(rng.random(fit.shape[:-1]) < 0.3, -1.0, 1.0)
+    upstream = torch.tensor(rng.normal(size=fit.shape).astype(npdt), device=DEV)
+    grads = []
+    for composed in (False, True):
+        t, c, f = (torch.tensor(a, device=DEV, requires_grad=True) for a in (target, const, fit))
+        if composed:
+            out = fitting._composed_fixed_point(t, c, f, 1)
+        else:
+            out, _ = fitting.fixed_point_iteration_to_relu(t, c, f, 1)
+        out.backward(upstream)
+        grads.append([out.detach().cpu().numpy()] + [v.grad.cpu().numpy() for v in (t, c, f)])
+    tol = 20 * TOL[dtype]                                   # two chained evaluations, a division, two backward passes
+    for got, want, what in zip(grads[0], grads[1], ("values", "grad target", "grad constant", "grad fitting")):
+        assert got.shape == want.shape, what
+        assert rel_l2(got, want) <= tol, what
+    # the constant's own output: relu(constant) stays a torch operation
+    t, c, f = (torch.tensor(a, device=DEV, requires_grad=True) for a in (target, const, fit))
+    _, rc = fitting.fixed_point_iteration_to_relu(t, c, f, 1)
+    rc.sum().backward()
+    assert np.array_equal(c.grad.cpu().numpy(), (const > 0).astype(npdt))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("D", [2, 3])
 def test_fused_moments_are_std_mean_of_the_sampled_values(D, dtype):
     """gmc_eval_cov_moments against torch.std_mean of the values that gm.evaluate returns and against numpy on the
