@@ -188,6 +188,29 @@ def test_several_point_groups_per_workgroup(dtype):
     _check_culled(mix, xes, gout, dtype, "tight", tag="wide, several groups")
 
 
+def test_mixture_beyond_the_reference_node_index_range():
+    """The reference stores node indices in 16 bits (lbvh/bvh.h:16-24: at most 32768 components per mixture); here
+    they are 32-bit.  One mixture of 70000 components: every component is exactly one leaf, every parent box is the
+    union of its children's (vectorised over the nodes), and the culled sums equal the masked sums."""
+    M, N, D = 70000, 1500, 3
+    mix, xes, gout = _case(1, 1, M, N, D, seed=4242, spread=6.0, cov_radius=0.05)
+    bvh, lo, up = _device_boxes(mix, xes, torch.float64, "tight")
+    nodes, nb = bvh.nodes()
+    torch.cuda.synchronize()
+    nd, bx = nodes.cpu().numpy()[0, 0], nb.cpu().numpy()[0, 0]
+    assert nd.shape == (2 * M - 1, 4)
+    assert np.array_equal(np.sort(nd[M - 1:, 3]), np.arange(M)), "every component is exactly one leaf"
+    left, right = nd[:M - 1, 1], nd[:M - 1, 2]
+    assert left.min() > 0 and right.min() > 0 and max(left.max(), right.max()) < 2 * M - 1
+    assert np.array_equal(nd[left, 0], np.arange(M - 1)) and np.array_equal(nd[right, 0], np.arange(M - 1))
+    assert np.array_equal(np.sort(np.concatenate([left, right])), np.arange(1, 2 * M - 1)), "one parent per node"
+    assert np.array_equal(bx[:M - 1, :D], np.minimum(bx[left, :D], bx[right, :D])), "parent box = union (lower)"
+    assert np.array_equal(bx[:M - 1, D:], np.maximum(bx[left, D:], bx[right, D:])), "parent box = union (upper)"
+    assert bvh.candidate_stats().cpu().numpy()[2] == 0
+    for dtype in (torch.float64, torch.float32):
+        _check_culled(mix, xes, gout, dtype, "tight", tag=f"M{M}")
+
+
 def test_culled_random_shapes():
     """differential run of the culled path over random shapes (one to four point groups per workgroup, ragged and
     empty trailing groups, broadcast points, identical Gaussians, narrow and wide boxes) against the masked sum"""
