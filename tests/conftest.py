@@ -22,7 +22,10 @@ def rel_l2(a, b, floor: float = 0.0) -> float:
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)
     nb = max(np.linalg.norm(b), floor * math.sqrt(max(b.size, 1)))
-    na = np.linalg.norm(a - b)
+    d = a - b
+    if floor > 0.0:
+        d = np.where(np.abs(d) < floor, 0.0, d)        # differences below the floor are underflow, not error
+    na = np.linalg.norm(d)
     if nb == 0.0:
         return 0.0 if na == 0.0 else float("inf")
     return float(na / nb)

@@ -5,31 +5,36 @@ every element: |got - ref| <= budget.  The budget of an element is a first-order
 through the pairs (Gaussian m, point n) that enter it.  With u the upper Cholesky factor of A = 1/2 log2(e) sym(C),
 y = u (x - b), q = |y|^2 and the pair value f = w norm exp2(-q):
 
-  dy    absolute error of y.  Shifted form (y = u x - u b without forming x - b, taken when bound_m = max_i sum_j
-        |u_ij b_j| is at most `limit`): CY eps bound_m, whatever the distance of the point.  Explicit x - b:
-        CC eps ya with ya_i = sum_j |u_ij| |t_j| >= |y_i| (products of mixed sign cancel for rotated, anisotropic
-        Gaussians).  `direct_form` (t^T C t straight from the stored matrix, as the culled path's leaves and the
+  dy    absolute error of y.  Shifted form (y_i = sum_j u_ij x_j - (u b)_i without forming x - b, taken when bound_m =
+        max_i sum_j |u_ij b_j| is at most `limit`): the D roundings of the chain act on partial sums of at most
+        sum_j |u_ij| (|b_j| + |t_j|) + |(u b)_i| <= 2 bound_m + ya_i, hence CY eps bound_m + CS eps ya with ya_i =
+        sum_j |u_ij| |t_j| >= |y_i| (products of mixed sign cancel for rotated, anisotropic Gaussians).  Explicit
+        x - b: CC eps ya.  `direct_form` (t^T C t straight from the stored matrix, as the culled path's leaves and the
         reference do): the same with sum_ij |C_ij| |t_i| |t_j| in place of ya^2.
   rel   relative error of f:  C0 eps (amplitude, exponential, accumulation over the other index) + CQ eps q (rounding
         of q = |y|^2 itself) + 2 ln2 |y| dy;  direct form: C0 eps + CD eps sum_ij |C_ij t_i t_j| / 2 (every product of
-        the quadratic form is rounded, and they cancel).
+        the quadratic form is rounded, and they cancel).  Both plus CO eps64 sum_ij |C_ij t_i t_j| / 2 for the oracle,
+        which evaluates the direct form in float64: for an ill-conditioned Gaussian (condition number 300, the sum
+        300 times t^T C t) that is 1e-12 of a term and what a float64 result differs by from the oracle.
   out, dL/dw                  sum of |f| rel                    (resp. |f / w| |g| rel)
   dL/dx, dL/db = -+ f g C t   sum of |f g| (rel |C t| + |u| dy / (1/2 log2 e)),   |C t| <= sqrt(2 v lambda_max(C))
   dL/dC = -1/2 f g t t^T + cofactor term
                               sum of |f g| (rel |t|^2 + 2 |t| dy / sigma_min(u)) / 2 + |cof| |w kappa g e| rel / (2 sqrt det)
 The gradient budgets are norm-wise per Gaussian (one value for all components of a position or a matrix).  Measured on
-the device over the whole test suite, the worst element uses 0.76 of its budget in float32 (0.34 for the matrix-core
-forward kernel at the edge of its shifted-form limit) and, with ORACLE_SHARE, 0.7 in float64; a wrong element (a
+the device over the whole test suite, the worst element uses 0.38 of its budget in float32 (0.24 for the matrix-core
+forward kernel at the edge of its shifted-form limit) and, with ORACLE_SHARE, 0.60 in float64; over 1100 further
+random shapes (dense and culled, both precisions, a hundred million elements) 0.32 and 0.70.  A wrong element (a
 dropped pair, a swapped index, a mis-rounded split) exceeds the budget by orders of magnitude.  float64 results are
 compared with a float64 oracle (numpy: other formulas, another summation order) whose own rounding is of the size of
-the error under test, hence the factor ORACLE_SHARE on the float64 budgets."""
+the error under test, hence the CO term and the factor ORACLE_SHARE on the float64 budgets."""
 import numpy as np
 
 import gm_oracle as o
 
 EPS = {np.dtype(np.float32): 2.0 ** -24, np.dtype(np.float64): 2.0 ** -53}
 HALF_LOG2E = 0.72134752044448170368
-C0, CQ, CY, CC, CD = 48.0, 3.0, 6.0, 8.0, 24.0
+C0, CQ, CY, CS, CC, CD, CO = 48.0, 3.0, 6.0, 3.0, 8.0, 24.0, 8.0
+EPS64 = 2.0 ** -53
 ORACLE_SHARE = {np.dtype(np.float32): 1.0, np.dtype(np.float64): 8.0}
 
 
@@ -70,7 +75,7 @@ def _masked_direct_budgets(mixture, xes, g, eps, mask):
             ynorm = np.sqrt(HALF_LOG2E * 2.0 * v)
             ya = np.sqrt(HALF_LOG2E * np.einsum('pi,pij,pj->p', np.abs(t), np.abs(c), np.abs(t)))
             dy = eps * CC * ya
-            rel = eps * C0 + CD * eps * ya * ya / (2.0 * HALF_LOG2E)
+            rel = eps * C0 + (CD * eps + CO * EPS64) * ya * ya / (2.0 * HALF_LOG2E)
             f = np.abs(w_all[b, l] * norm_all[b, l])[mi] * e
             gg = g[b, l][ni]
             out[b, l] = np.bincount(ni, f * rel, N)
@@ -126,11 +131,14 @@ def budgets(mixture, xes, grad_output, dtype, limit, chunk=32, mask=None, direct
             ya = np.sqrt(HALF_LOG2E * np.einsum('blmni,blmij,blmnj->blmn', np.abs(t), np.abs(c), np.abs(t)))
         else:
             ya = np.sqrt((np.einsum('blmij,blmnj->blmni', np.abs(u_all[sl]), np.abs(t)) ** 2).sum(-1))
-        dy = eps * np.where(shifted[sl][..., None], CY * bound[sl][..., None], CC * ya)
+        dy = eps * np.where(shifted[sl][..., None], CY * bound[sl][..., None] + CS * ya, CC * ya)
         if direct_form:
-            rel = eps * C0 + CD * eps * ya * ya / (2.0 * HALF_LOG2E)
+            direct = ya * ya / (2.0 * HALF_LOG2E)
+            rel = eps * C0 + CD * eps * direct
         else:
+            direct = 0.5 * np.einsum('blmni,blmij,blmnj->blmn', np.abs(t), np.abs(c), np.abs(t))
             rel = eps * (C0 + CQ * ynorm * ynorm) + 2.0 * np.log(2.0) * ynorm * dy
+        rel = rel + CO * EPS64 * direct
         f = np.abs(w * norm)[..., None] * e
         gg = g[:, :, None, :]
         out += (f * rel).sum(2)
