@@ -529,7 +529,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
         "config": {"workload": f"{args.workload}: D={D} {dt} B={wl.B} L={wl.L} M={wl.M} N={wl.N}, dense all-pairs, "
                                f"{wl.pairs:.4g} pairs per step, forward + backward (grad mixture and grad xes)"},
-        "timing": "ms_per_step: wall clock over all steps / steps; fwd.ms, roofline launch_ms: medians of per-step HIP event pairs",
+        "timing": "ms_per_step: wall clock over all steps / steps; fwd.ms, roofline launch_ms: medians of per-step HIP event pairs (launch_ms_mean: their means)",
         "fwd": {"ms": fwd_ms, "pairs_per_s": wl.pairs / (fwd_ms * 1e-3), "tflops": fwd_tf, "frac_of_peak": fwd_tf / peak,
                 "tflops_by_reference_literal_count": FLOP_FWD_LITERAL[D] * wl.pairs / (fwd_ms * 1e-3) / 1e12},
         "fwd_bwd": {"ms": ms_step, "pairs_per_s": wl.pairs / (ms_step * 1e-3), "tflops": step_tf,
@@ -538,11 +538,12 @@ def main():
                                "the time, are inside the event pair)",
                      "bound": "valu", "bound_detail": VALU_NOTE, "achieved": bwd_tf, "peak": peak, "unit": "TFLOP/s", "frac": bwd_tf / peak,
                      "traffic": profile_traffic(args.workload, "eval_bwd_rc_kernel"), "launch_ms": bwd_ms,
-                     "flop_per_pair": FLOP_BWD[D], **at_measured_clock(bwd_tf / peak, bwd_mhz)},
+                     "launch_ms_mean": r["bwd_ms_mean"], "flop_per_pair": FLOP_BWD[D], **at_measured_clock(bwd_tf / peak, bwd_mhz)},
         "roofline_fwd": {"kernel": fwd_kernel, "bound": "mfma" if fwd_kernel == "eval_fwd_mfma_kernel" else "valu",
                          "bound_detail": MFMA_NOTE if fwd_kernel == "eval_fwd_mfma_kernel" else VALU_NOTE,
                          "achieved": fwd_tf, "peak": peak,
-                         "unit": "TFLOP/s", "frac": fwd_tf / peak, "launch_ms": fwd_ms, "flop_per_pair": FLOP_FWD[D],
+                         "unit": "TFLOP/s", "frac": fwd_tf / peak, "launch_ms": fwd_ms, "launch_ms_mean": r["fwd_ms_mean"],
+                         "flop_per_pair": FLOP_FWD[D],
                          "traffic": profile_traffic(args.workload, fwd_kernel),
                          **(at_measured_clock(fwd_tf / peak, fwd_mhz) if fwd_kernel == "eval_fwd_mfma_kernel" else {})},
     }
@@ -629,6 +630,8 @@ def measure_dense(name: str, steps: int, warmup: int, copy_calibration: bool = F
     return {"wl": wl, "ms_step": wall * 1e3 / steps, "clocks_mhz": clocks,
             "fwd_ms": median([e[0].elapsed_time(e[1]) for e in events]),
             "bwd_ms": median([e[1].elapsed_time(e[2]) for e in events]),
+            "fwd_ms_mean": sum(e[0].elapsed_time(e[1]) for e in events) / steps,
+            "bwd_ms_mean": sum(e[1].elapsed_time(e[2]) for e in events) / steps,
             "fwd_kernel": _native.lib().gmc_eval_fwd_kernel_name(ctypes.byref(shape)).decode()}
 
 
