@@ -422,6 +422,54 @@ def test_points_changed_in_place_or_replaced_at_the_same_address(dtype):
     assert n(bvh.candidate_stats())[2] == 0
 
 
+def test_random_call_sequences_on_one_object():
+    """Stateful differential run: BVH objects go through random sequences of forward and backward calls (all need
+    flags) with in-place changes of the points, other point tensors and rebuilds in between; every result must be the
+    masked sum over the object's boxes for the points and the mixture of that call, and no error flag may rise."""
+    rng = np.random.default_rng(8128)
+    n = lambda t: t.cpu().numpy()
+    for obj in range(14):
+        dtype = torch.float32 if obj % 2 else torch.float64
+        tol, fl = TOL[dtype], FLOOR[dtype]
+        if obj % 3 == 0:
+            mix, xes, gout = _crowded_case(int(rng.integers(1, 3)), int(rng.integers(0, 10000)), bool(rng.random() < 0.3))
+        else:
+            B, L, M, N, D = (int(rng.integers(1, 4)), int(rng.integers(1, 3)), int(rng.integers(2, 800)),
+                             int(rng.integers(1, 9000)), int(rng.integers(2, 4)))
+            mix, xes, gout = _case(B, L, M, N, D, int(rng.integers(0, 100000)), broadcast=bool(rng.random() < 0.3),
+                                   spread=float(rng.choice([1.0, 4.0])), cov_radius=float(rng.choice([0.02, 0.3, 3.0])))
+        mode = "tight" if rng.random() < 0.6 else "reference"
+        m, x, g = (t.to(dtype).to(DEV).contiguous() for t in (mix, xes, gout))
+        bvh = _native.Bvh(m, x, 0.001, mode)
+        lo, up = (n(t).astype(np.float64) for t in bvh.boxes())
+        m_np, g_np = n(m), n(g)
+        for step in range(int(rng.integers(4, 9))):
+            op = str(rng.choice(["fwd", "bwd", "bwd_m", "bwd_x", "inplace", "other", "rebuild", "fwd"]))
+            tag = f"object {obj} ({tuple(m.shape)}, {tuple(x.shape)}, {dtype}, {mode}) step {step} {op}"
+            if op == "inplace":
+                k = int(rng.integers(1, 4))
+                x[:, :, ::k] = x[:, :, ::k] * float(rng.choice([-0.7, 1.3, 0.5])) + float(rng.choice([0.0, 0.25]))
+            elif op == "other":
+                gen = torch.Generator().manual_seed(int(rng.integers(0, 1 << 30)))
+                x = (torch.rand(x.shape, dtype=torch.float64, generator=gen) * 2 - 1).mul(float(rng.choice([0.3, 3.0, 6.0]))).to(dtype).to(DEV)
+            elif op == "rebuild":
+                if rng.random() < 0.5:
+                    bvh.rebuild(m, x)
+                else:
+                    bvh = _native.Bvh(m, x, 0.001, mode)
+                lo, up = (n(t).astype(np.float64) for t in bvh.boxes())
+            else:
+                ref, rgm, rgx = _masked_reference(g_np, m_np, n(x), lo, up)
+                if op == "fwd":
+                    assert rel_l2(n(_native.eval_bvh_fwd(m, x, bvh)), ref, fl) <= tol, tag
+                else:
+                    need_m, need_x = op != "bwd_x", op != "bwd_m"
+                    gm_, gx_ = _native.eval_bvh_bwd(g, m, x, bvh, need_m, need_x)
+                    assert not need_m or rel_l2(n(gm_), rgm, fl) <= tol, tag
+                    assert not need_x or rel_l2(n(gx_), rgx, fl) <= tol, tag
+                assert n(bvh.candidate_stats())[2] == 0, tag
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("D", [2, 3])
 def test_leaf_order_is_bit_exact(dtype, D):

@@ -90,6 +90,33 @@ def _check(mix, xes, gout, dtype, tag=""):
     _check_elements(gxes, rgx, bud["gx"], dtype, "grad xes", tag)
 
 
+def test_dense_random_shapes():
+    """differential run of the dense path over random shapes (both precisions and dimensions, broadcast points, one to
+    several tiles of Gaussians, ragged point chunks, scaled point clouds) against the oracle, every element included"""
+    rng = np.random.default_rng(4711)
+    for case in range(36):
+        D = int(rng.integers(2, 4))
+        dtype = torch.float32 if rng.random() < 0.6 else torch.float64
+        kind = int(rng.integers(0, 5))
+        if kind == 0:
+            B, L, M, N = int(rng.integers(1, 30)), int(rng.integers(1, 6)), int(rng.integers(1, 300)), int(rng.integers(1, 1200))
+        elif kind == 1:
+            B, L, M, N = 1, 1, int(rng.integers(200, 2500)), int(rng.integers(500, 6000))
+        elif kind == 2:
+            B, L, M, N = int(rng.integers(1, 4)), int(rng.integers(1, 4)), int(rng.integers(129, 700)), int(rng.integers(1, 3000))
+        elif kind == 3:
+            B, L, M, N = int(rng.integers(30, 200)), 1, int(rng.integers(1, 40)), int(rng.integers(1, 200))
+        else:
+            B, L, M, N = int(rng.integers(1, 6)), int(rng.integers(1, 6)), int(rng.integers(1, 140)), int(rng.integers(1, 2500))
+        while B * L * M * N > 3e6:
+            N = max(1, N // 2)
+        bc = bool(rng.random() < 0.25)
+        mix, xes, gout = _case(B, L, M, N, D, 52000 + case, bc)
+        if rng.random() < 0.3:
+            xes = xes * float(rng.choice([0.1, 3.0]))
+        _check(mix, xes, gout, dtype, tag=f"case {case}: B{B} L{L} M{M} N{N} D{D} broadcast {bc} {dtype}")
+
+
 def test_known_answer(golden_dir):
     data = json.load(open(os.path.join(golden_dir, "support_collections.json")))["known_answer"]
     for dtype, tol in ((torch.float32, 1e-7), (torch.float64, 1e-15)):
