@@ -849,23 +849,27 @@ __device__ __forceinline__ bool inside_box(const T (&x)[D], const T* box) {
     return in;
 }
 
-__device__ __forceinline__ float exp_neg_half(float q) { return __builtin_amdgcn_exp2f(q * -0.72134752044448170368f); }
-__device__ __forceinline__ double exp_neg_half(double q) { return exp(-0.5 * q); }
+// exp(-q / 2); `tab` is the workgroup's exp2 table (float: none)
+template <typename T>
+__device__ __forceinline__ T exp_neg_half(T q, const T* __restrict__ tab) {
+    return pair_exp2(q * T(-0.72134752044448170368), tab);
+}
 
 // e = exp(-1/2 t^T C t), u = C t for the leaf record r
 template <typename T, int D>
-__device__ __forceinline__ T leaf_terms(const T* __restrict__ r, const T (&x)[D], T (&t)[D], T (&u)[D]) {
+__device__ __forceinline__ T leaf_terms(const T* __restrict__ r, const T* __restrict__ tab, const T (&x)[D], T (&t)[D],
+                                        T (&u)[D]) {
     if constexpr (D == 2) {
         t[0] = x[0] - r[0]; t[1] = x[1] - r[1];
         u[0] = fma_(r[2], t[0], r[3] * t[1]);
         u[1] = fma_(r[3], t[0], r[4] * t[1]);
-        return exp_neg_half(fma_(t[0], u[0], t[1] * u[1]));
+        return exp_neg_half(fma_(t[0], u[0], t[1] * u[1]), tab);
     } else {
         t[0] = x[0] - r[0]; t[1] = x[1] - r[1]; t[2] = x[2] - r[2];
         u[0] = fma_(r[3], t[0], fma_(r[4], t[1], r[5] * t[2]));
         u[1] = fma_(r[4], t[0], fma_(r[6], t[1], r[7] * t[2]));
         u[2] = fma_(r[5], t[0], fma_(r[7], t[1], r[8] * t[2]));
-        return exp_neg_half(fma_(t[0], u[0], fma_(t[1], u[1], t[2] * u[2])));
+        return exp_neg_half(fma_(t[0], u[0], fma_(t[1], u[1], t[2] * u[2])), tab);
     }
 }
 
@@ -970,6 +974,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     __shared__ double rsum_mem[kTravWaves][NEED_GM ? kStageBatch * NR : 1];
     __shared__ int2 pend[kGroupsMax][kPendMax];             // pieces of a group's list that wait to be published
     __shared__ int piece_valid;                             // helper workgroups: the piece still describes the group's points
+    const T* exp2_tab = exp2_table<T>();                    // (published by the barrier in front of the first evaluation)
     const int per_mixture = (N + kWave - 1) / kWave;        // point groups of one mixture
     // The last `helpers` workgroups of a backward launch each take one published piece of a long candidate list
     // (no descent: one group, its points, a slice of its list); all others own `groups_per_workgroup` groups.
@@ -1189,7 +1194,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
 #pragma unroll
                     for (int k = 0; k < kAmp - 2 * D + 1; ++k) r[k] = lf[k];
                     T t[D], u[D];
-                    const T e = leaf_terms<T, D>(r, x, t, u);
+                    const T e = leaf_terms<T, D>(r, exp2_tab, x, t, u);
                     if (NEED_GX) {
                         const T s = has ? r[kAmp - 2 * D] * e : T(0);
 #pragma unroll
@@ -1226,7 +1231,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
 #pragma unroll
                 for (int k = 0; k < kAmp - 2 * D + 1; ++k) r[k] = lf[k];
                 T t[D], u[D];
-                const T e = leaf_terms<T, D>(r, x, t, u);
+                const T e = leaf_terms<T, D>(r, exp2_tab, x, t, u);
                 const T amp = r[kAmp - 2 * D];
                 if (MODE == 0) {
                     acc += has ? amp * e : T(0);

@@ -36,7 +36,8 @@ bool dense_forward_f32(const float* mixture, const float* xes, float* out, const
 constexpr int kTile = 256;   // Gaussians staged per LDS tile (one per lane)
 
 template <typename T, int D, int P, bool CENTRED>
-__device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, int begin, int end, const T (&x)[P][D], T (&acc)[P]) {
+__device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, const T* __restrict__ tab, int begin, int end,
+                                          const T (&x)[P][D], T (&acc)[P]) {
     constexpr int S = Rec<T, D>::kStride;
 #pragma unroll 2
     for (int g = begin; g < end; ++g) {
@@ -47,7 +48,7 @@ __device__ __forceinline__ void fwd_pairs(const T* __restrict__ lds, int begin, 
         for (int p = 0; p < P; ++p) {
             T y[D];
             const T q = quad_form<T, D, CENTRED>(r, x[p], y);
-            acc[p] = fma_(r[Rec<T, D>::kAmp], fast_exp2(-q), acc[p]);
+            acc[p] = fma_(r[Rec<T, D>::kAmp], pair_exp2(-q, tab), acc[p]);
         }
     }
 }
@@ -61,6 +62,7 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
     constexpr int S = Rec<T, D>::kStride;
     __shared__ __attribute__((aligned(16))) T lds[kTile * S];
     __shared__ int counts[10];
+    const T* exp2_tab = exp2_table<T>();            // (published by the barriers of stage_tile)
 
     int bl, chunk;
     map_workgroup(blockIdx.x, chunks * ts.slices, n_mixtures, bl, chunk);
@@ -90,8 +92,8 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
         const int cnt = (g_end - g0) < kTile ? (g_end - g0) : kTile;
         stage_tile<T, D>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts, covariance_form);
         const int n_shifted = counts[8];
-        fwd_pairs<T, D, P, false>(lds, 0, n_shifted, x, acc);
-        fwd_pairs<T, D, P, true>(lds, n_shifted, cnt, x, acc);
+        fwd_pairs<T, D, P, false>(lds, exp2_tab, 0, n_shifted, x, acc);
+        fwd_pairs<T, D, P, true>(lds, exp2_tab, n_shifted, cnt, x, acc);
     }
 #pragma unroll
     for (int p = 0; p < P; ++p) {
@@ -107,8 +109,8 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_kernel(const T* __restrict__ 
 // covers 64 P points for any P from 2 to 16, where the kernel above covers 256 P with P a power of two.  Used when
 // that pads the last chunk less (784 points: 832 instead of 1024).
 template <typename T, int D, int P, bool CENTRED>
-__device__ __forceinline__ void fwd_rc_pairs(const T* __restrict__ lds, int begin, int end, int row, const T (&x)[P][D],
-                                             T (&acc)[P]) {
+__device__ __forceinline__ void fwd_rc_pairs(const T* __restrict__ lds, const T* __restrict__ tab, int begin, int end,
+                                             int row, const T (&x)[P][D], T (&acc)[P]) {
     constexpr int S = Rec<T, D>::kStride;
 #pragma unroll 2
     for (int g = begin + row; g < end; g += 4) {
@@ -119,7 +121,7 @@ __device__ __forceinline__ void fwd_rc_pairs(const T* __restrict__ lds, int begi
         for (int p = 0; p < P; ++p) {
             T y[D];
             const T q = quad_form<T, D, CENTRED>(r, x[p], y);
-            acc[p] = fma_(r[Rec<T, D>::kAmp], fast_exp2(-q), acc[p]);
+            acc[p] = fma_(r[Rec<T, D>::kAmp], pair_exp2(-q, tab), acc[p]);
         }
     }
 }
@@ -133,6 +135,7 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_rc_kernel(const T* __restrict
     constexpr int S = Rec<T, D>::kStride;
     __shared__ __attribute__((aligned(16))) T lds[(kTile + 6) * S];
     __shared__ int counts[10];
+    const T* exp2_tab = exp2_table<T>();            // (published by the barriers of staging)
 
     int bl, chunk;
     map_workgroup(blockIdx.x, chunks * ts.slices, n_mixtures, bl, chunk);
@@ -163,8 +166,8 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_rc_kernel(const T* __restrict
         const int cnt = (g_end - g0) < kTile ? (g_end - g0) : kTile;
         stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts, covariance_form);
         const int centred_start = counts[8], padded_total = counts[9];
-        fwd_rc_pairs<T, D, P, false>(lds, 0, centred_start, row, x, acc);
-        fwd_rc_pairs<T, D, P, true>(lds, centred_start, padded_total, row, x, acc);
+        fwd_rc_pairs<T, D, P, false>(lds, exp2_tab, 0, centred_start, row, x, acc);
+        fwd_rc_pairs<T, D, P, true>(lds, exp2_tab, centred_start, padded_total, row, x, acc);
     }
 #pragma unroll
     for (int p = 0; p < P; ++p) {
@@ -186,8 +189,9 @@ __global__ __launch_bounds__(kBlock) void eval_fwd_rc_kernel(const T* __restrict
 template <typename T> struct SumCopies { static constexpr int k = sizeof(T) == 4 ? 4 : 1; };
 
 template <typename T, int D, int P, bool NEED_GM, bool NEED_GX, bool CENTRED>
-__device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __restrict__ block_sums, int begin, int end,
-                                             int row, const T (&x)[P][D], const T (&go)[P], T (&gx)[P][D]) {
+__device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, const T* __restrict__ tab,
+                                             T* __restrict__ block_sums, int begin, int end, int row, const T (&x)[P][D],
+                                             const T (&go)[P], T (&gx)[P][D]) {
     constexpr int S = Rec<T, D>::kStride;
     constexpr int NR = Sums<D>::k;
     for (int g = begin + row; g < end; g += 4) {
@@ -212,7 +216,7 @@ __device__ __forceinline__ void bwd_rc_pairs(const T* __restrict__ lds, T* __res
         for (int p = 0; p < P; ++p) {
             T y[D];
             const T q = quad_form<T, D, CENTRED>(r, x[p], y);
-            const T e = fast_exp2(-q);
+            const T e = pair_exp2(-q, tab);
             const T k = NEED_GM ? e * go[p] : e;
             T ky[D];
 #pragma unroll
@@ -314,6 +318,7 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
     // three float workgroups share a compute unit's LDS; measured: three of 53.6 KB are resident together, three of
     // 54.0 KB are not
     static_assert(sizeof(T) == 8 || sizeof(lds) + sizeof(block_sums) + 64 <= 53760, "LDS of the backward pair kernel");
+    const T* exp2_tab = exp2_table<T>();            // (published by the barriers of staging)
 
     const ClockProbe probe = clock_probe_begin();
     int bl, chunk;
@@ -358,8 +363,8 @@ void eval_bwd_rc_kernel(const T* __restrict__ grad_out, const T* __restrict__ mi
         stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0 / kHalfLog2e, lds, counts, covariance_form);
         const int centred_start = counts[8], padded_total = counts[9];
         T* wave_sums = block_sums + (NEED_GM && SumCopies<T>::k > 1 ? wave * kTile * NR : 0);
-        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, false>(lds, wave_sums, 0, centred_start, row, x, go, gx);
-        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, true>(lds, wave_sums, centred_start, padded_total, row, x, go, gx);
+        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, false>(lds, exp2_tab, wave_sums, 0, centred_start, row, x, go, gx);
+        bwd_rc_pairs<T, D, P, NEED_GM, NEED_GX, true>(lds, exp2_tab, wave_sums, centred_start, padded_total, row, x, go, gx);
         if (NEED_GM) {
             __syncthreads();
             T* __restrict__ dst = sums + (size_t(bl) * M + g0) * NR;
