@@ -18,7 +18,6 @@ template <> struct Kappa<3> { static constexpr double v = 0.06349363593424097; }
 constexpr double kHalfLog2e = 0.72134752044448170368;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ double fast_exp2(double x) { return exp2(x); }
 
 // exp2 of a non-positive argument for the pair loops.  float: the hardware instruction.  double: 2^x = 2^e 2^(j/256) 2^r
 // with x = e + j/256 + r, |r| <= 1/512: the integer 256 e + j comes out of the low mantissa bits of x * 256 + 1.5 * 2^52

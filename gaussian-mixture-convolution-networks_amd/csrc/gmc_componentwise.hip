@@ -16,6 +16,8 @@ __global__ __launch_bounds__(kBlock) void componentwise_fwd_kernel(const T* __re
                                                                   T* __restrict__ out, int L, int M, int N, int Bx, int Lx,
                                                                   int m_tiles, int chunks, bool covariance_form) {
     constexpr int G = 1 + D + D * D;
+    const T* exp2_tab = exp2_table<T>();
+    if constexpr (sizeof(T) == 8) __syncthreads();          // the table is complete (all wavefronts are still here)
     int id = blockIdx.x;
     const int chunk = id % chunks; id /= chunks;
     const int tile = id % m_tiles;
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(kBlock) void componentwise_fwd_kernel(const T* __re
         for (int d = 0; d < D; ++d) x[d] = x_bl[size_t(n) * D + d];
         T y[D];
         const T q = quad_form<T, D, true>(r, x, y);
-        if (valid) out[(size_t(bl) * N + n) * M + m] = r[Rec<T, D>::kAmp] * fast_exp2(-q);
+        if (valid) out[(size_t(bl) * N + n) * M + m] = r[Rec<T, D>::kAmp] * pair_exp2(-q, exp2_tab);
     }
 }
 
@@ -75,6 +77,8 @@ __global__ __launch_bounds__(kBlock) void componentwise_bwd_kernel(const T* __re
     constexpr int kU = Rec<T, D>::kU;
     __shared__ T point_grad[NEED_GX ? kCwPointsMax * D : 1];
     __shared__ T shared_sums[NEED_GM ? kBlock * NR : 1];
+    const T* exp2_tab = exp2_table<T>();
+    if constexpr (sizeof(T) == 8) __syncthreads();          // the table is complete
     int id = blockIdx.x;
     const int chunk = id % chunks; id /= chunks;
     const int group = id % m_groups;
@@ -131,7 +135,7 @@ __global__ __launch_bounds__(kBlock) void componentwise_bwd_kernel(const T* __re
             for (int u = 0; u < kCwUnroll; ++u) {
                 T y[D];
                 const T q = quad_form<T, D, true>(r, xs[u], y);
-                const T k = (valid && n0 + u < n_end) ? fast_exp2(-q) * go[u] : T(0);
+                const T k = (valid && n0 + u < n_end) ? pair_exp2(-q, exp2_tab) * go[u] : T(0);
                 T ky[D];
 #pragma unroll
                 for (int d = 0; d < D; ++d) ky[d] = k * y[d];

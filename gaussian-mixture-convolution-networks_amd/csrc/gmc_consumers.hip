@@ -28,8 +28,8 @@ template <typename T> struct EpiArgs {
 };
 
 template <typename T, int D, int P, bool CENTRED>
-__device__ __forceinline__ void rc_pairs(const T* __restrict__ lds, int begin, int end, int row, const T (&x)[P][D],
-                                         T (&acc)[P]) {
+__device__ __forceinline__ void rc_pairs(const T* __restrict__ lds, const T* __restrict__ tab, int begin, int end, int row,
+                                         const T (&x)[P][D], T (&acc)[P]) {
     constexpr int S = Rec<T, D>::kStride;
 #pragma unroll 2
     for (int g = begin + row; g < end; g += 4) {
@@ -40,7 +40,7 @@ __device__ __forceinline__ void rc_pairs(const T* __restrict__ lds, int begin, i
         for (int p = 0; p < P; ++p) {
             T y[D];
             const T q = quad_form<T, D, CENTRED>(r, x[p], y);
-            acc[p] = fma_(r[Rec<T, D>::kAmp], fast_exp2(-q), acc[p]);
+            acc[p] = fma_(r[Rec<T, D>::kAmp], pair_exp2(-q, tab), acc[p]);
         }
     }
 }
@@ -57,6 +57,7 @@ __global__ __launch_bounds__(kBlock) void consumer_fwd_kernel(const T* __restric
     __shared__ __attribute__((aligned(16))) T lds[(kTileC + 6) * S];
     __shared__ int counts[10];
     __shared__ double wave_moments[4][2];
+    const T* exp2_tab = exp2_table<T>();            // (published by the barriers of staging)
 
     int bl, chunk;
     map_workgroup(blockIdx.x, chunks, n_mixtures, bl, chunk);
@@ -82,8 +83,8 @@ __global__ __launch_bounds__(kBlock) void consumer_fwd_kernel(const T* __restric
         const T* over = KIND == kEpiRatio ? epi.weights + size_t(bl) * M + g0 : nullptr;
         stage_tile<T, D, 4>(mix_bl + size_t(g0) * G, cnt, 1.0, lds, counts, true, over);
         const int centred_start = counts[8], padded_total = counts[9];
-        rc_pairs<T, D, P, false>(lds, 0, centred_start, row, x, acc);
-        rc_pairs<T, D, P, true>(lds, centred_start, padded_total, row, x, acc);
+        rc_pairs<T, D, P, false>(lds, exp2_tab, 0, centred_start, row, x, acc);
+        rc_pairs<T, D, P, true>(lds, exp2_tab, centred_start, padded_total, row, x, acc);
     }
     double s1 = 0.0, s2 = 0.0;
 #pragma unroll
