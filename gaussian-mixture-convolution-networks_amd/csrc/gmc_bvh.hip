@@ -715,14 +715,14 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
     load_inverse_covariance<T, D>(g + 1 + D, covariance_form, cm);
     for (int d = 0; d < D; ++d) r[d] = g[1 + d];
     if constexpr (D == 2) {
-        const double det = cm[0][0] * cm[1][1] - cm[0][1] * cm[1][0];
+        const double det = determinant<T, 2>(cm);
         r[2] = T(cm[0][0]); r[3] = T(0.5 * (cm[0][1] + cm[1][0])); r[4] = T(cm[1][1]);
         r[5] = T(double(g[0]) * Kappa<2>::v * sqrt(det));
         reinterpret_cast<int*>(r + 6)[0] = comp;
     } else {
         const double c00 = cm[0][0], c01 = cm[0][1], c02 = cm[0][2], c10 = cm[1][0], c11 = cm[1][1], c12 = cm[1][2],
                      c20 = cm[2][0], c21 = cm[2][1], c22 = cm[2][2];
-        const double det = c00 * (c11 * c22 - c12 * c21) - c01 * (c10 * c22 - c12 * c20) + c02 * (c10 * c21 - c11 * c20);
+        const double det = determinant<T, 3>(cm);
         r[3] = T(c00); r[4] = T(0.5 * (c01 + c10)); r[5] = T(0.5 * (c02 + c20));
         r[6] = T(c11); r[7] = T(0.5 * (c12 + c21)); r[8] = T(c22);
         r[9] = T(double(g[0]) * Kappa<3>::v * sqrt(det));
@@ -1490,10 +1490,7 @@ __global__ __launch_bounds__(kBlock) void bvh_bwd_epilogue_kernel(const T* __res
     const double w = double(g[0]);
     double c[D][D];
     load_inverse_covariance<T, D>(g + 1 + D, covariance_form, c);
-    double det;
-    if constexpr (D == 2) det = c[0][0] * c[1][1] - c[0][1] * c[1][0];
-    else det = c[0][0] * (c[1][1] * c[2][2] - c[1][2] * c[2][1]) - c[0][1] * (c[1][0] * c[2][2] - c[1][2] * c[2][0]) +
-               c[0][2] * (c[1][0] * c[2][1] - c[1][1] * c[2][0]);
+    const double det = determinant<T, D>(c);
     const double root = sqrt(det);
     const double norm = Kappa<D>::v * root;
     const double R0 = double(rs[0]);

@@ -102,6 +102,55 @@ __device__ __forceinline__ void load_inverse_covariance(const T* __restrict__ c,
     }
 }
 
+// Determinant of the D x D matrix of a Gaussian.  For float32 inputs the plain expansion in double is exact enough
+// (its rounding error, up to a few thousand 2^-53 for condition numbers of several hundred, is far below 2^-24).  For
+// float64 inputs the signed products of the expansion are formed and added as unevaluated pairs hi + lo (error-free
+// product by FMA, error-free sum), so the result is the correctly rounded determinant of the stored entries also where
+// the products cancel: once per Gaussian and workgroup, about a hundred instructions.
+struct TwoDoubles { double hi, lo; };
+__device__ __forceinline__ TwoDoubles exact_product(double a, double b) {
+#pragma clang fp contract(off)
+    const double p = a * b;
+    return {p, __builtin_fma(a, b, -p)};
+}
+__device__ __forceinline__ TwoDoubles renormalised(double hi, double lo) {        // |hi| >= |lo|
+#pragma clang fp contract(off)
+    const double s = hi + lo;
+    return {s, lo - (s - hi)};
+}
+__device__ __forceinline__ TwoDoubles times(TwoDoubles x, double c) {
+#pragma clang fp contract(off)
+    const double p = x.hi * c;
+    const double e = __builtin_fma(x.lo, c, __builtin_fma(x.hi, c, -p));
+    return renormalised(p, e);
+}
+__device__ __forceinline__ TwoDoubles plus(TwoDoubles x, TwoDoubles y) {
+#pragma clang fp contract(off)
+    const double s = x.hi + y.hi;
+    const double v = s - x.hi;
+    const double e = ((x.hi - (s - v)) + (y.hi - v)) + (x.lo + y.lo);
+    return renormalised(s, e);
+}
+template <typename T, int D>
+__device__ __forceinline__ double determinant(const double (&m)[D][D]) {
+    if constexpr (sizeof(T) == 4) {
+        if constexpr (D == 2) return m[0][0] * m[1][1] - m[0][1] * m[1][0];
+        else return m[0][0] * (m[1][1] * m[2][2] - m[1][2] * m[2][1]) - m[0][1] * (m[1][0] * m[2][2] - m[1][2] * m[2][0]) +
+                    m[0][2] * (m[1][0] * m[2][1] - m[1][1] * m[2][0]);
+    } else if constexpr (D == 2) {
+        const TwoDoubles d = plus(exact_product(m[0][0], m[1][1]), exact_product(-m[0][1], m[1][0]));
+        return d.hi + d.lo;
+    } else {
+        TwoDoubles d = times(exact_product(m[0][0], m[1][1]), m[2][2]);
+        d = plus(d, times(exact_product(-m[0][0], m[1][2]), m[2][1]));
+        d = plus(d, times(exact_product(-m[0][1], m[1][0]), m[2][2]));
+        d = plus(d, times(exact_product(m[0][1], m[1][2]), m[2][0]));
+        d = plus(d, times(exact_product(m[0][2], m[1][0]), m[2][1]));
+        d = plus(d, times(exact_product(-m[0][2], m[1][1]), m[2][0]));
+        return d.hi + d.lo;
+    }
+}
+
 template <typename T, int D>
 __device__ __forceinline__ Derived<D> derive(const T* __restrict__ g, bool covariance_form = false) {
     Derived<D> r;
@@ -110,7 +159,7 @@ __device__ __forceinline__ Derived<D> derive(const T* __restrict__ g, bool covar
     load_inverse_covariance<T, D>(g + 1 + D, covariance_form, cm);
     if constexpr (D == 2) {
         const double c00 = cm[0][0], c01 = cm[0][1], c10 = cm[1][0], c11 = cm[1][1];
-        const double det = c00 * c11 - c01 * c10;
+        const double det = determinant<T, 2>(cm);
         const double a00 = kHalfLog2e * c00, a01 = kHalfLog2e * 0.5 * (c01 + c10), a11 = kHalfLog2e * c11;
         const double u00 = sqrt(a00);
         const double u01 = a01 / u00;
@@ -125,7 +174,7 @@ __device__ __forceinline__ Derived<D> derive(const T* __restrict__ g, bool covar
     } else {
         const double c00 = cm[0][0], c01 = cm[0][1], c02 = cm[0][2], c10 = cm[1][0], c11 = cm[1][1], c12 = cm[1][2],
                      c20 = cm[2][0], c21 = cm[2][1], c22 = cm[2][2];
-        const double det = c00 * (c11 * c22 - c12 * c21) - c01 * (c10 * c22 - c12 * c20) + c02 * (c10 * c21 - c11 * c20);
+        const double det = determinant<T, 3>(cm);
         const double a00 = kHalfLog2e * c00, a11 = kHalfLog2e * c11, a22 = kHalfLog2e * c22;
         const double a01 = kHalfLog2e * 0.5 * (c01 + c10), a02 = kHalfLog2e * 0.5 * (c02 + c20),
                      a12 = kHalfLog2e * 0.5 * (c12 + c21);

@@ -494,10 +494,7 @@ __device__ __forceinline__ void bwd_epilogue_one(const T* __restrict__ g, const 
             for (int t = 0; t < D; ++t) acc += m[r][t] * V[q][t];
             a[r][q] = acc;
         }
-    double det;
-    if constexpr (D == 2) det = c[0][0] * c[1][1] - c[0][1] * c[1][0];
-    else det = c[0][0] * (c[1][1] * c[2][2] - c[1][2] * c[2][1]) - c[0][1] * (c[1][0] * c[2][2] - c[1][2] * c[2][0]) +
-               c[0][2] * (c[1][0] * c[2][1] - c[1][1] * c[2][0]);
+    const double det = determinant<T, D>(c);
     const double kd = dv.w * Kappa<D>::v * R0 / (2.0 * sqrt(det));
     double gc[D][D];
 #pragma unroll

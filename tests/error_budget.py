@@ -22,8 +22,11 @@ y = u (x - b), q = |y|^2 and the pair value f = w norm exp2(-q):
                               sum of |f g| (rel |t|^2 + 2 |t| dy / sigma_min(u)) / 2 + |cof| |w kappa g e| rel / (2 sqrt det)
 The gradient budgets are norm-wise per Gaussian (one value for all components of a position or a matrix).  Measured on
 the device over the whole test suite, the worst element uses 0.38 of its budget in float32 (0.24 for the matrix-core
-forward kernel at the edge of its shifted-form limit) and, with ORACLE_SHARE, 0.60 in float64; over 1100 further
-random shapes (dense and culled, both precisions, a hundred million elements) 0.32 and 0.70.  A wrong element (a
+forward kernel at the edge of its shifted-form limit) and, with ORACLE_SHARE, 0.08 (dense) / 0.63 (culled, large cases
+against the C restatement) in float64; over 860 further random shapes (dense and culled, both precisions) 0.29 and
+0.11 / 0.48.  (Before the device took the determinant of a float64 Gaussian in compensated arithmetic these float64
+figures were 0.60 and 0.95: the plain cofactor expansion, which the reference and the C restatement use, is off by up
+to 2400 eps for condition numbers of a few hundred, numpy's by 110.)  A wrong element (a
 dropped pair, a swapped index, a mis-rounded split) exceeds the budget by orders of magnitude.  float64 results are
 compared with a float64 oracle (numpy: other formulas, another summation order) whose own rounding is of the size of
 the error under test, hence the CO term and the factor ORACLE_SHARE on the float64 budgets."""
