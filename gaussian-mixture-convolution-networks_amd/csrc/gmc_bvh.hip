@@ -923,11 +923,74 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Largest float not above / smallest float not below a coordinate: boxes rounded outwards stay conservative.
+__device__ __forceinline__ float float_below(float x) { return x; }
+__device__ __forceinline__ float float_above(float x) { return x; }
+__device__ __forceinline__ float float_below(double x) {
+    const float f = float(x);
+    const int b = __builtin_bit_cast(int, f);               // the next float towards -inf: one step in the bit pattern
+    const float down = __builtin_bit_cast(float, f > 0.0f ? b - 1 : (f < 0.0f ? b + 1 : int(0x80000001u)));
+    return double(f) > x ? down : f;
+}
+__device__ __forceinline__ float float_above(double x) {
+    const float f = float(x);
+    const int b = __builtin_bit_cast(int, f);
+    const float up = __builtin_bit_cast(float, f > 0.0f ? b + 1 : (f < 0.0f ? b - 1 : 1));
+    return double(f) < x ? up : f;
+}
+
+// Boxes of a group's 64 points for the descent (lanes = points in Morton order; every lane gets all values, lane 0
+// stores them: out = lower[D], upper[D] of the first box, then of the second).  Neighbours on the Morton curve are
+// neighbours in space except where the curve jumps, and a group that straddles a jump has a bounding box that spans a
+// large part of the scene: ten times the candidates of its neighbours for the same number of hits, and the launch
+// ends with such groups.  The points are therefore cut where two consecutive ones lie farthest apart (L1), and the two
+// runs get a box each when that at least halves the volume (extents padded by 1/32 of the whole extent, so flat
+// boxes compare sensibly); otherwise both boxes are the bounding box of all points.
+template <typename T, int D>
+__device__ __forceinline__ void group_boxes(const T (&x)[D], bool valid, int lane, float* __restrict__ out) {
+    float lo[D], hi[D], gap = 0.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        lo[d] = valid ? float_below(x[d]) : INFINITY;
+        hi[d] = valid ? float_above(x[d]) : -INFINITY;
+        const float mid = float(x[d]);
+        gap += fabsf(__shfl_down(mid, 1, 64) - mid);
+    }
+    const bool next_valid = __shfl_down(valid ? 1 : 0, 1, 64) != 0 && lane < 63;
+    // the jump after lane i competes with its lane index in the low bits (gap >= 0: its bit pattern is ordered)
+    unsigned key = (valid && next_valid && gap == gap) ? ((__builtin_bit_cast(unsigned, gap) & ~63u) | unsigned(lane)) : 0u;
+    key = wave_max(key);
+    const int cut = int(key & 63u);                         // the first run ends with this lane
+    const bool first = lane <= cut;
+    float alo[D], ahi[D], blo[D], bhi[D];
+    float one = 1.0f, two_a = 1.0f, two_b = 1.0f;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        alo[d] = wave_min(first ? lo[d] : INFINITY);  ahi[d] = wave_max(first ? hi[d] : -INFINITY);
+        blo[d] = wave_min(first ? INFINITY : lo[d]);  bhi[d] = wave_max(first ? -INFINITY : hi[d]);
+        const float whole = fmaxf(ahi[d], bhi[d]) - fminf(alo[d], blo[d]);
+        const float pad = fmaxf(whole * (1.0f / 32.0f), 1e-30f);
+        one *= whole + pad;
+        two_a *= fmaxf(ahi[d] - alo[d], 0.0f) + pad;
+        two_b *= fmaxf(bhi[d] - blo[d], 0.0f) + pad;
+    }
+    // (an empty second run counts with its padding only, so the sum is not below the whole and the cut is not taken)
+    const bool split = two_a + two_b < 0.5f * one;
+    if (lane == 0) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const float wlo = fminf(alo[d], blo[d]), whi = fmaxf(ahi[d], bhi[d]);
+            out[d] = split ? alo[d] : wlo;              out[D + d] = split ? ahi[d] : whi;
+            out[2 * D + d] = split ? blo[d] : wlo;      out[3 * D + d] = split ? bhi[d] : whi;
+        }
+    }
+}
+
 // Traversal of one tree by a workgroup of 8 wavefronts for up to kGroupsMax groups of 64 Morton-neighbouring
 // points, in two alternating phases.
 //   Phase 1 (wavefront i descends for group i, lanes = tree nodes): one stack of internal nodes per group in LDS;
 //   up to 64 of them are popped at a time, each lane fetches the two child boxes of its node and tests them against
-//   the bounding box of the group's points (a node that contains any of the points overlaps that box).
+//   the one or two boxes around the group's points (group_boxes; a node that contains any of the points overlaps one).
 //   Overlapping internal children go back on the stack, overlapping leaves into the group's candidate list (ballot
 //   + prefix-popcount compaction).  The descents of the groups are independent chains of memory round trips (about
 //   one per tree level) and run side by side.
@@ -962,7 +1025,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     __shared__ int state[kGroupsMax][2];                    // [0] candidates gathered, [1] nodes left on the stack
     __shared__ int pids[kGroupsMax][kWave];                 // index of every point, -1 beyond the end
     __shared__ T pts[kGroupsMax][D + 1][kWave];             // coordinates and upstream gradient of every point
-    __shared__ T gbox[kGroupsMax][2 * D];                   // bounding box of every group's points
+    __shared__ float gbox[kGroupsMax][4 * D];               // two boxes (lower, upper; rounded outwards) around every group's points
     // results per point, in double: the forward sums are added wavefront by wavefront (deterministic), dL/dx with
     // LDS atomics (cheap for doubles on distinct words, unlike floats)
     __shared__ double result[kGroupsMax][kVals][kWave];
@@ -1047,11 +1110,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
         T g = T(0);
         if (MODE == 1) g = valid ? grad_out[size_t(bl) * N + pid] : T(0);
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            pts[wave][d][lane] = x[d];
-            const T lo = wave_min(valid ? x[d] : T(INFINITY)), hi = wave_max(valid ? x[d] : T(-INFINITY));
-            if (lane == 0) { gbox[wave][d] = lo; gbox[wave][D + d] = hi; }
-        }
+        for (int d = 0; d < D; ++d) pts[wave][d][lane] = x[d];
         pts[wave][D][lane] = g;
         pids[wave][lane] = valid ? pid : -1;
         if (cache.count) my_stamp = points_stamp<T, D>(x, valid, lane);
@@ -1107,6 +1166,8 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
                 cache_slot = -1;
             }
         }
+        // only a wavefront that descends needs the boxes around its points (a known list or a piece does without)
+        if (sp > 0) group_boxes<T, D>(x, valid, lane, gbox[wave]);
     }
     for (int i = threadIdx.x; i < kGroupsMax * kVals * kWave; i += kTravBlock) (&result[0][0][0])[i] = 0.0;
 
@@ -1289,9 +1350,11 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             int n_leaf = 0;
             int* stk = stack[wave];
             int* cand = leaves[wave];
-            T glo[D], ghi[D];
+            T glo[2][D], ghi[2][D];
 #pragma unroll
-            for (int d = 0; d < D; ++d) { glo[d] = gbox[wave][d]; ghi[d] = gbox[wave][D + d]; }
+            for (int k = 0; k < 2; ++k)
+#pragma unroll
+                for (int d = 0; d < D; ++d) { glo[k][d] = T(gbox[wave][k * 2 * D + d]); ghi[k][d] = T(gbox[wave][k * 2 * D + D + d]); }
             // room in the pool for the list of a later round is asked for before the descent, so that the atomic's
             // round trip is over when the list is there (a whole list's worth; what is not used stays unused)
             int pool_at = 0;
@@ -1312,10 +1375,13 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
 #pragma unroll
                 for (int side = 0; side < 2; ++side) {
                     const int c = side == 0 ? ch.x : ch.y;
-                    bool ov = active & (c < M - 1) & (~c < M);          // a node of this tree
+                    bool meets[2] = {true, true};                       // the child's box overlaps the group's first / second box
 #pragma unroll
-                    for (int d = 0; d < D; ++d)
-                        ov = ov & (cb[side * 2 * D + d] <= ghi[d]) & (cb[side * 2 * D + D + d] >= glo[d]);
+                    for (int k = 0; k < 2; ++k)
+#pragma unroll
+                        for (int d = 0; d < D; ++d)
+                            meets[k] = meets[k] & (cb[side * 2 * D + d] <= ghi[k][d]) & (cb[side * 2 * D + D + d] >= glo[k][d]);
+                    const bool ov = active & (c < M - 1) & (~c < M) & (meets[0] | meets[1]);    // ... and is a node of this tree
                     push[side] = ov & (c >= 0);
                     hit[side] = ov & (c < 0);
                 }
@@ -1678,13 +1744,18 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
-// 64-point groups per traversal workgroup.  More groups per workgroup overlap more descents and pay off when the
-// launch has many times more groups than resident workgroups; with few groups, smaller workgroups balance better
-// over the compute units (measured: 1563 groups run fastest with 2 per workgroup, 4096 and more with 4).
-static int traversal_groups(size_t BL, int N) {
+// 64-point groups per traversal workgroup.  A forward pass on a new tree descends: more groups per workgroup overlap
+// more descents (each a chain of memory round trips that leaves the vector units idle), and the launch should fit
+// the resident workgroups in one go (measured on one mixture of 16384 Gaussians, groups -> best choice and time:
+// 391 -> 1, 43 us; 782 -> 2, 39 us; 1563 -> 4, 46 us against 63 us with 2; 3125 ... 25000 -> 4).  A backward pass
+// reads the candidate lists: small workgroups balance better over the compute units until the launch has many times
+// more groups than resident workgroups (1563 -> 1, 77 us against 85 us with 4; 3125 -> 2; 6250 -> 3; 25000 -> 4).
+static int traversal_groups(size_t BL, int N, bool backward) {
     const size_t per_mixture = (size_t(N) + kWave - 1) / kWave;
-    const size_t total = BL * per_mixture;
-    size_t g = total <= size_t(kTravSlots) ? 1 : total < 4 * size_t(kTravSlots) ? 2 : total < 8 * size_t(kTravSlots) ? 3 : kGroupsMax;
+    const size_t total = BL * per_mixture, slots = size_t(kTravSlots);
+    size_t g;
+    if (backward) g = total < 4 * slots ? 1 : total < 8 * slots ? 2 : total < 16 * slots ? 3 : kGroupsMax;
+    else g = total <= slots ? 1 : total <= 2 * slots ? 2 : kGroupsMax;
     if (g > per_mixture) g = per_mixture;
     return g < 1 ? 1 : int(g);
 }
@@ -1699,7 +1770,7 @@ static int bvh_fwd_t(const T* xes, char* bvh, T* out, const gmc_shape& s, hipStr
         fill_zero_kernel<T><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(out, n);
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    const int groups = traversal_groups(BL, s.N);
+    const int groups = traversal_groups(BL, s.N, false);
     const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kTravBlock), 0, st>>>(
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children),
@@ -1727,7 +1798,7 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bv
     }
     sums = (T*)(bvh + lay.sums);                   // inside the object and all zero here; the caller's workspace is not used
     if (gx && xes_shared) zero(grad_xes, n_x);
-    const int groups = traversal_groups(BL, s.N);
+    const int groups = traversal_groups(BL, s.N, true);
     const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     // one helper workgroup per piece that a forward pass may have published, behind the owners
     const int helpers = lay.pieces_max;
