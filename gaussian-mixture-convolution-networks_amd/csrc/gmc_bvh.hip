@@ -487,16 +487,13 @@ struct SortJob {
     int* err;                            // error flags of the BVH object
 };
 
-// One pass of the sort for two jobs in one launch (job b behind job a).  The block histograms of a pass are counted
-// by the kernel that writes the pass's input (the Morton kernel, or the pass before) with one atomic per key, which
-// saves a histogram launch per pass: the passes are short kernels, bound by launch latency.
-__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJob b) {
+// One pass of the sort by workgroup `id` of job j (all kBlock lanes of the workgroup call it).  The block histograms of
+// a pass are counted by the kernel that writes the pass's input (the Morton kernel, or the pass before) with one
+// atomic per key, which saves a histogram launch per pass: the passes are short kernels, bound by launch latency.
+__device__ __forceinline__ void radix_scatter_pass(const SortJob& j, unsigned id) {
     __shared__ uint32_t running[256];        // next output slot of every digit for this block
     __shared__ uint32_t wave_count[4][256];
     __shared__ uint32_t wave_total[4];
-    const bool first = blockIdx.x < a.blocks;
-    const SortJob& j = first ? a : b;
-    const unsigned id = first ? blockIdx.x : blockIdx.x - a.blocks;
     const int blocks_per_seg = j.blocks_per_seg, count = j.count, shift = j.shift;
     const int seg = id / blocks_per_seg, blk = id - seg * blocks_per_seg;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -592,6 +589,12 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJo
     }
 }
 
+// A pass for two jobs in one launch (job b behind job a).
+__global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJob b) {
+    if (blockIdx.x < a.blocks) radix_scatter_pass(a, blockIdx.x);
+    else radix_scatter_pass(b, blockIdx.x - a.blocks);
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // leaves, radix tree, bottom-up boxes
 // ---------------------------------------------------------------------------------------------------------------
@@ -661,14 +664,18 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
                                                            T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
                                                            int2* __restrict__ children, int* __restrict__ parent,
                                                            int2* __restrict__ node_range, int M, size_t total,
-                                                           bool covariance_form, T* __restrict__ sums) {
+                                                           bool covariance_form, T* __restrict__ sums,
+                                                           unsigned own_blocks, SortJob rider) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
     constexpr int NS = 1 + D + D * (D + 1) / 2;
+    // The sort of the query points does not depend on the trees: a pass of it rides behind this kernel's own
+    // workgroups, on compute units that would idle otherwise, instead of lengthening a pass of the leaves' sort.
+    if (blockIdx.x >= own_blocks) { radix_scatter_pass(rider, blockIdx.x - own_blocks); return; }
     // The records of the leaves and the internal nodes of the tree do not depend on each other, and both are
     // short chains of dependent memory reads: the first half of the grid writes the records, the second half
     // builds the nodes, side by side on different compute units.
-    const unsigned half = gridDim.x / 2;
+    const unsigned half = own_blocks / 2;
     const bool tree_job = blockIdx.x >= half;
     const size_t i = size_t(tree_job ? blockIdx.x - half : blockIdx.x) * kBlock + threadIdx.x;
     if (i >= total) return;
@@ -747,10 +754,12 @@ constexpr int kMergeBlock = 256;
 template <typename T, int D>
 __global__ __launch_bounds__(kMergeBlock) void bvh_merge_kernel(const int* __restrict__ parent, const int2* __restrict__ node_range,
                                                           const T* __restrict__ node_box, long long* enc_box, int M,
-                                                          size_t total) {
+                                                          size_t total, unsigned own_blocks, SortJob rider) {
     __shared__ long long local_box[kMergeBlock][2 * D];
     __shared__ int local_parent[kMergeBlock];
     __shared__ int is_local[kMergeBlock];
+    static_assert(kMergeBlock == kBlock, "the riding sort pass works with kBlock lanes");
+    if (blockIdx.x >= own_blocks) { radix_scatter_pass(rider, blockIdx.x - own_blocks); return; }   // (see bvh_leaves_kernel)
     const size_t first_leaf = size_t(blockIdx.x) * kMergeBlock;          // leaves of all mixtures, numbered through
     const size_t t = first_leaf + threadIdx.x;
     const size_t bl = t < total ? t / M : 0;
@@ -1720,24 +1729,39 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     // points neighbours, the top 8 bits for segments of at most kCoarseOrderMax points (32 points per cell; measured:
     // same traversal times, one sort pass less).  The sorted keys of the points are not needed afterwards: they
     // land in a spare buffer, which must not be the input of the last pass.
+    // The launches of the leaves' four passes are bound by their latency and would take twice as long with the six
+    // times more numerous points in them; the points' passes ride in the two longest launches of the tree
+    // construction instead (leaf records + radix tree, box merge), which use a quarter of the compute units.
+    const SortJob none = {};
+    SortJob jp_first = none, jp_second = none;
     for (int pass = 0; pass < 4; ++pass) {
         SortJob jg, jp;
         jobs_of_pass(pass, jg, jp);
-        if (jg.blocks + jp.blocks == 0) continue;
-        radix_scatter_kernel<<<dim3(jg.blocks + jp.blocks), dim3(kBlock), 0, st>>>(jg, jp);
+        if (pass == 0) jp_first = jp;
+        if (pass == 1) jp_second = jp;
+        if (jg.blocks == 0) continue;
+        radix_scatter_kernel<<<dim3(jg.blocks), dim3(kBlock), 0, st>>>(jg, none);
+    }
+    if (!have_g) {                                   // no trees to build: the points' passes are launches of their own
+        if (jp_first.blocks > 0) radix_scatter_kernel<<<dim3(jp_first.blocks), dim3(kBlock), 0, st>>>(jp_first, none);
+        if (jp_second.blocks > 0) radix_scatter_kernel<<<dim3(jp_second.blocks), dim3(kBlock), 0, st>>>(jp_second, none);
     }
     if (have_g) {
         const size_t n = BL * M;
-        bvh_leaves_kernel<T, D><<<dim3(2 * grid_for(n)), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi,
+        const unsigned leaf_blocks = 2 * grid_for(n);
+        bvh_leaves_kernel<T, D><<<dim3(leaf_blocks + jp_first.blocks), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi,
                                                                                   double(cfg.aabb_threshold), cfg.aabb_mode, g_order, g_keys,
                                                                            node_box, leaf_rec, enc_box, children, parent, node_range, M, n,
-                                                                           cfg.covariance_form != 0, (T*)(bvh + lay.sums));
+                                                                           cfg.covariance_form != 0, (T*)(bvh + lay.sums), leaf_blocks, jp_first);
         if (M > 1) {
             const size_t ni = BL * (M - 1);
-            bvh_merge_kernel<T, D><<<dim3(unsigned((n + kMergeBlock - 1) / kMergeBlock)), dim3(kMergeBlock), 0, st>>>(
-                parent, node_range, node_box, enc_box, M, n);
+            const unsigned merge_blocks = unsigned((n + kMergeBlock - 1) / kMergeBlock);
+            bvh_merge_kernel<T, D><<<dim3(merge_blocks + jp_second.blocks), dim3(kMergeBlock), 0, st>>>(
+                parent, node_range, node_box, enc_box, M, n, merge_blocks, jp_second);
             bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(
                 children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups);
+        } else if (jp_second.blocks > 0) {           // single leaves have no boxes to merge
+            radix_scatter_kernel<<<dim3(jp_second.blocks), dim3(kBlock), 0, st>>>(jp_second, none);
         }
     }
     if (have_p && !sort_p) iota_segments_kernel<<<dim3(grid_for(XL * N)), dim3(kBlock), 0, st>>>(p_order, N, XL * N);
@@ -1771,7 +1795,13 @@ static int bvh_fwd_t(const T* xes, char* bvh, T* out, const gmc_shape& s, hipStr
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
     const int groups = traversal_groups(BL, s.N, false);
-    const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
+    int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
+    // A launch that would leave resident slots empty is spread over all of them: workgroups whose last wavefront
+    // finds no group left serve one group fewer (1563 groups: 512 workgroups of 3 or 4 instead of 391 of 4, 50.6 -> 46.5 us).
+    if (groups > 1 && BL * size_t(chunks) < size_t(kTravSlots)) {
+        const size_t per_mixture = (size_t(s.N) + kWave - 1) / kWave, fill = size_t(kTravSlots) / BL;
+        chunks = int(fill < per_mixture ? fill : per_mixture);
+    }
     bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kTravBlock), 0, st>>>(
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children),
         (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, candidate_cache(bvh, lay), nullptr, 0,
