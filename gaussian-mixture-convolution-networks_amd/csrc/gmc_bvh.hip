@@ -887,6 +887,7 @@ template <int D> struct BvhSums { static constexpr int k = 1 + D + D * (D + 1) /
 constexpr int kStackCap = 512;          // soft capacity of a node stack (the array has 128 more)
 constexpr int kTravWaves = 8;           // wavefronts per workgroup of the traversal
 constexpr int kTravBlock = kTravWaves * kWave;
+constexpr int kTwoBoxLeaves = 256;      // trees with fewer leaves get one box per point group (see group_boxes)
 constexpr int kGroupsMax = 4;           // 64-point groups per workgroup (each descends the tree with its own wavefront)
 constexpr int kStageBatch = 20;         // candidate leaves a wavefront stages in LDS at a time
 constexpr int kTravSlots = 2 * 256;     // workgroups resident at once: two per compute unit
@@ -954,14 +955,27 @@ __device__ __forceinline__ float float_above(double x) {
 // large part of the scene: ten times the candidates of its neighbours for the same number of hits, and the launch
 // ends with such groups.  The points are therefore cut where two consecutive ones lie farthest apart (L1), and the two
 // runs get a box each when that at least halves the volume (extents padded by 1/32 of the whole extent, so flat
-// boxes compare sensibly); otherwise both boxes are the bounding box of all points.
+// boxes compare sensibly); otherwise both boxes are the bounding box of all points.  `may_cut` is false for small trees:
+// a list cannot be longer than the tree has leaves, and the cut costs a workgroup of a launch with thousands of small
+// trees more than the shorter lists save (measured with 64 and 128 leaves per tree: 8-10 % of the forward pass).
 template <typename T, int D>
-__device__ __forceinline__ void group_boxes(const T (&x)[D], bool valid, int lane, float* __restrict__ out) {
+__device__ __forceinline__ void group_boxes(const T (&x)[D], bool valid, int lane, bool may_cut, float* __restrict__ out) {
     float lo[D], hi[D], gap = 0.0f;
 #pragma unroll
     for (int d = 0; d < D; ++d) {
         lo[d] = valid ? float_below(x[d]) : INFINITY;
         hi[d] = valid ? float_above(x[d]) : -INFINITY;
+    }
+    if (!may_cut) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const float wlo = wave_min(lo[d]), whi = wave_max(hi[d]);
+            if (lane == 0) { out[d] = wlo; out[D + d] = whi; out[2 * D + d] = wlo; out[3 * D + d] = whi; }
+        }
+        return;
+    }
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
         const float mid = float(x[d]);
         gap += fabsf(__shfl_down(mid, 1, 64) - mid);
     }
@@ -1176,7 +1190,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             }
         }
         // only a wavefront that descends needs the boxes around its points (a known list or a piece does without)
-        if (sp > 0) group_boxes<T, D>(x, valid, lane, gbox[wave]);
+        if (sp > 0) group_boxes<T, D>(x, valid, lane, M >= kTwoBoxLeaves, gbox[wave]);
     }
     for (int i = threadIdx.x; i < kGroupsMax * kVals * kWave; i += kTravBlock) (&result[0][0][0])[i] = 0.0;
 
@@ -1384,12 +1398,15 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
 #pragma unroll
                 for (int side = 0; side < 2; ++side) {
                     const int c = side == 0 ? ch.x : ch.y;
-                    bool meets[2] = {true, true};                       // the child's box overlaps the group's first / second box
+                    bool meets[2] = {true, M >= kTwoBoxLeaves};         // the child's box overlaps the group's first / second box
 #pragma unroll
-                    for (int k = 0; k < 2; ++k)
+                    for (int d = 0; d < D; ++d)
+                        meets[0] = meets[0] & (cb[side * 2 * D + d] <= ghi[0][d]) & (cb[side * 2 * D + D + d] >= glo[0][d]);
+                    if (M >= kTwoBoxLeaves) {                           // (small trees have one box: the same for all wavefronts)
 #pragma unroll
                         for (int d = 0; d < D; ++d)
-                            meets[k] = meets[k] & (cb[side * 2 * D + d] <= ghi[k][d]) & (cb[side * 2 * D + D + d] >= glo[k][d]);
+                            meets[1] = meets[1] & (cb[side * 2 * D + d] <= ghi[1][d]) & (cb[side * 2 * D + D + d] >= glo[1][d]);
+                    }
                     const bool ov = active & (c < M - 1) & (~c < M) & (meets[0] | meets[1]);    // ... and is a node of this tree
                     push[side] = ov & (c >= 0);
                     hit[side] = ov & (c < 0);
