@@ -103,9 +103,9 @@ def cpu_baseline(name: str):
 
 def measure_bvh(aabb_mode: str, steps: int, warmup: int, copy_calibration: bool = False):
     """LBVH-culled path on C5 (3-D, float64, one mixture of 16384 Gaussians, 100000 points).  A step builds the
-    tree (the mixture changes every training step), evaluates forward and backward.  Returns the timings (HIP events
-    on the launch stream, medians over the steps; the step time is the wall clock over all steps) and the number of
-    pairs actually evaluated."""
+    tree (the mixture changes every training step), evaluates forward and backward.  Returns the step time (wall
+    clock over all steps), the timings of its parts (HIP events on the launch stream, medians over a second run of the
+    same steps) and the number of pairs actually evaluated."""
     import torch
     from gmc import _native, synthetic
     wl, mix, xes, gout = synthetic.make_workload("C5")
@@ -136,12 +136,18 @@ def measure_bvh(aabb_mode: str, steps: int, warmup: int, copy_calibration: bool 
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
+    # the step time: wall clock over `steps` steps with nothing else in the stream (a step is 0.2 ms in 13 launches,
+    # and four event records per step would add several microseconds of their own to it) ...
     t0 = time.perf_counter()
+    for k in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    # ... and its parts: the same steps again with HIP events between the calls
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(steps)]
     for k in range(steps):
         step(events[k])
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     build_ms, fwd_ms, bwd_ms = (median([e[i].elapsed_time(e[i + 1]) for e in events]) for i in range(3))
     # pairs actually evaluated: points inside the cutoff box of a Gaussian (counted outside the timed region)
     bvh = _native.Bvh(mix, xes, 0.001, aabb_mode)

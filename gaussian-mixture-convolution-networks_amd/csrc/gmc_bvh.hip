@@ -104,7 +104,9 @@ struct CandidateCache {
 constexpr int kErrStack = 1;            // a traversal's node stack was full and a push was dropped (results incomplete)
 constexpr int kErrSort = 2;             // a radix pass computed an output slot outside its segment
 constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
-constexpr int kSortBlocksMax = 256;                 // radix blocks per segment (more items per lane beyond that)
+constexpr int kSortBlocksMax = 128;                 // radix blocks per segment (more items per lane beyond that: every block sums
+                                                    // the counts of all blocks of its segment; 100000 keys in 98 instead of 196
+                                                    // blocks: the build 81 -> 77.5 us)
 constexpr int kCoarseOrderMax = 8192;               // point segments up to this size are ordered by 8 Morton bits only
 constexpr int kBoundsChunk = kBlock * 2;            // points per workgroup of the partial bounds of the query points
 
