@@ -348,6 +348,33 @@ def test_long_candidate_lists_are_shared_between_workgroups(broadcast):
     _check_culled(mix, xes, gout, torch.float32, "tight", tag=f"crowded, broadcast {broadcast}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
+def test_point_group_across_a_jump_of_the_morton_curve(dtype, D):
+    """64 points in two far-apart clusters form ONE group (consecutive on the Morton curve across a jump).  One box
+    around all of them spans the scene and every leaf of the tree becomes a candidate: a list of several rounds, cut
+    into pieces.  The descent tests against one box per cluster instead, so the group's list stays short (one round,
+    nothing in the pool of later rounds), and the sums are those of the brute-force masked evaluation either way.  A tree of fewer than 256
+    leaves keeps the single box: same sums."""
+    n = lambda t: t.cpu().numpy()
+    for M, expect_short in ((2048, True), (200, False)):
+        mix, _, gout = _case(1, 2, M, 64, D, seed=900 + M + D, spread=1.0, cov_radius=0.02)
+        g = torch.Generator().manual_seed(77 + D)
+        corner = torch.ones(D, dtype=torch.float64) * 0.8
+        xes = torch.cat([-corner + 0.05 * torch.rand((1, 2, 29, D), generator=g, dtype=torch.float64),
+                         corner - 0.05 * torch.rand((1, 2, 35, D), generator=g, dtype=torch.float64)], dim=2).contiguous()
+        m, x = mix.to(dtype).to(DEV).contiguous(), xes.to(dtype).to(DEV).contiguous()
+        bvh = _native.Bvh(m, x, 0.001, "tight")
+        _native.eval_bvh_fwd(m, x, bvh)
+        torch.cuda.synchronize()
+        stats = n(bvh.candidate_stats()).tolist()
+        assert stats[2] == 0
+        if expect_short:
+            # (one box around both clusters makes all 2048 leaves candidates: four rounds of 512, the later ones in the pool)
+            assert stats[1] == 0 and stats[0] <= 4, f"the lists of two small clusters fit one round, got {stats}"
+        _check_culled(mix, xes, gout, dtype, "tight", tag=f"two clusters, M {M}")
+
+
 def test_traversal_with_other_points_than_the_build():
     """Every candidate list kept in the BVH object carries a stamp of the 64 points it was gathered for.  A traversal
     that is given other points (another tensor) must not use the lists and pieces of the build's points: it gives
