@@ -988,19 +988,19 @@ __device__ __forceinline__ void group_boxes(const T (&x)[D], bool valid, int lan
     const int cut = int(key & 63u);                         // the first run ends with this lane
     const bool first = lane <= cut;
     float alo[D], ahi[D], blo[D], bhi[D];
-    float one = 1.0f, two_a = 1.0f, two_b = 1.0f;
+    float part_a = 1.0f, part_b = 1.0f;                     // volumes of the two boxes as fractions of the whole (any scale)
 #pragma unroll
     for (int d = 0; d < D; ++d) {
         alo[d] = wave_min(first ? lo[d] : INFINITY);  ahi[d] = wave_max(first ? hi[d] : -INFINITY);
         blo[d] = wave_min(first ? INFINITY : lo[d]);  bhi[d] = wave_max(first ? -INFINITY : hi[d]);
         const float whole = fmaxf(ahi[d], bhi[d]) - fminf(alo[d], blo[d]);
         const float pad = fmaxf(whole * (1.0f / 32.0f), 1e-30f);
-        one *= whole + pad;
-        two_a *= fmaxf(ahi[d] - alo[d], 0.0f) + pad;
-        two_b *= fmaxf(bhi[d] - blo[d], 0.0f) + pad;
+        const float inv = 1.0f / (whole + pad);
+        part_a *= (fmaxf(ahi[d] - alo[d], 0.0f) + pad) * inv;
+        part_b *= (fmaxf(bhi[d] - blo[d], 0.0f) + pad) * inv;
     }
-    // (an empty second run counts with its padding only, so the sum is not below the whole and the cut is not taken)
-    const bool split = two_a + two_b < 0.5f * one;
+    // (an empty second run leaves the first one as large as the whole: no cut; NaN or infinite coordinates: no cut)
+    const bool split = part_a + part_b < 0.5f;
     if (lane == 0) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
