@@ -49,6 +49,7 @@ struct BvhLayout {
     size_t hist_words;          // uint32 words from hist_g to the end of hist_p
     size_t p_order;             // int [BxLx][N]           Morton order of the query points
     size_t g_keys;              // uint32 [BL][M]          sorted Morton codes of the leaves
+    size_t frontier;            // int [BL][1 + kFrontier] count, then internal nodes that cut the tree a few levels below the root
     size_t cand_count;          // int [BL][ceil(N/64)]    candidate leaves of every point group, -1: not known
     size_t cand_list;           // int [BL][ceil(N/64)][kLeafCap], then a pool of pool_cap ints for the lists of
                                 // later rounds (all empty when the lists would exceed kCandCacheBytes)
@@ -101,6 +102,7 @@ struct CandidateCache {
     int2* piece_range;
     int pieces_max, pool_cap, pool_base;
 };
+constexpr int kFrontier = 64;           // internal nodes a descent starts from (see tree_frontier)
 constexpr int kErrStack = 1;            // a traversal's node stack was full and a push was dropped (results incomplete)
 constexpr int kErrSort = 2;             // a radix pass computed an output slot outside its segment
 constexpr int kSortItems = 2;                       // items per lane and radix block: small chunks, many workgroups
@@ -160,6 +162,7 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.hist_words = (o - l.hist_g) / 4;
     l.p_order = take(XL * N * 4);
     l.g_keys = take(BL * M * 4);
+    l.frontier = take(BL * (1 + kFrontier) * 4);
     {
         const size_t point_groups = BL * ((N + kWave - 1) / kWave);
         l.point_groups = point_groups;
@@ -739,6 +742,33 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
     }
 }
 
+// Where a descent starts.  The first levels below the root hold one, two, four ... nodes, and a descent spends a memory
+// round trip on each of them with most lanes idle; every descent of the tree goes through them.  One wavefront walks
+// the tree breadth-first as long as a level consists of internal nodes only and the next has at most kFrontier entries,
+// and leaves that level's nodes in the object: the descents push all of them at once (their children are tested in
+// the first step; a subtree that is entered without need costs one step of one lane).  out[0] = count, then the nodes.
+__device__ __forceinline__ void tree_frontier(const int2* __restrict__ kids, int M, int* __restrict__ out, int lane) {
+    __shared__ int level[4][kFrontier];                     // one wavefront of the workgroup per mixture
+    int* cur = level[threadIdx.x >> 6];
+    int n = 1;
+    if (lane == 0) cur[0] = 0;
+    for (int depth = 0; depth < 16; ++depth) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (2 * n > kFrontier) break;
+        const int node = lane < n ? cur[lane] : 0;
+        const int2 ch = lane < n ? kids[node] : make_int2(0, 0);
+        const bool leaf_below = lane < n && (ch.x < 0 || ch.y < 0);
+        if (__ballot(leaf_below) != 0ull) break;            // the next level would not be internal nodes only
+        __builtin_amdgcn_wave_barrier();                    // every lane has read its node before the level is overwritten
+        if (lane < n) { cur[2 * lane] = ch.x; cur[2 * lane + 1] = ch.y; }
+        n *= 2;
+    }
+    if (lane == 0) out[0] = n;
+    if (lane < n) out[1 + lane] = cur[lane];
+}
+
 // Bottom-up boxes without inter-lane ordering: one lane per leaf walks towards the root and merges ITS OWN leaf
 // box into every ancestor with atomic min/max, as long as it still enlarges the ancestor; it stops at the first
 // ancestor that already contains it.  Every extreme of that ancestor was set by some leaf that enlarged it and
@@ -756,11 +786,18 @@ constexpr int kMergeBlock = 256;
 template <typename T, int D>
 __global__ __launch_bounds__(kMergeBlock) void bvh_merge_kernel(const int* __restrict__ parent, const int2* __restrict__ node_range,
                                                           const T* __restrict__ node_box, long long* enc_box, int M,
-                                                          size_t total, unsigned own_blocks, SortJob rider) {
+                                                          size_t total, unsigned own_blocks, SortJob rider,
+                                                          const int2* __restrict__ children, int* __restrict__ frontier,
+                                                          size_t mixtures) {
     __shared__ long long local_box[kMergeBlock][2 * D];
     __shared__ int local_parent[kMergeBlock];
     __shared__ int is_local[kMergeBlock];
     static_assert(kMergeBlock == kBlock, "the riding sort pass works with kBlock lanes");
+    if (blockIdx.x >= own_blocks + rider.blocks) {          // behind both: one wavefront per tree finds where descents start
+        const size_t bl = size_t(blockIdx.x - own_blocks - rider.blocks) * (kMergeBlock / kWave) + (threadIdx.x >> 6);
+        if (bl < mixtures) tree_frontier(children + bl * (M - 1), M, frontier + bl * (1 + kFrontier), threadIdx.x & 63);
+        return;
+    }
     if (blockIdx.x >= own_blocks) { radix_scatter_pass(rider, blockIdx.x - own_blocks); return; }   // (see bvh_leaves_kernel)
     const size_t first_leaf = size_t(blockIdx.x) * kMergeBlock;          // leaves of all mixtures, numbered through
     const size_t t = first_leaf + threadIdx.x;
@@ -1040,7 +1077,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
         const int2* __restrict__ children, const T* __restrict__ leaf_rec, T* __restrict__ out,
         const T* __restrict__ grad_out, T* __restrict__ sums, T* __restrict__ grad_xes, CandidateCache cache,
         T* __restrict__ piece_gx, int helpers, int L, int M, int N, int Bx, int Lx, int chunks, int groups_per_workgroup,
-        int xes_shared) {
+        int xes_shared, const int* __restrict__ frontier) {
     constexpr int LS = LeafRec<D>::kStride;
     constexpr int NR = BvhSums<D>::k;
     constexpr int kVals = MODE == 0 ? 1 : D;
@@ -1127,6 +1164,12 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             for (int k = 0; k < kAhead; ++k)
                 if (lane + k * kWave < n_ahead) list_ahead[k] = src[lane + k * kWave];
         }
+        // the nodes the descent starts from (tree_frontier), fetched with everything else
+        int start_count = 0, start_node = 0;
+        if (piece < 0 && M > 1) {
+            start_count = frontier[size_t(bl) * (1 + kFrontier)];
+            start_node = frontier[size_t(bl) * (1 + kFrontier) + 1 + lane];
+        }
         int pid = valid ? p_order[xseg * N + j] : 0;
         pid = unsigned(pid) < unsigned(N) ? pid : 0;        // a permutation by construction; never index out of bounds
         T x[D];
@@ -1140,14 +1183,17 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
         pids[wave][lane] = valid ? pid : -1;
         if (cache.count) my_stamp = points_stamp<T, D>(x, valid, lane);
         const bool any = group * kWave < N;
+        start_count = __builtin_amdgcn_readfirstlane(start_count);
+        start_count = start_count < 1 ? 1 : (start_count > kFrontier ? kFrontier : start_count);
+        // (a count or a node outside the tree cannot come from the build; the clamps keep a bug from indexing out of bounds)
+        stack[wave][lane] = (lane < start_count && unsigned(start_node) < unsigned(M - 1)) ? start_node : 0;
         if (lane == 0) {
             // a single Gaussian is a tree without internal nodes: its leaf is the only candidate
-            stack[wave][0] = 0;
             leaves[wave][0] = 0;
             state[wave][0] = (any && M == 1) ? 1 : 0;
             state[wave][1] = 0;
         }
-        sp = (any && M > 1) ? 1 : 0;
+        sp = (any && M > 1) ? start_count : 0;
         if (piece >= 0) {
             // A piece is worked on only while it is one of the pieces its group has published last, for points with
             // the stamp of the ones loaded here; the owner of the group applies the same test to the list and
@@ -1775,8 +1821,10 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         if (M > 1) {
             const size_t ni = BL * (M - 1);
             const unsigned merge_blocks = unsigned((n + kMergeBlock - 1) / kMergeBlock);
-            bvh_merge_kernel<T, D><<<dim3(merge_blocks + jp_second.blocks), dim3(kMergeBlock), 0, st>>>(
-                parent, node_range, node_box, enc_box, M, n, merge_blocks, jp_second);
+            const unsigned frontier_blocks = unsigned((BL + kMergeBlock / kWave - 1) / (kMergeBlock / kWave));
+            bvh_merge_kernel<T, D><<<dim3(merge_blocks + jp_second.blocks + frontier_blocks), dim3(kMergeBlock), 0, st>>>(
+                parent, node_range, node_box, enc_box, M, n, merge_blocks, jp_second, children,
+                (int*)(bvh + lay.frontier), BL);
             bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(
                 children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups);
         } else if (jp_second.blocks > 0) {           // single leaves have no boxes to merge
@@ -1824,7 +1872,7 @@ static int bvh_fwd_t(const T* xes, char* bvh, T* out, const gmc_shape& s, hipStr
     bvh_traverse_kernel<T, D, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kTravBlock), 0, st>>>(
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children),
         (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, candidate_cache(bvh, lay), nullptr, 0,
-        s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, 0);
+        s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, 0, (const int*)(bvh + lay.frontier));
     return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
 }
 
@@ -1857,7 +1905,7 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bv
 #define GMC_TRAV(GM, GX) bvh_traverse_kernel<T, D, 1, GM, GX><<<grid, dim3(kTravBlock), 0, st>>>( \
         xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.child_box), (const int2*)(bvh + lay.children), \
         (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, cache, piece_gx, helpers, \
-        s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, xes_shared)
+        s.L, s.M, s.N, s.Bx, s.Lx, chunks, groups, xes_shared, (const int*)(bvh + lay.frontier))
     if (gm && gx) GMC_TRAV(true, true);
     else if (gm) GMC_TRAV(true, false);
     else if (gx) GMC_TRAV(false, true);
