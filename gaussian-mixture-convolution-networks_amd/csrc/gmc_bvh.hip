@@ -1091,9 +1091,12 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     // results per point, in double: the forward sums are added wavefront by wavefront (deterministic), dL/dx with
     // LDS atomics (cheap for doubles on distinct words, unlike floats)
     __shared__ double result[kGroupsMax][kVals][kWave];
-    // per wavefront: the staged leaf records of a batch; between two groups its partial results per point
-    static_assert(kStageBatch * LS >= kWave, "staging area too small for the partial results");
+    // per wavefront: the staged leaf records of a batch
     __shared__ __attribute__((aligned(16))) T staged_mem[kTravWaves][kStageBatch * LS];
+    // forward pass: what every wavefront has summed for every group in this round; added up in wavefront order when all
+    // groups of the round are through (one barrier per round; with a barrier pair per group the workgroup waited for
+    // its slowest wavefront once per group)
+    __shared__ T partial[MODE == 0 ? kGroupsMax : 1][MODE == 0 ? kTravWaves : 1][kWave];
     // double in both precisions: LDS atomic adds of doubles on distinct addresses cost a few cycles per
     // instruction, those of floats are serialised lane by lane
     __shared__ double rsum_mem[kTravWaves][NEED_GM ? kStageBatch * NR : 1];
@@ -1402,7 +1405,7 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             wave_lds_fence();
         }
         if (MODE == 0) {
-            staged[lane] = acc;                         // the staging area is idle now
+            partial[gi][wave][lane] = acc;
         } else if (NEED_GX) {
 #pragma unroll
             for (int d = 0; d < D; ++d) atomic_add(&result[gi][d][lane], double(gx[d]));
@@ -1525,17 +1528,16 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
             left_on_stack |= state[gi][1] > 0;
             if (n_leaf == 0) continue;                                  // uniform over the workgroup
             evaluate_share(gi);
-            if (MODE == 0) {
-                // forward: the wavefronts' partial sums are added in a fixed order (the backward pass has added
-                // its dL/dx with atomics and goes on to the next group without waiting for the other wavefronts)
-                __syncthreads();
-                if (wave == 0) {
-                    T v = T(0);
+        }
+        if (MODE == 0) {
+            // forward: the wavefronts' partial sums are added in a fixed order, by wavefront g for group g (the
+            // backward pass has added its dL/dx with atomics)
+            __syncthreads();
+            if (wave < groups && state[wave][0] > 0) {
+                T v = T(0);
 #pragma unroll
-                    for (int w = 0; w < kTravWaves; ++w) v += staged_mem[w][lane];
-                    result[gi][0][lane] += double(v);
-                }
-                __syncthreads();
+                for (int w = 0; w < kTravWaves; ++w) v += partial[wave][w][lane];
+                result[wave][0][lane] += double(v);
             }
         }
         if (publish) {
