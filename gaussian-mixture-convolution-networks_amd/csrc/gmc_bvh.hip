@@ -12,11 +12,14 @@
 //   evaluation records -> Karras radix tree over the unique keys (morton << 32 | rank), as lbvh/building.h:11-103
 //   -> bottom-up union of boxes with integer atomic min/max on order-preserving encodings.
 // Query points are Morton-sorted the same way (on their top 16 or 8 key bits) so that a wavefront owns 64
-// neighbouring points.
+// neighbouring points; their two sort passes ride as extra workgroups in the two longest launches of the tree
+// construction, and one wavefront per tree leaves a cut through the tree a few levels below the root (tree_frontier).
 //
 // Traversal: 64 sorted points form a group with ONE node stack (LDS); lanes work on tree nodes while the tree is
 // descended and on points while the gathered leaves are evaluated; a workgroup serves up to four groups, whose
-// descents overlap (see bvh_traverse_kernel).  Backward collects the per-Gaussian sums of a batch of leaves in LDS
+// descents overlap (see bvh_traverse_kernel).  A descent starts from the cut the build has left and tests node boxes
+// against one or two boxes around the group's points (two where the group straddles a jump of the Morton curve,
+// see group_boxes).  Backward collects the per-Gaussian sums of a batch of leaves in LDS
 // and issues one global atomic per non-zero scalar, leaf and wavefront.  The candidate leaves of every group stay
 // in the BVH object after the first traversal, so the backward pass after a forward pass does not descend, and
 // long lists are cut into pieces that helper workgroups of the backward launch take over (see kPieceLeaves).
