@@ -346,24 +346,6 @@ __device__ inline void box_half_extent(const T* __restrict__ g, double threshold
     for (int k = 0; k < D; ++k) delta[k] = s * (literal ? lit[k] : tight[k]);
 }
 
-// minimum / maximum over the workgroup of every lane's (lo, hi); thread t < 2D returns component t of
-// (min_0..min_D-1, max_0..max_D-1), the other threads return garbage
-template <typename T, int D>
-__device__ __forceinline__ T block_bounds(const T (&lo)[D], const T (&hi)[D], T (*red)[kBlock]) {
-    for (int d = 0; d < D; ++d) { red[d][threadIdx.x] = lo[d]; red[D + d][threadIdx.x] = hi[d]; }
-    __syncthreads();
-    for (int s = kBlock / 2; s > 0; s >>= 1) {
-        if (int(threadIdx.x) < s)
-            for (int d = 0; d < D; ++d) {
-                const T a = red[d][threadIdx.x + s], b = red[D + d][threadIdx.x + s];
-                if (a < red[d][threadIdx.x]) red[d][threadIdx.x] = a;
-                if (b > red[D + d][threadIdx.x]) red[D + d][threadIdx.x] = b;
-            }
-        __syncthreads();
-    }
-    return red[threadIdx.x < 2 * D ? threadIdx.x : 0][0];
-}
-
 // One launch for two independent jobs.
 // Workgroups [0, box_blocks): workgroup (blk, seg) leaves the bounds of its 256 centres in parts_g[seg][blk].  (The
 // cutoff boxes of the Gaussians, a long chain of double arithmetic, are not needed before the leaves are written:

@@ -449,6 +449,24 @@ __device__ __forceinline__ void clock_probe_end(const ClockProbe& c, long long* 
 //   R0 = sum_n e g,  R1_i = sum_n e g y_i,  R2_ij = sum_n e g y_i y_j (i <= j)     with e = exp2(-|y|^2)
 template <int D> struct Sums { static constexpr int k = 1 + D + D * (D + 1) / 2; };   // 6 / 10
 
+// minimum / maximum over the workgroup of every lane's (lo, hi); thread t < 2D returns component t of
+// (min_0..min_D-1, max_0..max_D-1), the other threads return garbage; red[k][0] holds component k for every thread
+template <typename T, int D>
+__device__ __forceinline__ T block_bounds(const T (&lo)[D], const T (&hi)[D], T (*red)[kBlock]) {
+    for (int d = 0; d < D; ++d) { red[d][threadIdx.x] = lo[d]; red[D + d][threadIdx.x] = hi[d]; }
+    __syncthreads();
+    for (int s = kBlock / 2; s > 0; s >>= 1) {
+        if (int(threadIdx.x) < s)
+            for (int d = 0; d < D; ++d) {
+                const T a = red[d][threadIdx.x + s], b = red[D + d][threadIdx.x + s];
+                if (a < red[d][threadIdx.x]) red[d][threadIdx.x] = a;
+                if (b > red[D + d][threadIdx.x]) red[D + d][threadIdx.x] = b;
+            }
+        __syncthreads();
+    }
+    return red[threadIdx.x < 2 * D ? threadIdx.x : 0][0];
+}
+
 template <typename T>
 inline void zero_async(T* p, size_t n, hipStream_t stream) {
     if (n == 0) return;

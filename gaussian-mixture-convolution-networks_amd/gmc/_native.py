@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 7
+ABI_VERSION = 8
 STATIC_SCRATCH_BYTES = 64 << 20
 
 
@@ -74,7 +74,9 @@ def lib() -> ctypes.CDLL:
     l.gmc_eval_componentwise_bwd.argtypes = [vp, vp, vp, vp, vp, vp, sz, shp, ci, ci, ci, vp]
     l.gmc_relu_fit_goal.argtypes = [vp, vp, vp, vp, shp, vp]
     l.gmc_relu_fit_step.argtypes = [vp, vp, vp, vp, shp, vp]
-    l.gmc_eval_cov_moments.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_double, shp, ci, vp]
+    l.gmc_eval_cov_moments_bytes.restype = sz
+    l.gmc_eval_cov_moments_bytes.argtypes = [shp]
+    l.gmc_eval_cov_moments.argtypes = [vp, vp, vp, vp, sz, vp, vp, vp, vp, vp, ctypes.c_double, shp, ci, vp]
     l.gmc_batch_norm_sampling_positions.argtypes = [vp, vp, shp, vp]
     l.gmc_validate_mixture.argtypes = [vp, vp, shp, vp]
     cshp = ctypes.POINTER(ConvShape)
@@ -335,9 +337,10 @@ def eval_cov_moments(mixture: torch.Tensor, constant: torch.Tensor, xes: torch.T
     sd = torch.empty(dims, dtype=mixture.dtype, device=mixture.device)
     mean = torch.empty_like(sd)
     inv = torch.empty_like(sd) if want_inverse else None
-    moments = torch.empty(dims + (2,), dtype=torch.float64, device=mixture.device)
+    scratch = int(lib().gmc_eval_cov_moments_bytes(ctypes.byref(shape)))
+    moments = torch.empty(max(scratch // 8, 1), dtype=torch.float64, device=mixture.device)
     with _on(mixture.device):
-        check(lib().gmc_eval_cov_moments(_p(mixture), _p(constant), _p(xes), _p(moments), _p(sd), _p(mean), _p(inv),
+        check(lib().gmc_eval_cov_moments(_p(mixture), _p(constant), _p(xes), _p(moments), scratch, _p(sd), _p(mean), _p(inv),
                                          _p(running_sd), _p(running_mean), float(alpha), ctypes.byref(shape),
                                          int(per_sample), _stream(mixture.device)))
     return (sd, mean, inv) if want_inverse else (sd, mean)

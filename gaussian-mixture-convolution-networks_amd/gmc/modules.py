@@ -22,11 +22,21 @@ class BatchNorm(torch.nn.Module):
     standard deviation, and takes the sampled mean off the constant.
 
     batch_norm=True: statistics over batch and samples with running averages (used at evaluation time as well);
-    batch_norm=False: per training sample.  The statistics carry no gradient; the scaling of the weights does."""
+    batch_norm=False: per training sample.  The statistics carry no gradient; the scaling of the weights does.
 
-    def __init__(self, n_layers: int, batch_norm: bool = True, learn_scaling: bool = True):
+    Two differences from the reference layer, both in evaluation mode with batch_norm=True, where the running
+    averages alone decide the result: the reference still draws its torch.rand sampling positions and evaluates
+    them (src/gmc/modules.py:396-401) before it discards the statistics (:411-412); this layer samples nothing, so
+    sampling positions passed to forward() are not used there, and the global random stream is not advanced unless
+    reference_rng_stream=True asks for the reference's draw (same shape and device, default dtype) to be made and
+    dropped.  Mixtures may be float64 (the reference's float32 sampling positions restrict it to float32): the
+    statistics are then formed in float64 and stored into the layer's buffers in the buffers' dtype."""
+
+    def __init__(self, n_layers: int, batch_norm: bool = True, learn_scaling: bool = True,
+                 reference_rng_stream: bool = False):
         super().__init__()
         self.batch_norm = batch_norm
+        self.reference_rng_stream = reference_rng_stream
         self.learnable_scaling = torch.nn.Parameter(torch.ones(n_layers)) if learn_scaling else None
         self.register_buffer("averaged_channel_sd", torch.ones(n_layers))
         self.register_buffer("averaged_channel_mean", torch.ones(n_layers))
@@ -52,8 +62,10 @@ class BatchNorm(torch.nn.Module):
         with torch.no_grad():
             if self.batch_norm and not self.training:
                 # the running averages alone decide: nothing to sample
-                mean = self.averaged_channel_mean
-                scaling = 1 / torch.clamp(self.averaged_channel_sd, min=0.001)
+                if self.reference_rng_stream:
+                    torch.rand(gm.n_batch(x_gm), n_channels, 10000 // gm.n_batch(x_gm), gm.n_dimensions(x_gm), device=x_gm.device)
+                mean = self.averaged_channel_mean.to(x_gm.dtype)
+                scaling = 1 / torch.clamp(self.averaged_channel_sd.to(x_gm.dtype), min=0.001)
             else:
                 if sampling_positions is None:
                     sampling_positions = self.sampling_positions(x_gm)
@@ -61,10 +73,17 @@ class BatchNorm(torch.nn.Module):
                 alpha = min(gm.n_batch(x_gm) / 1000, 0.1)
                 # evaluation, torch.std_mean, the update of the running averages and 1 / max(sd, 0.001) in three small
                 # launches: the sampled values never go to memory
+                run_sd = run_mean = None
+                if running:
+                    # (buffers of another dtype than the mixture: averaged in the mixture's dtype, stored back below)
+                    run_sd = self.averaged_channel_sd.to(x_gm.dtype)
+                    run_mean = self.averaged_channel_mean.to(x_gm.dtype)
                 _, mean, scaling = _native.eval_cov_moments(
                     x_gm.detach().contiguous(), x_constant.detach(), sampling_positions.contiguous(),
-                    per_sample=not self.batch_norm, running_sd=self.averaged_channel_sd if running else None,
-                    running_mean=self.averaged_channel_mean if running else None, alpha=alpha, want_inverse=True)
+                    per_sample=not self.batch_norm, running_sd=run_sd, running_mean=run_mean, alpha=alpha, want_inverse=True)
+                if running and run_sd is not self.averaged_channel_sd:
+                    self.averaged_channel_sd.copy_(run_sd)
+                    self.averaged_channel_mean.copy_(run_mean)
 
         if self.learnable_scaling is not None:
             scaling = scaling * self.learnable_scaling

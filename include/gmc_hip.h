@@ -100,7 +100,8 @@ int gmc_eval_cov_bwd(const void* grad_out, const void* mixture, const void* xes,
  * the call allocates nothing.  Shapes with gmc_eval_bwd_workspace_bytes(shape) > GMC_STATIC_SCRATCH_BYTES return
  * GMC_E_TOO_LARGE (need_grad_mixture == 0 needs no scratch and is never refused).  All calls on one GPU share the
  * array: calls that overlap on one GPU (two streams, two threads) race; stream-ordered calls are safe, each clears
- * what it uses.  The address of the array is looked up at the first call on a device. */
+ * what it uses.  The address of the array is looked up at the first call on a device (a symbol lookup, not a
+ * stream operation): make one eager call per device before a call is recorded under HIP graph capture. */
 #define GMC_STATIC_SCRATCH_BYTES (64u << 20)
 int gmc_eval_bwd_static(const void* grad_out, const void* mixture, const void* xes, void* grad_mixture, void* grad_xes,
                         const gmc_shape* shape, int need_grad_mixture, int need_grad_xes, int covariance_form,
@@ -136,13 +137,17 @@ int gmc_relu_fit_step(const void* fitting_mixture, const void* x_in, const void*
 /* Sampled moments of BatchNorm, src/gmc/modules.py:401-415: the mixture is evaluated at xes [B][L][N][D] and
  * torch.std_mean of (value + constant[b,l]) is returned without the values going to memory: over batch and samples
  * per channel (per_sample == 0: outputs [L]) or over the samples of every (b,l) (per_sample != 0: [B][L]); sd is the
- * unbiased one.  `moments`: device scratch of 2 doubles per output element (sum, sum of squares; cleared inside).
+ * unbiased one.  The statistics are formed as torch.std_mean forms them, from deviations around a mean (every workgroup
+ * leaves count, mean and squared deviations of its values, merged pairwise in a fixed order), so a large constant
+ * with a small spread of the values keeps its digits and the result is the same bit for bit from run to run.
+ * `moments`: device scratch of gmc_eval_cov_moments_bytes(shape) bytes (not cleared, fully written).
  * running_sd / running_mean (both or neither; may be NULL): the running averages of modules.py:405-410, updated in
  * place to (1 - alpha) * running + alpha * statistic; sd and mean then return the averages.  inv_sd (may be NULL)
  * receives 1 / max(sd, 0.001) (modules.py:414-415). */
-int gmc_eval_cov_moments(const void* mixture, const void* constant, const void* xes, double* moments, void* sd, void* mean,
-                         void* inv_sd, void* running_sd, void* running_mean, double alpha, const gmc_shape* shape,
-                         int per_sample, void* stream);
+size_t gmc_eval_cov_moments_bytes(const gmc_shape* shape);
+int gmc_eval_cov_moments(const void* mixture, const void* constant, const void* xes, double* moments, size_t moments_bytes,
+                         void* sd, void* mean, void* inv_sd, void* running_sd, void* running_mean, double alpha,
+                         const gmc_shape* shape, int per_sample, void* stream);
 /* Sampling positions of BatchNorm, src/gmc/modules.py:394-400: uniform numbers in [0, 1) [B][L][N][D] are turned, in
  * place, into positions inside the box of all centres of their batch entry (2-D: widened by u * 1.3 - 0.15). */
 int gmc_batch_norm_sampling_positions(const void* mixture, void* uniform_in_positions_out, const gmc_shape* shape, void* stream);
@@ -176,6 +181,14 @@ int gmc_convolution_bwd(const void* grad_out, const void* data, const void* kern
  *   out[b,l,n] = sum over Gaussians m whose own box contains x_n (closed interval, lbvh/aabb.h:39-47).
  */
 enum { GMC_AABB_REFERENCE = 0, GMC_AABB_TIGHT = 1 };
+
+/* Of lbvh::Config (lbvh/Config.h:5-10) the box rule and its threshold are configurable.  Its MortonCodeAlgorithm has
+ * one value here, `Old` (lbvh/morton_code.h:145-168: 30 bits of the normalised centre, extended by the component
+ * index; the reference's default).  The variants Cov1 ... Cov4 (lbvh/bvh.cu:87-101) mix bits of the covariance into
+ * the key and so give trees of another shape; every internal box is the exact union of its children's boxes and the
+ * query visits a leaf exactly when its own box contains the point, so the culled sums and gradients are the same for
+ * any key: the choice could only change the time a traversal takes, and there is no `make_aabbs = false` mode (trees
+ * without boxes cannot be queried). */
 
 typedef struct gmc_bvh_config {
     int aabb_mode;          /* GMC_AABB_REFERENCE: the rule of lbvh/bvh.cu:190-223; GMC_AABB_TIGHT: exact box */

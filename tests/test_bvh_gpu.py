@@ -609,6 +609,94 @@ def test_workload_c5_full(mode):
     _c5_check(16384, 100000, mode)
 
 
+# Relative agreement of the device's boxes with the oracle's rule that the tests above assert (float32 boxes are the
+# rounded float64 ones; the reference's trigonometric 3x3 eigen-solver is ill-conditioned, so its device and numpy
+# restatements agree less closely than the closed-form tight rule).
+BOX_AGREEMENT = {(torch.float32, "reference"): 2e-6, (torch.float32, "tight"): 2e-6,
+                 (torch.float64, "reference"): 1e-6, (torch.float64, "tight"): 1e-12}
+FLIP_COUNTS = {}
+
+
+def _membership_flips(lo_a, up_a, lo_b, up_b, x_np, chunk=4096):
+    """(b, l, m, n) of every pair whose point-in-box test (closed interval, lbvh/aabb.h:39-47) differs between the
+    two sets of boxes, and the number of pairs inside the second set.  Exact comparisons in float64, chunked over
+    the points so that a full-size workload never holds a [M, N] mask."""
+    B, L, M, D = lo_a.shape
+    Bx, Lx, N, _ = x_np.shape
+    flips, inside = [], 0
+    for b in range(B):
+        for l in range(L):
+            x = torch.from_numpy(np.ascontiguousarray(x_np[min(b, Bx - 1), min(l, Lx - 1)], dtype=np.float64))
+            la, ua, lb, ub = (torch.from_numpy(np.ascontiguousarray(t[b, l], dtype=np.float64))[:, None, :]
+                              for t in (lo_a, up_a, lo_b, up_b))
+            for n0 in range(0, N, chunk):
+                xc = x[None, n0:n0 + chunk, :]
+                in_a = ((xc >= la) & (xc <= ua)).all(-1)
+                in_b = ((xc >= lb) & (xc <= ub)).all(-1)
+                inside += int(in_b.sum())
+                m_idx, n_idx = torch.nonzero(in_a != in_b, as_tuple=True)
+                flips += [(b, l, int(m), int(n) + n0) for m, n in zip(m_idx.tolist(), n_idx.tolist())]
+    return flips, inside
+
+
+def _check_against_oracle_boxes(mix, xes, gout, dtype, mode, tag):
+    """The reference's rule is the sum over the Gaussians whose box, as lbvh/bvh.cu:164-231 computes it, contains
+    the point (lbvh/aabb.h:39-47).  The device result is compared with the masked sum over the ORACLE's boxes (not
+    the device's own): every pair whose membership differs between the two sets of boxes is listed, must lie within
+    the boxes' agreement of a face, and their number must be what that agreement predicts; every point and every
+    Gaussian that no such pair touches must agree to the parity bar."""
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    m_np, x_np, g_np = (t.numpy().astype(npdt) for t in (mix, xes, gout))
+    D = x_np.shape[-1]
+    _, dlo, dup = _device_boxes(mix, xes, dtype, mode)
+    olo, oup = o.gaussian_aabbs(m_np, mode=mode)
+    olo, oup = olo.astype(npdt).astype(np.float64), oup.astype(npdt).astype(np.float64)   # Aabb<T> holds scalars of type T
+    out, gmix, gxes = _run_culled(mix, xes, gout, dtype, mode)
+    flips, inside = _membership_flips(dlo, dup, olo, oup, x_np)
+    agree = BOX_AGREEMENT[(dtype, mode)]
+    FLIP_COUNTS[tag] = (len(flips), inside)
+    print(f"oracle-box parity {tag}: {len(flips)} membership flips among {inside} pairs inside a box", flush=True)
+    # a pair can flip only if its point lies within the boxes' disagreement of a face
+    Bx, Lx = x_np.shape[:2]
+    for b, l, m, n in flips:
+        x = x_np[min(b, Bx - 1), min(l, Lx - 1), n].astype(np.float64)
+        ext = oup[b, l, m] - olo[b, l, m]
+        dist = np.minimum(np.abs(x - olo[b, l, m]), np.abs(x - oup[b, l, m])) / ext
+        assert dist.min() <= 4 * agree, f"{tag}: pair {(b, l, m, n)} flipped {dist.min():.3g} box extents away from a face"
+    # the shell of relative width `agree` on either side of the 2D faces holds about 2 D agree of a box's points
+    assert len(flips) <= 10 + 8 * D * agree * inside, f"{tag}: {len(flips)} flips among {inside} pairs"
+    ref = cpu_ref.forward(m_np.astype(np.float64), x_np.astype(np.float64), olo, oup, n_threads=16)
+    rgm, rgx = cpu_ref.backward(g_np.astype(np.float64), m_np.astype(np.float64), x_np.astype(np.float64), olo, oup, n_threads=16)
+    keep_n = np.ones(out.shape, dtype=bool)               # points / Gaussians that no flipped pair touches
+    keep_m = np.ones(gmix.shape[:3], dtype=bool)
+    for b, l, m, n in flips:
+        keep_n[b, l, n] = False
+        keep_m[b, l, m] = False
+    tol, fl = TOL[dtype], FLOOR[dtype]
+    assert rel_l2(out[keep_n], ref[keep_n], fl) <= tol, f"forward {tag}"
+    assert rel_l2(gmix[keep_m], rgm[keep_m], fl) <= tol, f"grad mixture {tag}"
+    if x_np.shape[:2] == out.shape[:2]:
+        assert rel_l2(gxes[keep_n], rgx[keep_n], fl) <= tol, f"grad xes {tag}"
+    else:                                                  # broadcast points: a flip in any mixture touches the shared row
+        shared = keep_n.all(axis=(0, 1))
+        assert rel_l2(gxes[0, 0][shared], rgx[0, 0][shared], fl) <= tol, f"grad xes {tag}"
+
+
+@pytest.mark.parametrize("mode", ["reference", "tight"])
+def test_culled_result_against_the_oracles_own_boxes(mode):
+    for dtype, (B, L, M, N, D, bc) in ((torch.float32, (3, 2, 300, 3000, 3, False)),
+                                       (torch.float32, (4, 3, 200, 2500, 2, True)),
+                                       (torch.float64, (2, 2, 400, 2000, 2, False))):
+        mix, xes, gout = _case(B, L, M, N, D, seed=8100 + D + B, broadcast=bc)
+        _check_against_oracle_boxes(mix, xes, gout, dtype, mode, f"B{B} L{L} M{M} N{N} D{D} {dtype} {mode}")
+
+
+@pytest.mark.parametrize("mode", ["reference", "tight"])
+def test_workload_c5_full_against_the_oracles_own_boxes(mode):
+    wl, mix, xes, gout = synthetic.make_workload("C5")
+    _check_against_oracle_boxes(mix, xes, gout, torch.float64, mode, f"C5 {mode}")
+
+
 def test_step_is_capturable_in_a_hip_graph():
     """The library only enqueues kernels on the caller's stream (no allocation, no synchronisation, no memset
     nodes), so a whole step -- LBVH build, culled forward and backward, dense forward and backward -- can be

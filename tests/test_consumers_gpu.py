@@ -138,6 +138,43 @@ def test_batch_norm(batch_norm):
     assert torch.all(mt.grad[..., 1:] == 0) and torch.all(mt.grad[..., 0] != 0)
 
 
+def test_batch_norm_float64_training_and_the_random_stream():
+    """A float64 mixture through a layer whose buffers are float32 (the default): the statistics are formed in float64
+    and stored into the buffers; in evaluation mode the layer draws nothing unless the reference's draw is asked for."""
+    rng = np.random.default_rng(32)
+    m = _cov_mixture(rng, 4, 3, 30, 2, cov=0.1)
+    const = rng.normal(size=(4, 3))
+    layer = modules.BatchNorm(3, batch_norm=True, learn_scaling=False).to(DEV)
+    mt, ct = torch.tensor(m, device=DEV), torch.tensor(const, device=DEV)
+    xes = layer.sampling_positions(mt)
+    assert xes.dtype == torch.float64
+    scaled, new_const = layer((mt, ct), sampling_positions=xes)
+    values = o.evaluate(m, xes.cpu().numpy()) + const[..., None]
+    vt = np.transpose(values, (1, 0, 2)).reshape(3, -1)
+    alpha = min(4 / 1000, 0.1)
+    sd = (1 - alpha) * 1.0 + alpha * vt.std(axis=1, ddof=1)
+    mean = (1 - alpha) * 1.0 + alpha * vt.mean(axis=1)
+    assert scaled.dtype == torch.float64 and layer.averaged_channel_sd.dtype == torch.float32
+    assert rel_l2(scaled[..., 0].cpu().numpy(), m[..., 0] / sd[None, :, None]) <= 1e-12
+    assert rel_l2(new_const.cpu().numpy(), const - mean[None, :]) <= 1e-12
+    assert rel_l2(layer.averaged_channel_sd.cpu().numpy(), sd) <= 1e-6
+    assert rel_l2(layer.averaged_channel_mean.cpu().numpy(), mean) <= 1e-6
+    # evaluation mode: the running averages decide, whatever positions are passed; no random numbers are drawn ...
+    layer.eval()
+    torch.manual_seed(5)
+    state = torch.cuda.get_rng_state(DEV)
+    a, _ = layer((mt, ct))
+    b, _ = layer((mt, ct), sampling_positions=xes)
+    assert torch.equal(a, b) and torch.equal(torch.cuda.get_rng_state(DEV), state)
+    # ... unless the reference's draw (src/gmc/modules.py:396) is asked for: the stream then advances as it does there
+    layer.reference_rng_stream = True
+    layer((mt, ct))
+    after_layer = torch.rand(3, device=DEV)
+    torch.cuda.set_rng_state(state, DEV)
+    torch.rand(4, 3, 10000 // 4, 2, device=DEV)
+    assert torch.equal(after_layer, torch.rand(3, device=DEV))
+
+
 def test_layer_pipeline_against_the_oracle_composition():
     """convolution -> batch norm (per sample) -> ReLU fixed-point fitting -> evaluation on a grid, the order in which
     a network layer of the reference chains these pieces (src/gmc/modules.py:163, :374-425, src/gmc/fitting.py:287-312),
@@ -268,6 +305,35 @@ def test_fused_moments_are_std_mean_of_the_sampled_values(D, dtype):
                 assert torch.isnan(sd).all()                  # one value: torch.std_mean returns nan as well
             else:
                 assert rel_l2(sd.cpu().numpy(), ref_sd) <= 10 * TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("ratio", [1e4, 1e5])
+def test_fused_moments_behind_a_large_constant(dtype, ratio):
+    """A constant `ratio` times the spread of the sampled values (BatchNorm behind a large bias): the standard deviation
+    must come out as numpy.std(ddof=1) of the oracle's values gives it (torch.std_mean, src/gmc/modules.py:401-415, works
+    on deviations from the mean as well); sums of values and of squares would lose ratio^2 ulps of it.  Several
+    workgroups per statistic, per channel and per (b, l), and twice in a row: the result is the same bit for bit."""
+    rng = np.random.default_rng(77)
+    npdt = np.float32 if dtype == torch.float32 else np.float64
+    for B, L, M, N, D in ((3, 2, 40, 700, 2), (2, 3, 25, 100, 3)):
+        m = _cov_mixture(rng, B, L, M, D, cov=0.1).astype(npdt)
+        xes = rng.uniform(-1.5, 1.5, (B, L, N, D)).astype(npdt)
+        plain = o.evaluate(m.astype(np.float64), xes.astype(np.float64))
+        const = np.broadcast_to((ratio * plain.std(axis=(0, 2)))[None, :], (B, L)).astype(npdt)    # one constant per channel, as BatchNorm's bias
+        values = plain + const.astype(np.float64)[..., None]
+        mt, ct, xt = (torch.tensor(np.ascontiguousarray(a), device=DEV) for a in (m, const, xes))
+        for per_sample in (False, True):
+            sd, mean = _native.eval_cov_moments(mt, ct, xt, per_sample)
+            sd2, mean2 = _native.eval_cov_moments(mt, ct, xt, per_sample)
+            assert torch.equal(sd, sd2) and torch.equal(mean, mean2)
+            if per_sample:
+                ref_sd, ref_mean = values.std(axis=2, ddof=1), values.mean(axis=2)
+            else:
+                flat = np.transpose(values, (1, 0, 2)).reshape(L, -1)
+                ref_sd, ref_mean = flat.std(axis=1, ddof=1), flat.mean(axis=1)
+            assert rel_l2(mean.cpu().numpy(), ref_mean) <= TOL[dtype]
+            assert rel_l2(sd.cpu().numpy(), ref_sd) <= 10 * TOL[dtype], (per_sample, rel_l2(sd.cpu().numpy(), ref_sd))
 
 
 def test_batch_norm_sampling_positions_and_running_averages():

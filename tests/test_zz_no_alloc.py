@@ -40,13 +40,19 @@ def _both(mix, xes, gout, need_m, need_x, cov):
                      ws.data_ptr(), ws_bytes, ctypes.byref(shape), int(need_m), int(need_x), stream))
     # the entry point under test: outputs allocated here, nothing allocated inside
     gm_new, gx_new = torch.full_like(mix, 7.0), torch.full_like(xes, 7.0)
+    call = lambda: _native.check(lib.gmc_eval_bwd_static(gout.data_ptr(), mix.data_ptr(), xes.data_ptr(), gm_new.data_ptr(),
+                                                         gx_new.data_ptr(), ctypes.byref(shape), int(need_m), int(need_x),
+                                                         int(cov), stream))
+    call()                   # (the first call on a device looks up the array's address; code objects are loaded by now)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
-    _native.check(lib.gmc_eval_bwd_static(gout.data_ptr(), mix.data_ptr(), xes.data_ptr(), gm_new.data_ptr(),
-                                          gx_new.data_ptr(), ctypes.byref(shape), int(need_m), int(need_x), int(cov),
-                                          stream))
+    # free device memory as the driver reports it (hipMemGetInfo): an allocation inside the library, which torch's
+    # own counters would not see, lowers it
+    free_before, _ = torch.cuda.mem_get_info()
+    reserved_before = torch.cuda.memory_reserved()
+    call()
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    free_after, _ = torch.cuda.mem_get_info()
+    assert torch.cuda.memory_reserved() == reserved_before and free_after == free_before
     return (gm_ref.cpu().numpy(), gx_ref.cpu().numpy()), (gm_new.cpu().numpy(), gx_new.cpu().numpy())
 
 
@@ -79,11 +85,55 @@ def test_static_scratch_backward_two_calls_in_a_row(dtype):
 def test_static_scratch_backward_rejects_oversized_shapes():
     lib = _native.lib()
     null = ctypes.c_void_p(0)
-    one = ctypes.c_void_p(256)          # never dereferenced: the call must return before any launch
-    # 64 MiB / (10 floats) = 1 677 721 Gaussians in 3-D float32
+    # 64 MiB / (10 floats) = 1 677 721 Gaussians in 3-D float32.  Real buffers of the shape's sizes are passed: the call
+    # must return before any launch, but a regression of that check should give a wrong code, not a fault.
     big = _native.Shape(64, 64, 512, 16, 3, 64, 64, 0)
     assert lib.gmc_eval_bwd_workspace_bytes(ctypes.byref(big)) > _native.STATIC_SCRATCH_BYTES
-    rc = lib.gmc_eval_bwd_static(one, one, one, one, one, ctypes.byref(big), 1, 1, 0, null)
+    mix = torch.zeros(64, 64, 512, 13, device=DEV)
+    mix[..., [4, 8, 12]] = 1.0
+    xes = torch.zeros(64, 64, 16, 3, device=DEV)
+    gout = torch.zeros(64, 64, 16, device=DEV)
+    gmix, gxes = torch.empty_like(mix), torch.empty_like(xes)
+    rc = lib.gmc_eval_bwd_static(gout.data_ptr(), mix.data_ptr(), xes.data_ptr(), gmix.data_ptr(), gxes.data_ptr(),
+                                 ctypes.byref(big), 1, 1, 0, _native._stream(mix.device))
+    torch.cuda.synchronize()
     assert rc == -8 and b"static scratch" in lib.gmc_error_string(rc)
     assert lib.gmc_eval_bwd_static(null, null, null, null, null, ctypes.byref(_native.Shape(2, 2, 4, 5, 3, 2, 2, 0)),
                                    1, 1, 0, null) == -4
+
+
+def test_static_scratch_backward_in_a_captured_graph():
+    """After one eager call on the device (which looks up the address of the static array) the entry point only
+    enqueues kernels: it is captured into a HIP graph with outputs allocated beforehand, and every replay, with eager
+    work of the same entry point in between, gives what gmc_eval_bwd gives."""
+    lib = _native.lib()
+    mix, xes, gout = _inputs(3, 4, 300, 2500, 3, torch.float32, 4300)
+    shape = _native.check_input(mix, xes)
+    gm_ref, gx_ref = _native.eval_bwd(gout, mix, xes, True, True)
+    gm_new, gx_new = torch.empty_like(mix), torch.empty_like(xes)
+    small = _inputs(2, 2, 40, 300, 3, torch.float32, 4301)
+    small_shape = _native.check_input(small[0], small[1])
+    gm_small, gx_small = torch.empty_like(small[0]), torch.empty_like(small[1])
+
+    def call(stream):
+        _native.check(lib.gmc_eval_bwd_static(gout.data_ptr(), mix.data_ptr(), xes.data_ptr(), gm_new.data_ptr(),
+                                              gx_new.data_ptr(), ctypes.byref(shape), 1, 1, 0, stream))
+
+    call(_native._stream(mix.device))                       # the eager call that must precede a capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(_native._stream(mix.device))
+    torch.cuda.synchronize()
+    for _ in range(3):
+        gm_new.fill_(7.0)
+        gx_new.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert rel_l2(gm_new.cpu().numpy(), gm_ref.cpu().numpy()) <= 1e-5
+        assert rel_l2(gx_new.cpu().numpy(), gx_ref.cpu().numpy()) <= 1e-5
+        # eager work on the shared array between the replays
+        _native.check(lib.gmc_eval_bwd_static(small[2].data_ptr(), small[0].data_ptr(), small[1].data_ptr(), gm_small.data_ptr(),
+                                              gx_small.data_ptr(), ctypes.byref(small_shape), 1, 1, 0,
+                                              _native._stream(mix.device)))
+        torch.cuda.synchronize()
