@@ -101,14 +101,14 @@ def cpu_baseline(name: str):
     }
 
 
-def measure_bvh(aabb_mode: str, steps: int, warmup: int, copy_calibration: bool = False):
-    """LBVH-culled path on C5 (3-D, float64, one mixture of 16384 Gaussians, 100000 points).  A step builds the
-    tree (the mixture changes every training step), evaluates forward and backward.  Returns the step time (wall
-    clock over all steps), the timings of its parts (HIP events on the launch stream, medians over a second run of the
-    same steps) and the number of pairs actually evaluated."""
+def measure_bvh(aabb_mode: str, steps: int, warmup: int, copy_calibration: bool = False, name: str = "C5"):
+    """LBVH-culled path on a workload (default C5: 3-D, float64, one mixture of 16384 Gaussians, 100000 points).  A step
+    builds the trees (the mixtures change every training step), evaluates forward and backward.  Returns the step time
+    (wall clock over all steps), the timings of its parts (HIP events on the launch stream, medians over a second run of
+    the same steps) and the number of pairs actually evaluated."""
     import torch
     from gmc import _native, synthetic
-    wl, mix, xes, gout = synthetic.make_workload("C5")
+    wl, mix, xes, gout = synthetic.make_workload(name)
     dev = torch.device("cuda:0")
     mix, xes, gout = mix.to(dev), xes.to(dev), gout.to(dev)
     torch.cuda.synchronize()
@@ -153,9 +153,10 @@ def measure_bvh(aabb_mode: str, steps: int, warmup: int, copy_calibration: bool 
     bvh = _native.Bvh(mix, xes, 0.001, aabb_mode)
     lo, up = bvh.boxes()
     hits = 0
-    for n0 in range(0, wl.N, 2048):
-        x = xes[0, 0, n0:n0 + 2048].unsqueeze(1)                       # [n, 1, D]
-        hits += int(((x >= lo[0, 0].unsqueeze(0)) & (x <= up[0, 0].unsqueeze(0))).all(dim=-1).sum().item())
+    for b in range(wl.B):
+        for n0 in range(0, wl.N, 2048):
+            x = xes[b, :, n0:n0 + 2048].unsqueeze(2)                   # [L, n, 1, D]
+            hits += int(((x >= lo[b].unsqueeze(1)) & (x <= up[b].unsqueeze(1))).all(dim=-1).sum().item())
     return {"wl": wl, "ms_step": wall * 1e3 / steps, "build_ms": build_ms, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "hits": hits}
 
 
@@ -582,6 +583,13 @@ def main():
             "fwd_kernel": o["fwd_kernel"]}
         others["C5"] = {"config": "D=3 f64 B=1 L=1 M=16384 N=100000, LBVH-culled (threshold 0.001): build + forward + backward per step",
                         "by_aabb_mode": [bvh_summary(measure_bvh(mode, 20, 3), mode) for mode in ("reference", "tight")]}
+        for name in ("C2", "C3"):
+            r = measure_bvh("tight", 20, 3, name=name)
+            w = r["wl"]
+            others[name + "_culled"] = {
+                "config": f"{name} through the LBVH-culled path (aabb_mode=tight, threshold 0.001): build + forward + backward per step",
+                **bvh_summary(r, "tight"), "evaluated_fraction_of_dense": r["hits"] / w.pairs,
+                "dense_ms_per_step": others[name]["ms_per_step"]}
         line["other_workloads"] = others
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(dense_name)

@@ -306,8 +306,8 @@ __device__ inline void box_half_extent(const T* __restrict__ g, double threshold
             for (int j = 0; j < D; ++j) sigma[i][j] = double(c[i * D + j]);
     } else if constexpr (D == 2) {
         const double m00 = c[0], m01 = c[2], m10 = c[1], m11 = c[3];
-        const double det = m00 * m11 - m01 * m10;
-        sigma[0][0] = m11 / det; sigma[0][1] = -m01 / det; sigma[1][0] = -m10 / det; sigma[1][1] = m00 / det;
+        const double inv = 1.0 / (m00 * m11 - m01 * m10);        // one division; the entries are products with it
+        sigma[0][0] = m11 * inv; sigma[0][1] = -m01 * inv; sigma[1][0] = -m10 * inv; sigma[1][1] = m00 * inv;
     } else {
         double m[3][3];
         for (int i = 0; i < 3; ++i)
@@ -315,16 +315,20 @@ __device__ inline void box_half_extent(const T* __restrict__ g, double threshold
         const double c00 = m[1][1] * m[2][2] - m[1][2] * m[2][1];
         const double c01 = m[1][2] * m[2][0] - m[1][0] * m[2][2];
         const double c02 = m[1][0] * m[2][1] - m[1][1] * m[2][0];
-        const double det = m[0][0] * c00 + m[0][1] * c01 + m[0][2] * c02;
-        sigma[0][0] = c00 / det;
-        sigma[1][0] = c01 / det;
-        sigma[2][0] = c02 / det;
-        sigma[0][1] = (m[0][2] * m[2][1] - m[0][1] * m[2][2]) / det;
-        sigma[1][1] = (m[0][0] * m[2][2] - m[0][2] * m[2][0]) / det;
-        sigma[2][1] = (m[0][1] * m[2][0] - m[0][0] * m[2][1]) / det;
-        sigma[0][2] = (m[0][1] * m[1][2] - m[0][2] * m[1][1]) / det;
-        sigma[1][2] = (m[0][2] * m[1][0] - m[0][0] * m[1][2]) / det;
-        sigma[2][2] = (m[0][0] * m[1][1] - m[0][1] * m[1][0]) / det;
+        const double inv = 1.0 / (m[0][0] * c00 + m[0][1] * c01 + m[0][2] * c02);
+        sigma[0][0] = c00 * inv;
+        sigma[1][1] = (m[0][0] * m[2][2] - m[0][2] * m[2][0]) * inv;
+        sigma[2][2] = (m[0][0] * m[1][1] - m[0][1] * m[1][0]) * inv;
+        if (mode == GMC_AABB_REFERENCE) {                        // the tight box needs the diagonal only
+            sigma[1][0] = c01 * inv;
+            sigma[2][0] = c02 * inv;
+            sigma[0][1] = (m[0][2] * m[2][1] - m[0][1] * m[2][2]) * inv;
+            sigma[2][1] = (m[0][1] * m[2][0] - m[0][0] * m[2][1]) * inv;
+            sigma[0][2] = (m[0][1] * m[1][2] - m[0][2] * m[1][1]) * inv;
+            sigma[1][2] = (m[0][2] * m[1][0] - m[0][0] * m[1][2]) * inv;
+        } else {
+            sigma[1][0] = sigma[2][0] = sigma[0][1] = sigma[2][1] = sigma[0][2] = sigma[1][2] = 0.0;
+        }
     }
     double tight[D];
     for (int k = 0; k < D; ++k) tight[k] = sqrt(fmax(sigma[k][k], 0.0));
@@ -597,47 +601,59 @@ __device__ __forceinline__ long long ordered_bits(double v) {
 __device__ __forceinline__ double from_ordered_bits(long long k) {
     return __builtin_bit_cast(double, k ^ ((k >> 63) & 0x7fffffffffffffffll));
 }
-
-// number of leading bits shared by the unique keys (morton[i] << 32 | i) and (morton[j] << 32 | j); -1 outside
-__device__ __forceinline__ int common_prefix(const uint32_t* __restrict__ keys, int n, int i, int j) {
-    if (j < 0 || j >= n) return -1;
-    const uint32_t a = keys[i], b = keys[j];
-    if (a != b) return __clz(a ^ b);
-    return 32 + __clz(uint32_t(i) ^ uint32_t(j));
+__device__ __forceinline__ int ordered_bits(float v) {
+    const int b = __builtin_bit_cast(int, v);
+    return b ^ ((b >> 31) & 0x7fffffff);
 }
+__device__ __forceinline__ float from_ordered_bits(int k) { return __builtin_bit_cast(float, k ^ ((k >> 31) & 0x7fffffff)); }
 
-// internal node i of the radix tree of mixture bl (Karras 2012; lbvh/building.h:11-103)
-__device__ __forceinline__ void build_internal_node(const uint32_t* __restrict__ keys, int2* __restrict__ children,
-                                                    int* __restrict__ parent, int2* __restrict__ node_range, int M,
-                                                    size_t bl, int i) {
-    const size_t t = bl * (M - 1) + i;
-    const uint32_t* k = keys + bl * M;
+// Internal node i of the radix tree over the M sorted keys (Karras 2012; lbvh/building.h:11-103); key_at(j) returns the
+// j-th sorted Morton code, the unique keys are (code << 32 | j).  first / last: the range of leaves below the node;
+// left / right: its children, >= 0 an internal node, < 0 leaf ~index.
+template <typename KeyAt>
+__device__ __forceinline__ void radix_tree_node(KeyAt key_at, int M, int i, int& first, int& last, int& left, int& right) {
+    // number of leading bits shared by the unique keys a and b; -1 outside
+    auto common_prefix = [&](int a, int b) -> int {
+        if (b < 0 || b >= M) return -1;
+        const uint32_t ka = key_at(a), kb = key_at(b);
+        if (ka != kb) return __clz(ka ^ kb);
+        return 32 + __clz(uint32_t(a) ^ uint32_t(b));
+    };
     // range of keys covered by internal node i
-    int first, last;
     if (i == 0) { first = 0; last = M - 1; }
     else {
-        const int dl = common_prefix(k, M, i, i - 1), dr = common_prefix(k, M, i, i + 1);
+        const int dl = common_prefix(i, i - 1), dr = common_prefix(i, i + 1);
         const int dir = dr > dl ? 1 : -1;
         const int dmin = dr > dl ? dl : dr;
         int lmax = 2;
-        while (common_prefix(k, M, i, i + lmax * dir) > dmin) lmax <<= 1;
+        while (common_prefix(i, i + lmax * dir) > dmin) lmax <<= 1;
         int len = 0;
         for (int step = lmax >> 1; step > 0; step >>= 1)
-            if (common_prefix(k, M, i, i + (len + step) * dir) > dmin) len += step;
+            if (common_prefix(i, i + (len + step) * dir) > dmin) len += step;
         const int j = i + len * dir;
         first = i < j ? i : j;
         last = i < j ? j : i;
     }
     // split: the highest key that shares more than the node's prefix with the first key
-    const int dnode = common_prefix(k, M, first, last);
+    const int dnode = common_prefix(first, last);
     int split = first, stride = last - first;
     do {
         stride = (stride + 1) >> 1;
         const int mid = split + stride;
-        if (mid < last && common_prefix(k, M, first, mid) > dnode) split = mid;
+        if (mid < last && common_prefix(first, mid) > dnode) split = mid;
     } while (stride > 1);
-    const int left = (split == first) ? ~split : split;               // leaf `split` or internal node `split`
-    const int right = (split + 1 == last) ? ~(split + 1) : split + 1;
+    left = (split == first) ? ~split : split;               // leaf `split` or internal node `split`
+    right = (split + 1 == last) ? ~(split + 1) : split + 1;
+}
+
+// internal node i of the radix tree of mixture bl, keys in memory
+__device__ __forceinline__ void build_internal_node(const uint32_t* __restrict__ keys, int2* __restrict__ children,
+                                                    int* __restrict__ parent, int2* __restrict__ node_range, int M,
+                                                    size_t bl, int i) {
+    const size_t t = bl * (M - 1) + i;
+    const uint32_t* k = keys + bl * M;
+    int first, last, left, right;
+    radix_tree_node([&](int j) { return k[j]; }, M, i, first, last, left, right);
     children[t] = make_int2(left, right);
     node_range[t] = make_int2(first, last);
     int* par = parent + bl * (2 * size_t(M) - 1);
@@ -646,45 +662,24 @@ __device__ __forceinline__ void build_internal_node(const uint32_t* __restrict__
     if (i == 0) par[0] = -1;
 }
 
+// Leaf `leaf` (Morton order) of mixture bl, which holds component `comp`: the cutoff box of the Gaussian
+// (lbvh/bvh.cu:164-231; kept in component order too for gmc_bvh_export_boxes, and as the leaf's node box), its
+// evaluation record behind its own box, zeroed sums of the backward pass.  blo / bhi receive the box.
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
-                                                           T* __restrict__ box_hi, double threshold, int mode,
-                                                           const uint32_t* __restrict__ order,
-                                                           const uint32_t* __restrict__ keys, T* __restrict__ node_box,
-                                                           T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
-                                                           int2* __restrict__ children, int* __restrict__ parent,
-                                                           int2* __restrict__ node_range, int M, size_t total,
-                                                           bool covariance_form, T* __restrict__ sums,
-                                                           unsigned own_blocks, SortJob rider) {
+__device__ __forceinline__ void write_leaf(const T* __restrict__ mixture, T* __restrict__ box_lo, T* __restrict__ box_hi,
+                                           double threshold, int mode, bool covariance_form, T* __restrict__ node_box,
+                                           T* __restrict__ leaf_rec, int* __restrict__ parent, T* __restrict__ sums, int M,
+                                           size_t bl, int leaf, int comp, T (&blo)[D], T (&bhi)[D]) {
     constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
     constexpr int NS = 1 + D + D * (D + 1) / 2;
-    // The sort of the query points does not depend on the trees: a pass of it rides behind this kernel's own
-    // workgroups, on compute units that would idle otherwise, instead of lengthening a pass of the leaves' sort.
-    if (blockIdx.x >= own_blocks) { radix_scatter_pass(rider, blockIdx.x - own_blocks); return; }
-    // The records of the leaves and the internal nodes of the tree do not depend on each other, and both are
-    // short chains of dependent memory reads: the first half of the grid writes the records, the second half
-    // builds the nodes, side by side on different compute units.
-    const unsigned half = own_blocks / 2;
-    const bool tree_job = blockIdx.x >= half;
-    const size_t i = size_t(tree_job ? blockIdx.x - half : blockIdx.x) * kBlock + threadIdx.x;
-    if (i >= total) return;
-    const size_t bl = i / M;
-    const int leaf = int(i - bl * M);
-    if (tree_job) {
-        // lane <-> internal node `leaf` of its mixture (there are M-1 of them)
-        if (leaf < M - 1) build_internal_node(keys, children, parent, node_range, M, bl, leaf);
-        return;
-    }
+    const size_t i = bl * M + leaf;
     // the per-Gaussian sums of the backward pass start from zero (and return to zero after every backward pass)
     for (int k = 0; k < NS; ++k) sums[i * NS + k] = T(0);
-    int comp = int(order[i]);
     comp = (comp >= 0 && comp < M) ? comp : 0;      // a permutation by construction; never index out of bounds
     const size_t gi = bl * M + comp;
     const size_t node = bl * (2 * size_t(M) - 1) + (M - 1) + leaf;
     const T* g = mixture + gi * G;
-    // cutoff box of the Gaussian (lbvh/bvh.cu:164-231), kept in component order too (gmc_bvh_export_boxes)
-    T blo[D], bhi[D];
     {
         double delta[D];
         box_half_extent<T, D>(g, threshold, mode, covariance_form, delta);
@@ -698,11 +693,6 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
     for (int d = 0; d < D; ++d) {
         node_box[node * 2 * D + d] = blo[d];
         node_box[node * 2 * D + D + d] = bhi[d];
-    }
-    if (leaf < M - 1) {
-        // empty box of internal node `leaf`: lower = +inf, upper = -inf in the ordered-integer encoding
-        long long* e = enc_box + (bl * (M - 1) + leaf) * 2 * D;
-        for (int d = 0; d < D; ++d) { e[d] = ordered_bits(double(INFINITY)); e[D + d] = ordered_bits(double(-INFINITY)); }
     }
     if (M == 1) parent[node] = -1;                  // a single leaf is its own root
     T* r = leaf_rec + i * RS;
@@ -725,6 +715,63 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         r[9] = T(double(g[0]) * Kappa<3>::v * sqrt(det));
         reinterpret_cast<int*>(r + 10)[0] = comp;
     }
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
+                                                           T* __restrict__ box_hi, double threshold, int mode,
+                                                           const uint32_t* __restrict__ order,
+                                                           const uint32_t* __restrict__ keys, T* __restrict__ node_box,
+                                                           T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
+                                                           int2* __restrict__ children, int* __restrict__ parent,
+                                                           int2* __restrict__ node_range, int M, size_t total,
+                                                           bool covariance_form, T* __restrict__ sums,
+                                                           unsigned own_blocks, SortJob rider) {
+    // The sort of the query points does not depend on the trees: a pass of it rides behind this kernel's own
+    // workgroups, on compute units that would idle otherwise, instead of lengthening a pass of the leaves' sort.
+    if (blockIdx.x >= own_blocks) { radix_scatter_pass(rider, blockIdx.x - own_blocks); return; }
+    // The records of the leaves and the internal nodes of the tree do not depend on each other, and both are
+    // short chains of dependent memory reads: the first half of the grid writes the records, the second half
+    // builds the nodes, side by side on different compute units.
+    const unsigned half = own_blocks / 2;
+    const bool tree_job = blockIdx.x >= half;
+    const size_t i = size_t(tree_job ? blockIdx.x - half : blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const size_t bl = i / M;
+    const int leaf = int(i - bl * M);
+    if (tree_job) {
+        // lane <-> internal node `leaf` of its mixture (there are M-1 of them)
+        if (leaf < M - 1) build_internal_node(keys, children, parent, node_range, M, bl, leaf);
+        return;
+    }
+    T blo[D], bhi[D];
+    write_leaf<T, D>(mixture, box_lo, box_hi, threshold, mode, covariance_form, node_box, leaf_rec, parent, sums, M, bl, leaf,
+                     int(order[i]), blo, bhi);
+    if (leaf < M - 1) {
+        // empty box of internal node `leaf`: lower = +inf, upper = -inf in the ordered-integer encoding
+        long long* e = enc_box + (bl * (M - 1) + leaf) * 2 * D;
+        for (int d = 0; d < D; ++d) { e[d] = ordered_bits(double(INFINITY)); e[D + d] = ordered_bits(double(-INFINITY)); }
+    }
+}
+
+// orders the LDS traffic of one wavefront: stores of some lanes before loads of other lanes
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_min(T v) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) { const T o = __shfl_xor(v, off, 64); v = o < v ? o : v; }
+    return v;
+}
+template <typename T>
+__device__ __forceinline__ T wave_max(T v) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) { const T o = __shfl_xor(v, off, 64); v = o > v ? o : v; }
+    return v;
 }
 
 // Where a descent starts.  The first levels below the root hold one, two, four ... nodes, and a descent spends a memory
@@ -870,6 +917,327 @@ __global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __r
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// small trees: the whole build in one launch
+// ---------------------------------------------------------------------------------------------------------------
+// The chain of launches above costs about ten launch latencies whatever the size of the trees.  Mixtures of at most
+// kSmallTreeMax components with at most kCoarseOrderMax query points per segment (the shapes of network layers:
+// hundreds of mixtures of 64 ... 128 components) are built by ONE launch instead: a workgroup (a single wavefront for
+// trees of at most 64 leaves) builds its tree entirely in LDS -- bounds of the centres, Morton codes, a bitonic sort of the unique keys (code << 32 | component: any
+// sorting network gives the stable order), leaf boxes and records, the radix tree, the bottom-up box unions with LDS
+// atomics, the decoded boxes (every node stores its own box with its parent), the cut below the root -- and the
+// workgroups behind the trees' Morton-order one segment of query points each (bounds, one stable counting pass over
+// the top 8 key bits).  Same trees and boxes as the chain of launches, bit for bit; the order of the points may differ
+// where a point lies on the border of a Morton cell (any order of the points gives the same sums).
+constexpr int kSmallTreeMax = 1024;
+
+template <typename T> struct SmallBuild {
+    T* box_lo; T* box_hi; T* node_box; T* child_box; T* leaf_rec; T* sums;
+    int2* children; int* parent; int2* node_range; int* leaf_comp; uint32_t* g_keys; int* frontier;
+    int* p_order; int* cand_count; int* ctl;
+    double threshold;
+    int mode, covariance_form, M, N, per_mixture /* 64-point groups per mixture */, sort_points;
+    unsigned tree_blocks;
+};
+
+template <typename T> struct OrderedInt;
+template <> struct OrderedInt<float> { using type = int; static constexpr int kEmptyLo = 0x7fffffff, kEmptyHi = -0x7fffffff - 1; };
+template <> struct OrderedInt<double> {
+    using type = long long;
+    static constexpr long long kEmptyLo = 0x7fffffffffffffffll, kEmptyHi = -0x7fffffffffffffffll - 1;
+};
+
+// Morton order of one segment of at most kCoarseOrderMax query points by the top 8 bits of their keys, stable.  Wavefront
+// w owns a contiguous quarter of the points: per-wavefront digit counts, one scan, then every wavefront places its
+// points round by round on its own (ranks inside a round from ballots), without workgroup barriers.
+struct SmallPointsLds {
+    uint32_t whist[4][256];
+    uint32_t wtotal[4];
+};
+
+// (PP: points per lane, at least N / 256; the points stay in registers between the two passes and all their loads are in
+// flight at once -- a loop that waits for every point's load would cost a memory round trip per 256 points)
+template <typename T, int D, int PP>
+__device__ __forceinline__ void order_points_small(const T* __restrict__ p, int N, int* __restrict__ order, T (*red)[kBlock],
+                                                   SmallPointsLds& s) {
+    uint32_t (*whist)[256] = s.whist;
+    uint32_t* wtotal = s.wtotal;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int share = (N + kBlock - 1) / kBlock * kWave;
+    const int begin = wave * share, end = begin + share < N ? begin + share : N;
+    T x[PP][D];
+#pragma unroll
+    for (int r = 0; r < PP; ++r) {
+        const int i = begin + r * kWave + lane;
+#pragma unroll
+        for (int d = 0; d < D; ++d) x[r][d] = i < end ? p[size_t(i) * D + d] : T(0);
+    }
+    T lo[D], hi[D];
+    for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
+#pragma unroll
+    for (int r = 0; r < PP; ++r)
+        if (begin + r * kWave + lane < end)
+            for (int d = 0; d < D; ++d) {
+                lo[d] = x[r][d] < lo[d] ? x[r][d] : lo[d];
+                hi[d] = x[r][d] > hi[d] ? x[r][d] : hi[d];
+            }
+    for (int w = 0; w < 4; ++w) whist[w][threadIdx.x] = 0u;
+    block_bounds<T, D>(lo, hi, red);
+    // The top 8 bits of the 30-bit key, i.e. bits 9, 8 (and 7 of the first two axes) of the 10-bit cell coordinates.  The
+    // order of the points only groups neighbours: the cell is formed with one reciprocal per axis instead of a division
+    // per coordinate (a point on a cell border may land in the neighbouring cell, which is as good a group).
+    T base[D], scale[D];
+    for (int d = 0; d < D; ++d) {
+        const T ext = red[D + d][0] - red[d][0];
+        base[d] = red[d][0];
+        scale[d] = ext > T(0) ? T(1024) / ext : T(0);
+    }
+    uint32_t digit[PP];
+#pragma unroll
+    for (int r = 0; r < PP; ++r) {
+        uint32_t cell[3] = {0u, 0u, 0u};
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            T q = (x[r][d] - base[d]) * scale[d];
+            q = q < T(0) ? T(0) : (q > T(1023) ? T(1023) : q);
+            q = (q == q) ? q : T(0);
+            cell[d] = uint32_t(q);
+        }
+        digit[r] = ((cell[0] >> 9) & 1u) << 7 | ((cell[1] >> 9) & 1u) << 6 | ((cell[2] >> 9) & 1u) << 5 |
+                   ((cell[0] >> 8) & 1u) << 4 | ((cell[1] >> 8) & 1u) << 3 | ((cell[2] >> 8) & 1u) << 2 |
+                   ((cell[0] >> 7) & 1u) << 1 | ((cell[1] >> 7) & 1u);
+        if (begin + r * kWave + lane < end) atomicAdd(&whist[wave][digit[r]], 1u);
+    }
+    __syncthreads();
+    {   // thread d: first slot of digit d for every wavefront
+        uint32_t c[4], mine = 0;
+        for (int w = 0; w < 4; ++w) { c[w] = whist[w][threadIdx.x]; mine += c[w]; }
+        uint32_t scan = mine;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const uint32_t up = __shfl_up(scan, off, kWave);
+            scan += lane >= off ? up : 0u;
+        }
+        if (lane == kWave - 1) wtotal[wave] = scan;
+        __syncthreads();
+        for (int w = 0; w < wave; ++w) scan += wtotal[w];
+        uint32_t at = scan - mine;
+        for (int w = 0; w < 4; ++w) { whist[w][threadIdx.x] = at; at += c[w]; }
+    }
+    __syncthreads();
+    const unsigned long long below = (1ull << lane) - 1ull;
+#pragma unroll
+    for (int r = 0; r < PP; ++r) {
+        if (begin + r * kWave >= end) break;                // (wave-uniform)
+        const int i = begin + r * kWave + lane;
+        const bool valid = i < end;
+        const uint32_t dg = valid ? digit[r] : 0u;
+        unsigned long long same = __ballot(valid);
+#pragma unroll
+        for (int bit = 0; bit < 8; ++bit) {
+            const unsigned long long m = __ballot((dg >> bit) & 1u);
+            same &= ((dg >> bit) & 1u) ? m : ~m;
+        }
+        const int rank = __popcll(same & below);
+        uint32_t slot = 0;
+        if (valid) slot = whist[wave][dg] + rank;
+        wave_lds_fence();
+        if (valid) {
+            if (slot < uint32_t(N)) order[slot] = i;        // always true for consistent counts
+            if (rank == 0) whist[wave][dg] = slot + uint32_t(__popcll(same));
+        }
+        wave_lds_fence();
+    }
+}
+
+// LDS of one tree that THREADS lanes build, K leaves per lane
+template <typename T, int D, int THREADS, int K> struct SmallTreeLds {
+    static constexpr int kCap = THREADS * K;
+    using Enc = typename OrderedInt<T>::type;
+    unsigned long long keys[kCap];              // code << 32 | component, sorted in place
+    int parent[2 * kCap];                       // [0, M-1): internal nodes, [M-1, 2M-1): leaves
+    int2 kids[kCap];
+    Enc box[kCap][2 * D];                       // boxes of the internal nodes, order-preserving integers
+};
+
+// The lanes that build one tree wait for each other: a wavefront (its LDS traffic ordered) or the workgroup.  (Trees of
+// 128 lanes share a workgroup in pairs and go through the same barriers side by side: every tree of a launch has the
+// same number of leaves, and the loops whose length depends on the data hold no barrier.)
+template <int THREADS> __device__ __forceinline__ void tree_sync() {
+    if constexpr (THREADS == kWave) wave_lds_fence(); else __syncthreads();
+}
+
+// Tree bl by THREADS lanes (tid = 0 ... THREADS-1): one wavefront (trees of at most 64 leaves: four trees per
+// workgroup, no workgroup barriers) or the whole workgroup.
+template <typename T, int D, int THREADS, int K>
+__device__ __forceinline__ void build_small_tree(const T* __restrict__ mixture, const SmallBuild<T>& a, size_t bl, int tid,
+                                                 SmallTreeLds<T, D, THREADS, K>& s, T (*red)[kBlock]) {
+    constexpr int G = 1 + D + D * D;
+    using Enc = typename OrderedInt<T>::type;
+    const int M = a.M;
+    // a new tree: no candidate list is known yet
+    if (a.cand_count)
+        for (int g = tid; g < a.per_mixture; g += THREADS) a.cand_count[bl * a.per_mixture + g] = -1;
+    // bounds of the centres and keys
+    T c[K][D], bounds[2 * D];
+    {
+        T lo[D], hi[D];
+        for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const int i = tid + k * THREADS;
+            for (int d = 0; d < D; ++d) {
+                c[k][d] = i < M ? mixture[(bl * M + i) * G + 1 + d] : T(0);
+                if (i < M) {
+                    lo[d] = c[k][d] < lo[d] ? c[k][d] : lo[d];       // a NaN coordinate is skipped
+                    hi[d] = c[k][d] > hi[d] ? c[k][d] : hi[d];
+                }
+            }
+        }
+        for (int d = 0; d < D; ++d) { bounds[d] = wave_min(lo[d]); bounds[D + d] = wave_max(hi[d]); }
+        if constexpr (THREADS > kWave) {                    // combine the wavefronts of this tree
+            const int wave = threadIdx.x >> 6, first = (threadIdx.x / THREADS) * (THREADS / kWave);
+            T mine = bounds[0];
+            for (int k = 1; k < 2 * D; ++k) mine = int(threadIdx.x & 63) == k ? bounds[k] : mine;
+            if ((threadIdx.x & 63) < 2 * D) red[threadIdx.x & 63][wave] = mine;
+            __syncthreads();
+            for (int k = 0; k < 2 * D; ++k) bounds[k] = red[k][first];
+            for (int w = 1; w < THREADS / kWave; ++w)
+                for (int d = 0; d < D; ++d) {
+                    const T a = red[d][first + w], b = red[D + d][first + w];
+                    bounds[d] = a < bounds[d] ? a : bounds[d];
+                    bounds[D + d] = b > bounds[D + d] ? b : bounds[D + d];
+                }
+        }
+    }
+    int Mp = 1;
+    while (Mp < M) Mp <<= 1;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int i = tid + k * THREADS;
+        if (i < Mp) s.keys[i] = i < M ? ((unsigned long long)morton30<T, D>(c[k], bounds) << 32) | (unsigned)i : ~0ull;
+    }
+    tree_sync<THREADS>();
+    // bitonic sort of the unique keys
+    for (int size = 2; size <= Mp; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int q = tid; q < Mp / 2; q += THREADS) {
+                const int i0 = ((q & ~(stride - 1)) << 1) | (q & (stride - 1)), i1 = i0 | stride;
+                const unsigned long long k0 = s.keys[i0], k1 = s.keys[i1];
+                if ((k0 > k1) == ((i0 & size) == 0)) { s.keys[i0] = k1; s.keys[i1] = k0; }
+            }
+            tree_sync<THREADS>();
+        }
+    // leaves: lane <-> leaf i (Morton order) and, below, internal node i
+    T blo[K][D], bhi[K][D];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int i = tid + k * THREADS;
+        if (i < M) {
+            const unsigned long long key = s.keys[i];
+            const int comp = int(unsigned(key));
+            a.g_keys[bl * M + i] = uint32_t(key >> 32);
+            a.leaf_comp[bl * M + i] = comp;
+            write_leaf<T, D>(mixture, a.box_lo, a.box_hi, a.threshold, a.mode, a.covariance_form != 0, a.node_box, a.leaf_rec,
+                             a.parent, a.sums, M, bl, i, comp, blo[k], bhi[k]);
+        }
+    }
+    if (M < 2) return;
+    int* par = a.parent + bl * (2 * size_t(M) - 1);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int i = tid + k * THREADS;
+        if (i < M - 1) {
+            int first, last, left, right;
+            radix_tree_node([&](int j) { return uint32_t(s.keys[j] >> 32); }, M, i, first, last, left, right);
+            a.children[bl * (M - 1) + i] = make_int2(left, right);
+            a.node_range[bl * (M - 1) + i] = make_int2(first, last);
+            s.kids[i] = make_int2(left, right);
+            const int li = left >= 0 ? left : (M - 1) + ~left, ri = right >= 0 ? right : (M - 1) + ~right;
+            par[li] = i; par[ri] = i;
+            s.parent[li] = i; s.parent[ri] = i;
+            if (i == 0) { par[0] = -1; s.parent[0] = -1; }
+            for (int d = 0; d < D; ++d) { s.box[i][d] = OrderedInt<T>::kEmptyLo; s.box[i][D + d] = OrderedInt<T>::kEmptyHi; }
+        }
+    }
+    tree_sync<THREADS>();
+    // bottom-up unions: every leaf merges its own box into its ancestors until one already contains it (see bvh_merge_kernel)
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int i = tid + k * THREADS;
+        if (i < M) {
+            Enc lo[D], hi[D];
+            for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(blo[k][d]); hi[d] = ordered_bits(bhi[k][d]); }
+            int node = s.parent[(M - 1) + i];
+            for (int level = 0; node >= 0 && node < M - 1 && level < 128; ++level) {
+                bool grew = false;
+                for (int d = 0; d < D; ++d) {
+                    grew |= lo[d] < atomicMin(&s.box[node][d], lo[d]);
+                    grew |= hi[d] > atomicMax(&s.box[node][D + d], hi[d]);
+                }
+                if (!grew) break;
+                node = s.parent[node];
+            }
+        }
+    }
+    tree_sync<THREADS>();
+    // every node stores its box with its parent (child_box) and, internal nodes, as its own node box
+    const size_t nbase = bl * (2 * size_t(M) - 1);
+    T* cb = a.child_box + bl * (M - 1) * 4 * D;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int i = tid + k * THREADS;
+        if (i < M - 1) {
+            T v[2 * D];
+            for (int d = 0; d < 2 * D; ++d) v[d] = from_ordered_bits(s.box[i][d]);
+            for (int d = 0; d < 2 * D; ++d) a.node_box[(nbase + i) * 2 * D + d] = v[d];
+            const int up = s.parent[i];
+            if (up >= 0 && up < M - 1) {
+                const int side = s.kids[up].x == i ? 0 : 1;
+                for (int d = 0; d < 2 * D; ++d) cb[(size_t(up) * 2 + side) * 2 * D + d] = v[d];
+            }
+        }
+        if (i < M) {
+            const int up = s.parent[(M - 1) + i];
+            if (up >= 0 && up < M - 1) {
+                const int side = s.kids[up].x == ~i ? 0 : 1;
+                for (int d = 0; d < D; ++d) {
+                    cb[(size_t(up) * 2 + side) * 2 * D + d] = blo[k][d];
+                    cb[(size_t(up) * 2 + side) * 2 * D + D + d] = bhi[k][d];
+                }
+            }
+        }
+    }
+    if (tid < kWave) tree_frontier(s.kids, M, a.frontier + bl * (1 + kFrontier), tid);
+}
+
+template <typename T, int D, int THREADS, int K, int PP>
+__global__ __launch_bounds__(kBlock) void bvh_build_small_kernel(const T* __restrict__ mixture, const T* __restrict__ xes,
+                                                                SmallBuild<T> a, size_t mixtures) {
+    using Trees = SmallTreeLds<T, D, THREADS, K>[kBlock / THREADS];
+    __shared__ T red[2 * D][kBlock];
+    // a workgroup builds trees or orders points: one piece of LDS for either
+    __shared__ __attribute__((aligned(16))) unsigned char lds[sizeof(Trees) > sizeof(SmallPointsLds) ? sizeof(Trees) : sizeof(SmallPointsLds)];
+    Trees& trees = *reinterpret_cast<Trees*>(lds);
+    if (blockIdx.x == 0 && threadIdx.x < 4) a.ctl[threadIdx.x] = 0;     // a new tree: no published pieces, no error
+    if (blockIdx.x >= a.tree_blocks) {
+        const size_t seg = blockIdx.x - a.tree_blocks;
+        const int N = a.N;
+        int* order = a.p_order + seg * N;
+        if (!a.sort_points) { for (int i = threadIdx.x; i < N; i += kBlock) order[i] = i; return; }
+        order_points_small<T, D, PP>(xes + seg * N * D, N, order, red, *reinterpret_cast<SmallPointsLds*>(lds));
+        return;
+    }
+    const int sub = threadIdx.x / THREADS;                  // trees of THREADS lanes: kBlock / THREADS of them per workgroup
+    size_t bl = size_t(blockIdx.x) * (kBlock / THREADS) + sub;
+    if constexpr (THREADS == kWave) {
+        if (bl >= mixtures) return;                         // (a wavefront on its own: no barriers ahead)
+    } else {
+        bl = bl < mixtures ? bl : mixtures - 1;             // a spare half builds the last tree once more: same values, same barriers
+    }
+    build_small_tree<T, D, THREADS, K>(mixture, a, bl, threadIdx.x % THREADS, trees[sub], red);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // traversal
 // ---------------------------------------------------------------------------------------------------------------
 // closed-interval test of a point against a box given as (lower[D], upper[D]); every comparison is evaluated
@@ -935,26 +1303,6 @@ __device__ __forceinline__ unsigned long long points_stamp(const T (&x)[D], bool
     // the same value in every lane: kept in scalar registers (it stays alive until the list is published)
     const unsigned lo = __builtin_amdgcn_readfirstlane(unsigned(h)), hi = __builtin_amdgcn_readfirstlane(unsigned(h >> 32));
     return ((unsigned long long)hi << 32) | lo;
-}
-
-template <typename T>
-__device__ __forceinline__ T wave_min(T v) {
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) { const T o = __shfl_xor(v, off, 64); v = o < v ? o : v; }
-    return v;
-}
-template <typename T>
-__device__ __forceinline__ T wave_max(T v) {
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) { const T o = __shfl_xor(v, off, 64); v = o > v ? o : v; }
-    return v;
-}
-
-// orders the LDS traffic of one wavefront: stores of some lanes before loads of other lanes
-__device__ __forceinline__ void wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Largest float not above / smallest float not below a coordinate: boxes rounded outwards stay conservative.
@@ -1754,6 +2102,30 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     int* p_order = (int*)(bvh + lay.p_order);
     const bool have_g = BL > 0 && M > 0, have_p = XL > 0 && N > 0;
     const bool sort_p = have_p && xes != nullptr;
+    if (have_g && M <= kSmallTreeMax && (!sort_p || N <= kCoarseOrderMax) && BL + XL < (size_t(1) << 31)) {
+        const CandidateCache cache = candidate_cache(bvh, lay);
+        SmallBuild<T> a{box_lo, box_hi, node_box, child_box, leaf_rec, (T*)(bvh + lay.sums), children, parent, node_range,
+                        leaf_comp, g_keys, (int*)(bvh + lay.frontier), p_order, cache.count, (int*)(bvh + lay.cand_ctl),
+                        double(cfg.aabb_threshold), cfg.aabb_mode, cfg.covariance_form != 0 ? 1 : 0, M, N,
+                        (N + kWave - 1) / kWave, sort_p ? 1 : 0, 0u};
+        // trees of at most 64 leaves: one wavefront each, four per workgroup; of at most 128: two wavefronts each, two per
+        // workgroup (no idle vector units while the leaves are written: the double arithmetic of a leaf's box and record is
+        // the longest part of the chain); larger ones: one workgroup each, with one, two or four leaves per lane
+        const int lanes = M <= kWave ? kWave : M <= 2 * kWave ? 2 * kWave : kBlock;      // lanes per tree
+        a.tree_blocks = unsigned((BL + kBlock / lanes - 1) / (kBlock / lanes));
+        const dim3 grid(a.tree_blocks + unsigned(have_p ? XL : 0));
+        const int pp = !sort_p || N <= 4 * kBlock ? 4 : N <= 16 * kBlock ? 16 : 32;
+#define GMC_SMALL(THREADS, K, PP) bvh_build_small_kernel<T, D, THREADS, K, PP><<<grid, dim3(kBlock), 0, st>>>(mixture, xes, a, BL)
+#define GMC_SMALL_PP(THREADS, K) do { if (pp == 4) GMC_SMALL(THREADS, K, 4); else if (pp == 16) GMC_SMALL(THREADS, K, 16); else GMC_SMALL(THREADS, K, 32); } while (0)
+        if (lanes == kWave) GMC_SMALL_PP(kWave, 1);
+        else if (lanes == 2 * kWave) GMC_SMALL_PP(2 * kWave, 1);
+        else if (M <= kBlock) GMC_SMALL_PP(kBlock, 1);
+        else if (M <= 2 * kBlock) GMC_SMALL_PP(kBlock, 2);
+        else GMC_SMALL_PP(kBlock, 4);
+#undef GMC_SMALL_PP
+#undef GMC_SMALL
+        return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+    }
     const int bpm = (M + kBlock - 1) / kBlock;               // workgroups per mixture (boxes, keys)
     const int nbp = (N + kBoundsChunk - 1) / kBoundsChunk;   // partial bounds per point segment
     const int bpx = (N + kBlock - 1) / kBlock;               // workgroups per point segment (keys)
