@@ -801,17 +801,17 @@ __device__ __forceinline__ void tree_frontier(const int2* __restrict__ kids, int
     if (lane < n) out[1 + lane] = cur[lane];
 }
 
-// Bottom-up boxes without inter-lane ordering: one lane per leaf walks towards the root and merges ITS OWN leaf
-// box into every ancestor with atomic min/max, as long as it still enlarges the ancestor; it stops at the first
-// ancestor that already contains it.  Every extreme of that ancestor was set by some leaf that enlarged it and
-// therefore walks on itself, so all higher ancestors end up containing the stopped leaf as well: the final boxes
-// are the exact unions of the leaves below each node.  Nothing is read back except the atomics' own return
-// values, so no fences are needed; the decoded boxes are produced by the next kernel.
+// Bottom-up boxes without inter-lane ordering: a walker goes towards the root and merges ITS OWN box into every
+// ancestor with atomic min/max, as long as it still enlarges the ancestor; it stops at the first ancestor that
+// already contains it.  Every extreme of that ancestor was set by some walker that enlarged it and therefore walks
+// on itself, so all higher ancestors end up containing the stopped box as well: the final boxes are the exact unions
+// of the leaves below each node.  Nothing is read back except the atomics' own return values, so no fences are
+// needed; the decoded boxes are produced by the next kernel.
 // A walk is a chain of atomic round trips, one per tree level.  The lower levels stay inside the workgroup: an
 // internal node whose leaves all belong to the kMergeBlock leaves of this workgroup is touched by these lanes only, so its
-// box lives in LDS while the walks run (internal node i lies inside its own leaf range, hence slot i - first leaf
-// of the workgroup is free for it) and is stored once at the end; only the ancestors that reach beyond the
-// workgroup's leaves are merged with global atomics.
+// box lives in LDS while the leaves walk (internal node i lies inside its own leaf range, hence slot i - first leaf
+// of the workgroup is free for it) and is stored once at the end.  The ancestors that reach beyond the workgroup's
+// leaves are merged with global atomics by the roots of the local subtrees alone, with their finished boxes.
 // leaves per workgroup of the box merge (1024 keep two more tree levels in LDS but occupy too few compute units: slower)
 constexpr int kMergeBlock = 256;
 
@@ -850,34 +850,56 @@ __global__ __launch_bounds__(kMergeBlock) void bvh_merge_kernel(const int* __res
         local_box[threadIdx.x][D + d] = -0x7fffffffffffffffll - 1;
     }
     __syncthreads();
-    if (t < total) {
-        const T* box = node_box + (nbase + (M - 1) + leaf) * 2 * D;
-        long long* enc = enc_box + bl * (M - 1) * 2 * D;
-        long long lo[D], hi[D];
-        for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(double(box[d])); hi[d] = ordered_bits(double(box[D + d])); }
-        int node = parent[nbase + (M - 1) + leaf];
+    // Two phases.  First every leaf walks through its local ancestors only (LDS atomics).  Then the roots of the local
+    // subtrees -- local internal nodes and leaves whose parent reaches beyond the workgroup, a dozen or two per
+    // workgroup -- walk on through the global ancestors with the finished box of their subtree: a few global atomics
+    // per workgroup and tree level instead of one per leaf on the same few addresses.
+    auto is_local_node = [&](int node) -> bool {
+        const long long slot = (long long)(bl * M + node) - (long long)first_leaf;
+        return slot >= 0 && slot < kMergeBlock && is_local[slot];
+    };
+    long long* enc = enc_box + bl * (M - 1) * 2 * D;
+    // walk from `node` upwards through global ancestors with the box (lo, hi)
+    auto global_walk = [&](int node, const long long (&lo)[D], const long long (&hi)[D]) {
         // the radix tree over 64-bit keys is at most 64 levels deep; the bound also ends a walk on a malformed chain
         for (int level = 0; node >= 0 && node < M - 1 && level < 128; ++level) {
-            const long long slot = (long long)(bl * M + node) - (long long)first_leaf;
-            const bool local = slot >= 0 && slot < kMergeBlock && is_local[slot];
+            const int up = parent[nbase + node];            // fetched alongside the atomics: one round trip per level
+            long long* e = enc + size_t(node) * 2 * D;
             bool grew = false;
-            int up;
-            if (local) {
-                up = local_parent[slot];
-                for (int d = 0; d < D; ++d) {
-                    grew |= lo[d] < atomicMin(&local_box[slot][d], lo[d]);
-                    grew |= hi[d] > atomicMax(&local_box[slot][D + d], hi[d]);
-                }
-            } else {
-                up = parent[nbase + node];          // fetched alongside the atomics: one round trip per level
-                long long* e = enc + size_t(node) * 2 * D;
-                for (int d = 0; d < D; ++d) {
-                    grew |= lo[d] < atomicMin(&e[d], lo[d]);
-                    grew |= hi[d] > atomicMax(&e[D + d], hi[d]);
-                }
+            for (int d = 0; d < D; ++d) {
+                grew |= lo[d] < atomicMin(&e[d], lo[d]);
+                grew |= hi[d] > atomicMax(&e[D + d], hi[d]);
             }
             if (!grew) break;
             node = up;
+        }
+    };
+    long long leaf_lo[D], leaf_hi[D];
+    int leaf_exit = -1;                                     // the first ancestor of this leaf that is not local
+    if (t < total) {
+        const T* box = node_box + (nbase + (M - 1) + leaf) * 2 * D;
+        for (int d = 0; d < D; ++d) { leaf_lo[d] = ordered_bits(double(box[d])); leaf_hi[d] = ordered_bits(double(box[D + d])); }
+        int node = parent[nbase + (M - 1) + leaf];
+        if (node >= 0 && node < M - 1 && !is_local_node(node)) leaf_exit = node;
+        for (int level = 0; node >= 0 && node < M - 1 && level < 128 && is_local_node(node); ++level) {
+            const int slot = int((long long)(bl * M + node) - (long long)first_leaf);
+            bool grew = false;
+            for (int d = 0; d < D; ++d) {
+                grew |= leaf_lo[d] < atomicMin(&local_box[slot][d], leaf_lo[d]);
+                grew |= leaf_hi[d] > atomicMax(&local_box[slot][D + d], leaf_hi[d]);
+            }
+            if (!grew) break;
+            node = local_parent[slot];
+        }
+    }
+    __syncthreads();
+    if (leaf_exit >= 0) global_walk(leaf_exit, leaf_lo, leaf_hi);
+    if (mine) {
+        const int up = local_parent[threadIdx.x];
+        if (up >= 0 && up < M - 1 && !is_local_node(up)) {
+            long long lo[D], hi[D];
+            for (int d = 0; d < D; ++d) { lo[d] = local_box[threadIdx.x][d]; hi[d] = local_box[threadIdx.x][D + d]; }
+            global_walk(up, lo, hi);
         }
     }
     __syncthreads();
