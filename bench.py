@@ -149,6 +149,31 @@ def measure_bvh(aabb_mode: str, steps: int, warmup: int, copy_calibration: bool 
         step(events[k])
     torch.cuda.synchronize()
     build_ms, fwd_ms, bwd_ms = (median([e[i].elapsed_time(e[i + 1]) for e in events]) for i in range(3))
+    # ... and without the host between the launches: ten builds, and ten whole steps, captured into HIP graphs and
+    # replayed (the build of small trees is one launch of about 20 us, shorter than the host needs to enqueue it, so
+    # the event pair above measures the host there)
+    def in_graph(fn, repeats=10, replays=5):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            keep = [fn() for _ in range(repeats)]
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(replays):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        del keep
+        return e0.elapsed_time(e1) / (repeats * replays)
+    build_graph_ms = in_graph(lambda: _native.Bvh(mix, xes, 0.001, aabb_mode))
+    step_graph_ms = in_graph(step)
     # pairs actually evaluated: points inside the cutoff box of a Gaussian (counted outside the timed region)
     bvh = _native.Bvh(mix, xes, 0.001, aabb_mode)
     lo, up = bvh.boxes()
@@ -157,14 +182,16 @@ def measure_bvh(aabb_mode: str, steps: int, warmup: int, copy_calibration: bool 
         for n0 in range(0, wl.N, 2048):
             x = xes[b, :, n0:n0 + 2048].unsqueeze(2)                   # [L, n, 1, D]
             hits += int(((x >= lo[b].unsqueeze(1)) & (x <= up[b].unsqueeze(1))).all(dim=-1).sum().item())
-    return {"wl": wl, "ms_step": wall * 1e3 / steps, "build_ms": build_ms, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "hits": hits}
+    return {"wl": wl, "ms_step": wall * 1e3 / steps, "build_ms": build_ms, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms, "hits": hits,
+            "build_graph_ms": build_graph_ms, "step_graph_ms": step_graph_ms}
 
 
 def bvh_summary(r, aabb_mode):
     """the C5 numbers of one box rule as a compact object (entry of `other_workloads`)"""
     wl = r["wl"]
     return {"aabb_mode": aabb_mode, "ms_per_step": r["ms_step"], "build_ms": r["build_ms"], "fwd_ms": r["fwd_ms"],
-            "bwd_ms": r["bwd_ms"], "dense_equivalent_pairs_per_s": wl.pairs / (r["ms_step"] * 1e-3),
+            "bwd_ms": r["bwd_ms"], "build_ms_in_graph": r["build_graph_ms"], "ms_per_step_in_graph": r["step_graph_ms"],
+            "dense_equivalent_pairs_per_s": wl.pairs / (r["ms_step"] * 1e-3),
             "evaluated_pairs": r["hits"], "evaluated_pairs_per_s": r["hits"] / (r["ms_step"] * 1e-3)}
 
 
@@ -172,36 +199,40 @@ def bench_bvh(args):
     """`--workload C5`: the LBVH-culled step (build + forward + backward).  Throughput is reported in dense-equivalent
     pairs (B L M N per step); the roofline entries are against HBM with the compulsory bytes of the pass (Gaussians,
     node boxes and links, points in, values and gradients out)."""
-    r = measure_bvh(args.aabb_mode, args.steps, args.warmup, args.copy_calibration)
+    r = measure_bvh(args.aabb_mode, args.steps, args.warmup, args.copy_calibration, name=args.workload)
     wl, ms_step, build_ms, fwd_ms, bwd_ms, hits = r["wl"], r["ms_step"], r["build_ms"], r["fwd_ms"], r["bwd_ms"], r["hits"]
-    s, M, N, D = 8, wl.M, wl.N, 3
-    bytes_fwd = M * 13 * s + (2 * M - 1) * (2 * D * s + 8) + N * (D + 1) * s
-    bytes_bwd = bytes_fwd + N * s + M * 13 * s + N * D * s
+    import torch
+    s, M, N, D, BL = (8 if wl.dtype == torch.float64 else 4), wl.M, wl.N, wl.dims, wl.B * wl.L
+    G = 1 + D + D * D
+    bytes_fwd = BL * (M * G * s + (2 * M - 1) * (2 * D * s + 8) + N * (D + 1) * s)
+    bytes_bwd = bytes_fwd + BL * (N * s + M * G * s + N * D * s)
+    dt = "f64" if s == 8 else "f32"
     reference_rule = args.aabb_mode == "reference"
     line = {
         "metric": "Gaussian-point evals/sec fwd and fwd+bwd at 1 GPU; % of FP32 VALU peak",
         "value": wl.pairs / (ms_step * 1e-3), "unit": "dense-equivalent Gaussian-point pairs/s (LBVH build + forward + backward step)",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
-        "config": {"workload": f"C5: D=3 f64 B=1 L=1 M={M} N={N}, LBVH-culled (aabb_mode={args.aabb_mode}, "
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dt, "data": "synthetic",
+        "config": {"workload": f"{args.workload}: D={D} {dt} B={wl.B} L={wl.L} M={M} N={N}, LBVH-culled (aabb_mode={args.aabb_mode}, "
                                f"threshold 0.001), {wl.pairs:.4g} dense-equivalent pairs per step"},
         "build_ms": build_ms, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+        "build_ms_in_graph": r["build_graph_ms"], "ms_per_step_in_graph": r["step_graph_ms"],
         "evaluated_pairs": hits, "evaluated_pairs_per_s": hits / (ms_step * 1e-3),
         "evaluated_fraction_of_dense": hits / wl.pairs,
         "roofline": {"kernel": "bvh_traverse_kernel (backward mode; event pair also holds its zero-fill and epilogue)",
                      "bound": "hbm", "achieved": bytes_bwd / (bwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
                      "frac": bytes_bwd / (bwd_ms * 1e-3) / 8e12,
-                     "traffic": profile_traffic("C5", "bvh_traverse_kernel<double, 3, 1") if reference_rule else None,
+                     "traffic": profile_traffic("C5", "bvh_traverse_kernel<double, 3, 1") if reference_rule and args.workload == "C5" else None,
                      "launch_ms": bwd_ms, "algorithmic_bytes": bytes_bwd,
                      "bound_detail": "latency-bound: dependent tree-node fetches and double-precision leaf "
                                      "evaluation; the tree (about 4 MB) is fetched once per XCD (8 L2 caches)"},
         "roofline_fwd": {"kernel": "bvh_traverse_kernel (forward mode)", "bound": "hbm",
                          "achieved": bytes_fwd / (fwd_ms * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
                          "frac": bytes_fwd / (fwd_ms * 1e-3) / 8e12,
-                         "traffic": profile_traffic("C5", "bvh_traverse_kernel<double, 3, 0") if reference_rule else None,
+                         "traffic": profile_traffic("C5", "bvh_traverse_kernel<double, 3, 0") if reference_rule and args.workload == "C5" else None,
                          "launch_ms": fwd_ms, "algorithmic_bytes": bytes_fwd},
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.workload == "C5":
         line["cpu_baseline"] = cpu_baseline_bvh(args.aabb_mode)
     print(json.dumps(line))
 
@@ -490,6 +521,8 @@ def main():
                          "backward per step); layer: gm.evaluate on covariances forward + backward, the ReLU fixed-point "
                          "fitting and BatchNorm on the C2 shape")
     ap.add_argument("--aabb-mode", default="reference", choices=["reference", "tight"])
+    ap.add_argument("--culled", action="store_true",
+                    help="C2 or C3 through the LBVH-culled path (build + forward + backward per step), like C5")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="C4 only: leave out the `other_workloads` object (C1, C2, C3 and C5 measured after C4)")
@@ -505,7 +538,7 @@ def main():
     import torch
     from gmc import _native, synthetic
 
-    if args.workload == "C5":
+    if args.workload == "C5" or (args.culled and args.workload in ("C2", "C3")):
         return bench_bvh(args)
     if args.workload == "conv":
         return bench_convolution(args)

@@ -951,6 +951,7 @@ __global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __r
 // the top 8 key bits).  Same trees and boxes as the chain of launches, bit for bit; the order of the points may differ
 // where a point lies on the border of a Morton cell (any order of the points gives the same sums).
 constexpr int kSmallTreeMax = 1024;
+static int g_build_path = 0;            // test knob (gmc_bvh_set_build_path): 1 = always the chain of launches
 
 template <typename T> struct SmallBuild {
     T* box_lo; T* box_hi; T* node_box; T* child_box; T* leaf_rec; T* sums;
@@ -2124,7 +2125,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     int* p_order = (int*)(bvh + lay.p_order);
     const bool have_g = BL > 0 && M > 0, have_p = XL > 0 && N > 0;
     const bool sort_p = have_p && xes != nullptr;
-    if (have_g && M <= kSmallTreeMax && (!sort_p || N <= kCoarseOrderMax) && BL + XL < (size_t(1) << 31)) {
+    if (g_build_path != 1 && have_g && M <= kSmallTreeMax && (!sort_p || N <= kCoarseOrderMax) && BL + XL < (size_t(1) << 31)) {
         const CandidateCache cache = candidate_cache(bvh, lay);
         SmallBuild<T> a{box_lo, box_hi, node_box, child_box, leaf_rec, (T*)(bvh + lay.sums), children, parent, node_range,
                         leaf_comp, g_keys, (int*)(bvh + lay.frontier), p_order, cache.count, (int*)(bvh + lay.cand_ctl),
@@ -2327,6 +2328,8 @@ static int bvh_export_t(const char* bvh, T* lower, T* upper, int32_t* nodes, T* 
 }  // namespace gmc
 
 extern "C" {
+
+void gmc_bvh_set_build_path(int path) { gmc::g_build_path = path == 1 ? 1 : 0; }
 
 size_t gmc_bvh_bytes(const gmc_shape* shape) {
     if (gmc::check_shape(shape) != GMC_OK) return 0;

@@ -197,6 +197,13 @@ typedef struct gmc_bvh_config {
                                the inversion is fused into the build (boxes, leaf records), as in gmc_eval_cov_* */
 } gmc_bvh_config;
 
+/* Test knob (no counterpart in the reference; process-wide): trees of at most 1024 components whose query points come
+ * in segments of at most 8192 are built by one launch (every tree inside one workgroup's LDS), all others by a chain
+ * of launches (global radix sort, leaf and tree kernels, box merge).  path == 1 forces the chain for every shape,
+ * path == 0 returns to the automatic choice.  Both give the same trees, boxes and leaf order bit for bit; the Morton
+ * order of the query points may differ for points on the border of a Morton cell. */
+void gmc_bvh_set_build_path(int path);
+
 /* Bytes of the opaque BVH object for `shape` (nodes, boxes, sorted orders, build scratch). */
 size_t gmc_bvh_bytes(const gmc_shape* shape);
 /* Builds one LBVH per (b,l) mixture into `bvh` (gmc_bvh_bytes bytes) and, when `xes` is not NULL, a

@@ -499,6 +499,41 @@ def test_random_call_sequences_on_one_object():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("D", [2, 3])
+def test_one_launch_build_gives_the_trees_of_the_chain_of_launches(dtype, D):
+    """Small trees are built by one launch (a wavefront, two wavefronts or a workgroup per tree, everything in LDS),
+    larger ones by a chain of launches; with the chain forced for the same inputs every integer and every box of the
+    object must be identical: leaf order and Morton codes, children and parents, node boxes, per-Gaussian boxes.  The
+    culled sums agree to rounding (the Morton order of the query points, hence the order of additions, may differ)."""
+    lib = _native.lib()
+    for k, (B, L, M, N) in enumerate(((3, 2, 1, 50), (2, 2, 2, 10), (2, 3, 3, 70), (5, 4, 64, 700), (3, 3, 65, 1100), (4, 2, 128, 784),
+                                      (2, 2, 129, 4096), (2, 2, 257, 300), (1, 2, 700, 5000), (1, 1, 1024, 8192))):
+        mix, xes, gout = _case(B, L, M, N, D, seed=7300 + k)
+        if k == 3:
+            mix[:, :, 5:30] = mix[:, :, 5:6]               # identical Gaussians: equal keys, ties broken by the component index
+        m, x = mix.to(dtype).to(DEV).contiguous(), xes.to(dtype).to(DEV).contiguous()
+        got = []
+        for path in (0, 1):
+            lib.gmc_bvh_set_build_path(path)
+            try:
+                bvh = _native.Bvh(m, x, 0.001, "reference")
+                lo, up = bvh.boxes()
+                nodes, nb = bvh.nodes()
+                keys, comps = bvh.leaf_order()
+                out = _native.eval_bvh_fwd(m, x, bvh)
+                gmix, gxes = _native.eval_bvh_bwd(gout.to(dtype).to(DEV), m, x, bvh, True, True)
+                torch.cuda.synchronize()
+                assert n_errors(bvh) == 0
+                got.append([t.cpu().numpy() for t in (lo, up, nodes, nb, keys, comps, out, gmix, gxes)])
+            finally:
+                lib.gmc_bvh_set_build_path(0)
+        for a, b, what in zip(got[0][:6], got[1][:6], ("lower", "upper", "nodes", "node boxes", "keys", "components")):
+            assert np.array_equal(a, b), f"{what} differ between the two build paths, B{B} L{L} M{M} N{N} D{D}"
+        for a, b, what in zip(got[0][6:], got[1][6:], ("out", "grad mixture", "grad xes")):
+            assert rel_l2(a, b, FLOOR[dtype]) <= TOL[dtype], what
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("D", [2, 3])
 def test_leaf_order_is_bit_exact(dtype, D):
     """Integer part of the build: the 30-bit Morton codes of the centres (lbvh/morton_code.h:77-85,145-168, positions
     normalised as lbvh/bvh.cu:281-287 in the tensors' precision) and the sorted leaf order, which must be the
