@@ -358,6 +358,15 @@ def test_batch_norm_sampling_positions_and_running_averages():
         assert torch.allclose(sd, 0.75 * 2.0 + 0.25 * sd0, rtol=1e-6) and torch.allclose(mean, 0.75 * -1.0 + 0.25 * mean0, rtol=1e-6, atol=1e-7)
         assert torch.equal(run_sd, sd) and torch.equal(run_mean, mean)
         assert torch.allclose(inv, 1 / torch.clamp(sd, min=0.001), rtol=1e-6)
+    # many numbers per batch entry: they are dealt to several workgroups, each of which finds the box of the centres itself
+    for B, L, N, D in ((2, 8, 5000, 3), (1, 64, 10000, 2)):
+        m = torch.tensor(_cov_mixture(rng, B, L, 30, D).astype(np.float32), device=DEV)
+        u = torch.rand(B, L, N, D, device=DEV)
+        centres = gm.positions(m).reshape(B, -1, D)
+        lo = centres.min(dim=1)[0].view(B, 1, 1, D)
+        hi = centres.max(dim=1)[0].view(B, 1, 1, D)
+        want = (u * 1.3 - 0.15 if D == 2 else u) * (hi - lo) + lo
+        assert torch.allclose(_native.batch_norm_sampling_positions(m, u.clone()), want, rtol=1e-6, atol=1e-6)
     # a channel without spread: the reciprocal is clamped
     flat = torch.tensor(_cov_mixture(rng, 2, 2, 3, 2).astype(np.float32), device=DEV)
     flat[..., 0] = 0.0
