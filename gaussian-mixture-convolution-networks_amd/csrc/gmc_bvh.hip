@@ -1942,6 +1942,162 @@ __global__ __launch_bounds__(kTravBlock) __attribute__((amdgpu_waves_per_eu(4)))
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// small trees: all leaves against all points, the box test in front of every evaluation (no descent)
+// ---------------------------------------------------------------------------------------------------------------
+// A tree of a few dozen leaves has nothing to cull per 64-point group that a box test per leaf does not find faster:
+// the descent, the candidate lists and the lane-by-lane evaluation cost more than they save.  Measured, 64 mixtures of
+// 4096 points, forward / backward us without the tree against the traversal: 32 leaves 16 / 28 against 21 / 40 (6 % of
+// the pairs inside a box; the same ratio at 0.1 %), 64 leaves 25 / 44 against 23 / 49, and with a quarter of the pairs
+// inside (336 mixtures) 78 / 159 against 130 / 262; from 128 leaves on the traversal wins unless most boxes contain
+// most points (22 / 42 against 39 / 56 at 0.6 % inside).  Mixtures of at most kAllPairsMax components are therefore
+// evaluated without the tree: the leaf records of the mixture (own box + evaluation record,
+// as the build left them) are staged in LDS, a wavefront owns P groups of 64 Morton-neighbouring points (lanes =
+// points), walks over ALL leaves and applies the per-point rule of lbvh/aabb.h:39-47 itself; a leaf is evaluated for a
+// group only when its box contains at least one of the group's points (one ballot: neighbouring points mostly agree).
+// Same per-pair arithmetic as the traversal (centred form), same sums: the result is the sum over the Gaussians
+// whose own box contains the point.  Backward: dL/dx in registers; the sums of a leaf are accumulated over the
+// wavefront's P groups in registers, reduced over the wavefront once per leaf and added to the workgroup's LDS copy
+// (double), which leaves with one global atomic per non-zero scalar; the wavefronts start at different leaves.
+constexpr int kAllPairsMax = 64;
+static int g_eval_path = 0;             // test knob (gmc_bvh_set_eval_path): 1 = always the traversal
+
+template <typename T, int D, int P, int MODE, bool NEED_GM, bool NEED_GX>
+__global__ __launch_bounds__(kBlock) void bvh_all_pairs_kernel(const T* __restrict__ xes, const int* __restrict__ p_order,
+                                                              const T* __restrict__ leaf_rec, T* __restrict__ out,
+                                                              const T* __restrict__ grad_out, T* __restrict__ sums,
+                                                              T* __restrict__ grad_xes, int L, int M, int N, int Bx, int Lx,
+                                                              int chunks, int xes_shared) {
+    constexpr int LS = LeafRec<D>::kStride;
+    constexpr int NR = BvhSums<D>::k;
+    constexpr int kAmp = 2 * D + D + D * (D + 1) / 2;       // position of the amplitude inside a leaf record
+    constexpr int kRec = kAmp - 2 * D + 1;                  // centre, symmetric matrix, amplitude
+    __shared__ __attribute__((aligned(16))) T recs[kAllPairsMax * LS];
+    __shared__ double lsum[MODE == 1 && NEED_GM ? kAllPairsMax * NR : 1];
+    const T* exp2_tab = exp2_table<T>();                    // (published by the barrier below)
+    const int bl = blockIdx.x / chunks, chunk = blockIdx.x - bl * chunks;
+    const int b = bl / L, l = bl - b * L;
+    const size_t xseg = size_t(b < Bx ? b : Bx - 1) * Lx + (l < Lx ? l : Lx - 1);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    {
+        const T* src = leaf_rec + size_t(bl) * M * LS;
+        for (int i = threadIdx.x; i < M * LS; i += kBlock) recs[i] = src[i];
+        if (MODE == 1 && NEED_GM)
+            for (int i = threadIdx.x; i < M * NR; i += kBlock) lsum[i] = 0.0;
+    }
+    T x[P][D], go[P], acc[P], gx[P][D];
+    int pid[P];
+    bool any_point = false;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int j = ((chunk * (kBlock / kWave) + wave) * P + p) * kWave + lane;
+        pid[p] = -1;
+        if (j < N) {
+            const int id = p_order[xseg * N + j];
+            pid[p] = unsigned(id) < unsigned(N) ? id : 0;   // a permutation by construction; never index out of bounds
+        }
+        const size_t at = xseg * N + (pid[p] >= 0 ? pid[p] : 0);
+#pragma unroll
+        for (int d = 0; d < D; ++d) { x[p][d] = xes[at * D + d]; gx[p][d] = T(0); }
+        go[p] = (MODE == 1 && pid[p] >= 0) ? grad_out[size_t(bl) * N + pid[p]] : T(0);
+        acc[p] = T(0);
+        any_point |= pid[p] >= 0;
+    }
+    __syncthreads();
+    if (__ballot(any_point) != 0ull) {
+        // the wavefronts of a workgroup start at different leaves: their additions to the LDS sums do not meet
+        const int rot = wave * (M / (kBlock / kWave));
+        for (int ii = 0; ii < M; ++ii) {
+            int i = ii + rot;
+            i -= i >= M ? M : 0;
+            const T* r = recs + i * LS;
+            T box[2 * D];
+#pragma unroll
+            for (int k = 0; k < 2 * D; ++k) box[k] = r[k];
+            T rs[NR];
+#pragma unroll
+            for (int k = 0; k < NR; ++k) rs[k] = T(0);
+            bool touched = false;
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                const bool in = (pid[p] >= 0) & inside_box<T, D>(x[p], box);
+                if (__ballot(in) == 0ull) continue;
+                touched = true;
+                T rec[kRec];
+#pragma unroll
+                for (int k = 0; k < kRec; ++k) rec[k] = r[2 * D + k];
+                T t[D], u[D];
+                const T e = leaf_terms<T, D>(rec, exp2_tab, x[p], t, u);
+                const T s = in ? rec[kRec - 1] * e : T(0);
+                if (MODE == 0) {
+                    acc[p] += s;
+                } else {
+                    if (NEED_GX) {
+#pragma unroll
+                        for (int d = 0; d < D; ++d) gx[p][d] = fma_(s, u[d], gx[p][d]);
+                    }
+                    if (NEED_GM) {
+                        const T k0 = in ? e * go[p] : T(0);
+                        rs[0] += k0;
+                        T rt[D];
+#pragma unroll
+                        for (int d = 0; d < D; ++d) { rt[d] = k0 * t[d]; rs[1 + d] += rt[d]; }
+                        int k = 1 + D;
+#pragma unroll
+                        for (int a = 0; a < D; ++a)
+#pragma unroll
+                            for (int c = a; c < D; ++c) { rs[k] = fma_(rt[a], t[c], rs[k]); ++k; }
+                    }
+                }
+            }
+            if (MODE == 1 && NEED_GM && touched) {
+                // four sums at a time; the lane at the end of row r receives sum {0, 2, 1, 3}[r] of the four
+                const int row = lane >> 4, mine = ((row & 1) << 1) | (row >> 1);
+#pragma unroll
+                for (int q0 = 0; q0 < NR; q0 += 4) {
+                    const T total = wave_sum4_to_row_ends(rs[q0], q0 + 1 < NR ? rs[q0 + 1] : T(0), q0 + 2 < NR ? rs[q0 + 2] : T(0),
+                                                          q0 + 3 < NR ? rs[q0 + 3] : T(0), lane);
+                    if ((lane & 15) == 15 && q0 + mine < NR && total != T(0)) atomic_add(&lsum[i * NR + q0 + mine], double(total));
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        if (pid[p] < 0) continue;
+        if (MODE == 0) {
+            out[size_t(bl) * N + pid[p]] = acc[p];
+        } else if (NEED_GX) {
+            T* dst = grad_xes + (xseg * N + pid[p]) * D;
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                const T v = -go[p] * gx[p][d];
+                if (xes_shared) atomic_add(&dst[d], v); else dst[d] = v;
+            }
+        }
+    }
+    if (MODE == 1 && NEED_GM) {
+        __syncthreads();
+        for (int s = threadIdx.x; s < M * NR; s += kBlock) {
+            const T v = T(lsum[s]);
+            if (v != T(0)) {
+                const int i = s / NR, k = s - i * NR;
+                int comp = reinterpret_cast<const int*>(recs + i * LS + kAmp + 1)[0];
+                comp = unsigned(comp) < unsigned(M) ? comp : 0;
+                atomic_add(&sums[(size_t(bl) * M + comp) * NR + k], v);
+            }
+        }
+    }
+}
+
+// points per lane of the all-pairs kernels: as many as still leave a thousand workgroups
+static int all_pairs_points(size_t BL, int N, int p_max) {
+    const size_t groups = (size_t(N) + kWave - 1) / kWave;
+    for (int P = p_max; P > 1; P >>= 1)
+        if (BL * ((groups + 4 * P - 1) / (4 * P)) >= 1024) return P;
+    return 1;
+}
+
 // (R0, sum r t, sum r t t^T) -> (dw, db, dC); see the dense epilogue for the formulas (here y = t, u = identity).
 // covariance_form: the record holds S with C = (S^-1)^T; the matrix gradient is carried on to S as
 // MatrixInverse.backward does (src/gmc/cpp/extensions/math/matrix_inverse.py:30-33: -S^-1 g S^-1 without transposes,
@@ -2243,6 +2399,16 @@ static int bvh_fwd_t(const T* xes, char* bvh, T* out, const gmc_shape& s, hipStr
         fill_zero_kernel<T><<<dim3(grid_for(n) < 4096 ? grid_for(n) : 4096), dim3(kBlock), 0, st>>>(out, n);
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
+    if (g_eval_path != 1 && s.M <= kAllPairsMax) {
+        const int P = all_pairs_points(BL, s.N, 4);
+        const int chunks = int((size_t(s.N) + size_t(kBlock) * P - 1) / (size_t(kBlock) * P));
+#define GMC_ALL(PP) bvh_all_pairs_kernel<T, D, PP, 0, false, false><<<dim3(unsigned(BL * chunks)), dim3(kBlock), 0, st>>>( \
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.leaf_rec), out, nullptr, nullptr, nullptr, s.L, s.M, s.N, \
+        s.Bx, s.Lx, chunks, 0)
+        if (P == 4) GMC_ALL(4); else if (P == 2) GMC_ALL(2); else GMC_ALL(1);
+#undef GMC_ALL
+        return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+    }
     const int groups = traversal_groups(BL, s.N, false);
     int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     // A launch that would leave resident slots empty is spread over all of them: workgroups whose last wavefront
@@ -2277,6 +2443,25 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bv
     }
     sums = (T*)(bvh + lay.sums);                   // inside the object and all zero here; the caller's workspace is not used
     if (gx && xes_shared) zero(grad_xes, n_x);
+    if (g_eval_path != 1 && s.M <= kAllPairsMax) {
+        const int P = all_pairs_points(BL, s.N, sizeof(T) == 8 ? 2 : 4);
+        const int chunks = int((size_t(s.N) + size_t(kBlock) * P - 1) / (size_t(kBlock) * P));
+#define GMC_ALL(PP, GM, GX) bvh_all_pairs_kernel<T, D, PP, 1, GM, GX><<<dim3(unsigned(BL * chunks)), dim3(kBlock), 0, st>>>( \
+        xes, (const int*)(bvh + lay.p_order), (const T*)(bvh + lay.leaf_rec), nullptr, grad_out, sums, grad_xes, s.L, s.M, s.N, \
+        s.Bx, s.Lx, chunks, xes_shared)
+#define GMC_ALL_P(GM, GX) do { if (P == 4) { if constexpr (sizeof(T) == 4) GMC_ALL(4, GM, GX); } else if (P == 2) GMC_ALL(2, GM, GX); else GMC_ALL(1, GM, GX); } while (0)
+        if (gm && gx) GMC_ALL_P(true, true);
+        else if (gm) GMC_ALL_P(true, false);
+        else if (gx) GMC_ALL_P(false, true);
+#undef GMC_ALL_P
+#undef GMC_ALL
+        if (gm) {
+            bvh_bwd_epilogue_kernel<T, D><<<dim3(grid_for(n_g)), dim3(kBlock), 0, st>>>(
+                mixture, sums, grad_mixture, n_g, covariance_form, candidate_cache(bvh, lay), nullptr, (const int*)(bvh + lay.p_order),
+                grad_xes, xes, grid_for(n_g), s.L, s.N, s.Bx, s.Lx);
+        }
+        return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
+    }
     const int groups = traversal_groups(BL, s.N, true);
     const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     // one helper workgroup per piece that a forward pass may have published, behind the owners
@@ -2330,6 +2515,7 @@ static int bvh_export_t(const char* bvh, T* lower, T* upper, int32_t* nodes, T* 
 extern "C" {
 
 void gmc_bvh_set_build_path(int path) { gmc::g_build_path = path == 1 ? 1 : 0; }
+void gmc_bvh_set_eval_path(int path) { gmc::g_eval_path = path == 1 ? 1 : 0; }
 
 size_t gmc_bvh_bytes(const gmc_shape* shape) {
     if (gmc::check_shape(shape) != GMC_OK) return 0;

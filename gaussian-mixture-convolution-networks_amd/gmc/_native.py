@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 9
+ABI_VERSION = 10
 STATIC_SCRATCH_BYTES = 64 << 20
 
 
@@ -85,6 +85,8 @@ def lib() -> ctypes.CDLL:
     if hasattr(l, "gmc_bvh_bytes"):
         l.gmc_bvh_set_build_path.restype = None
         l.gmc_bvh_set_build_path.argtypes = [ci]
+        l.gmc_bvh_set_eval_path.restype = None
+        l.gmc_bvh_set_eval_path.argtypes = [ci]
         l.gmc_bvh_bytes.restype = sz
         l.gmc_bvh_bytes.argtypes = [shp]
         l.gmc_bvh_build.argtypes = [vp, vp, vp, sz, shp, cfg, vp]

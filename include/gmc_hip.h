@@ -203,6 +203,10 @@ typedef struct gmc_bvh_config {
  * path == 0 returns to the automatic choice.  Both give the same trees, boxes and leaf order bit for bit; the Morton
  * order of the query points may differ for points on the border of a Morton cell. */
 void gmc_bvh_set_build_path(int path);
+/* Test knob like the one above: mixtures of at most 64 components are evaluated without the tree (all leaves against
+ * all points with the box test in front of every evaluation: same rule, same sums); path == 1 forces the traversal for
+ * every shape, path == 0 returns to the automatic choice. */
+void gmc_bvh_set_eval_path(int path);
 
 /* Bytes of the opaque BVH object for `shape` (nodes, boxes, sorted orders, build scratch). */
 size_t gmc_bvh_bytes(const gmc_shape* shape);

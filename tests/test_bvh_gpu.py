@@ -31,6 +31,17 @@ def _report_budget_use():
     print("\nworst |error| / budget per tensor (culled path):", {k: round(v, 4) for k, v in sorted(BUDGET_USE.items())}, flush=True)
 
 
+@pytest.fixture(params=["automatic", "traversal"])
+def eval_path(request):
+    """Mixtures of at most 64 components are evaluated without the tree (all leaves against all points, the box test in
+    front of every evaluation); tests that take this fixture run once with the automatic choice and once with the
+    traversal forced for every shape."""
+    lib = _native.lib()
+    lib.gmc_bvh_set_eval_path(1 if request.param == "traversal" else 0)
+    yield request.param
+    lib.gmc_bvh_set_eval_path(0)
+
+
 def _case(B, L, M, N, D, seed, broadcast=False, spread=4.0, cov_radius=0.3):
     g = torch.Generator().manual_seed(seed)
     mix = synthetic.random_inversed_mixture(B, L, M, D, g, pos_radius=spread, cov_radius=cov_radius, dtype=torch.float64)
@@ -155,7 +166,7 @@ def test_tree_invariants(D):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("D", [2, 3])
 @pytest.mark.parametrize("mode", ["reference", "tight"])
-def test_culled_matches_masked_dense_sum(dtype, D, mode):
+def test_culled_matches_masked_dense_sum(dtype, D, mode, eval_path):
     seed = 300
     for B, L, M, N, bc in ((1, 1, 1, 1, False), (2, 3, 2, 70, False), (1, 2, 33, 130, False), (3, 2, 100, 257, True),
                            (1, 1, 600, 1000, False)):
@@ -171,7 +182,7 @@ def test_culled_matches_masked_dense_sum(dtype, D, mode):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
-def test_several_point_groups_per_workgroup(dtype):
+def test_several_point_groups_per_workgroup(dtype, eval_path):
     """Launches with more 64-point groups than resident workgroups give every workgroup two to four groups (their
     descents overlap); the last groups are ragged or empty.  Narrow Gaussians exercise the lane-by-lane evaluation
     with LDS atomics, wide ones the wavefront reduction and candidate lists that are evaluated in several rounds."""
@@ -186,6 +197,17 @@ def test_several_point_groups_per_workgroup(dtype):
     _check_culled(mix, xes, gout, dtype, "tight", tag="wide")
     mix, xes, gout = _case(9, 1, 600, 64 * 60, 2, seed + 2, spread=1.0, cov_radius=3.0)
     _check_culled(mix, xes, gout, dtype, "tight", tag="wide, several groups")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_small_trees_many_mixtures(dtype):
+    """Hundreds of mixtures of a few dozen components (the shapes of network layers): built by one launch and evaluated
+    without the tree, with one, two and four 64-point groups per wavefront (the choice follows the number of
+    workgroups), ragged last groups, broadcast points; against the masked sum like every other culled result."""
+    for k, (B, L, M, N, D, bc) in enumerate(((24, 24, 10, 600, 3, False), (24, 24, 6, 1100, 2, False), (3, 4, 64, 1300, 3, False),
+                                             (6, 7, 17, 5000, 2, True))):
+        mix, xes, gout = _case(B, L, M, N, D, seed=5200 + k, broadcast=bc, cov_radius=0.2)
+        _check_culled(mix, xes, gout, dtype, "tight" if k % 2 else "reference", tag=f"B{B} L{L} M{M} N{N} D{D} bc{bc}")
 
 
 def test_mixture_beyond_the_reference_node_index_range():
@@ -211,7 +233,7 @@ def test_mixture_beyond_the_reference_node_index_range():
         _check_culled(mix, xes, gout, dtype, "tight", tag=f"M{M}")
 
 
-def test_culled_random_shapes():
+def test_culled_random_shapes(eval_path):
     """differential run of the culled path over random shapes (one to four point groups per workgroup, ragged and
     empty trailing groups, broadcast points, identical Gaussians, narrow and wide boxes) against the masked sum"""
     rng = np.random.default_rng(777)
@@ -241,7 +263,7 @@ def test_culled_random_shapes():
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("D", [2, 3])
 @pytest.mark.parametrize("mode", ["reference", "tight"])
-def test_covariance_form_matches_explicit_inversion(dtype, D, mode):
+def test_covariance_form_matches_explicit_inversion(dtype, D, mode, eval_path):
     """gm.evaluate(mixture with covariances, bvh=...) inverts inside the LBVH build; it must agree with the route of
     the reference's gm.evaluate (src/gmc/mixture.py:144-149): mat_tools.inverse, transpose, pack, evaluate_inversed --
     same boxes, same values, and the same gradients after autograd has carried them through the inversion."""
@@ -570,7 +592,7 @@ def n_errors(bvh):
     return int(bvh.candidate_stats().cpu().numpy()[2])
 
 
-def test_points_outside_every_box_and_need_flags():
+def test_points_outside_every_box_and_need_flags(eval_path):
     mix, xes, gout = _case(1, 2, 40, 64, 3, seed=400)
     far = xes + 1000.0
     out, gmix, gxes = _run_culled(mix, far, gout, torch.float64, "tight")
@@ -606,7 +628,7 @@ def test_empty_and_config_errors():
         _native.eval_bvh_bwd(torch.zeros(1, 1, 2, device=DEV, dtype=torch.float64), mix.double(), xes.double(), bvh, True, True)
 
 
-def test_gradcheck_culled_fp64():
+def test_gradcheck_culled_fp64(eval_path):
     mix, xes, _ = _case(2, 2, 9, 12, 3, seed=500, spread=1.0, cov_radius=0.5)
     # keep points away from box faces so that finite differences do not cross the (fixed) mask
     m = mix.to(DEV).requires_grad_(True)
