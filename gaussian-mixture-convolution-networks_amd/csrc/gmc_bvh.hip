@@ -15,6 +15,11 @@
 // neighbouring points; their two sort passes ride as extra workgroups in the two longest launches of the tree
 // construction, and one wavefront per tree leaves a cut through the tree a few levels below the root (tree_frontier).
 //
+// Small trees take short cuts: mixtures of at most 1024 components (query points in segments of at most 8192) are built
+// by ONE launch, every tree inside the LDS of a wavefront or a workgroup (bvh_build_small_kernel: same trees bit for
+// bit), and mixtures of at most 64 components are evaluated without the tree, all leaves against all points with the
+// box test in front (bvh_all_pairs_kernel: same rule, same sums).
+//
 // Traversal: 64 sorted points form a group with ONE node stack (LDS); lanes work on tree nodes while the tree is
 // descended and on points while the gathered leaves are evaluated; a workgroup serves up to four groups, whose
 // descents overlap (see bvh_traverse_kernel).  A descent starts from the cut the build has left and tests node boxes
