@@ -48,6 +48,26 @@ def test_c_abi_rejects_bad_shapes_without_launching():
     assert lib.gmc_eval_bwd(null, null, null, null, null, null, 0, ctypes.byref(ok), 1, 1, null) == -4
 
 
+def test_scratch_sizes_and_knobs_without_a_device():
+    """Host-only entry points: the scratch of the fused BatchNorm moments (three doubles per workgroup: 128 points per
+    workgroup up to 128 points per mixture, 256 up to 256, then 512), the size of the opaque BVH object (grows with
+    every dimension, 0 for an invalid shape), the two process-wide test knobs."""
+    lib = _native.lib()
+    S = _native.Shape
+    for N, per_workgroup in ((1, 128), (100, 128), (128, 128), (129, 256), (256, 256), (257, 512), (1300, 512), (10000, 512)):
+        chunks = (N + per_workgroup - 1) // per_workgroup
+        assert lib.gmc_eval_cov_moments_bytes(ctypes.byref(S(3, 4, 30, N, 2, 3, 4, 0))) == 3 * 4 * chunks * 3 * 8
+    assert lib.gmc_eval_cov_moments_bytes(ctypes.byref(S(3, 4, 30, 100, 2, 1, 1, 0))) == 0       # points must be per mixture
+    assert lib.gmc_eval_cov_moments_bytes(ctypes.byref(S(3, 4, 30, 100, 5, 3, 4, 0))) == 0
+    sizes = [lib.gmc_bvh_bytes(ctypes.byref(S(2, 3, M, N, 3, 2, 3, 1))) for M, N in ((10, 100), (100, 100), (100, 5000), (5000, 5000))]
+    assert all(a < b for a, b in zip(sizes, sizes[1:])) and sizes[0] > 0
+    assert lib.gmc_bvh_bytes(ctypes.byref(S(2, 3, 10, 100, 4, 2, 3, 1))) == 0
+    assert lib.gmc_bvh_bytes(ctypes.byref(S(2, 3, 10, 100, 3, 2, 3, 0))) < lib.gmc_bvh_bytes(ctypes.byref(S(2, 3, 10, 100, 3, 2, 3, 1)))
+    for knob in (lib.gmc_bvh_set_build_path, lib.gmc_bvh_set_eval_path):
+        knob(1)
+        knob(0)
+
+
 def test_python_boundary_errors():
     m = torch.zeros(2, 3, 4, 13)
     x = torch.zeros(2, 3, 5, 3)
