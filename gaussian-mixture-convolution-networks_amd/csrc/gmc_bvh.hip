@@ -48,7 +48,9 @@ struct BvhLayout {
     size_t parent;              // int [BL][2M-1]
     size_t node_range;          // int2 [BL][M-1]          first and last leaf below every internal node
     size_t leaf_comp;           // int [BL][M]             component id of each leaf
-    size_t enc_box;             // int64 [BL][M-1][2D]     boxes of the internal nodes as order-preserving integers
+    size_t run_box;             // intT [ceil(BL*M/kBoxBlock)*kBoxBlock][2][2D] leaves of all mixtures numbered through, in blocks of
+                                //                          kBoxBlock: union of the leaf boxes from the start of the block up to the
+                                //                          leaf, and from the leaf to the end of the block (order-preserving integers)
     size_t parts_g, parts_p;    // T [segments][blocks][2D] per-block partial bounds of the centres / the query points
     size_t keys_a, keys_b, vals_a, vals_b;       // uint32 [BL*M]   radix ping-pong of the leaves
     size_t pkeys_a, pkeys_b, pvals_a, pvals_b;   // uint32 [BxLx*N] radix ping-pong of the query points
@@ -110,6 +112,7 @@ struct CandidateCache {
     int2* piece_range;
     int pieces_max, pool_cap, pool_base;
 };
+constexpr int kBoxBlock = 128;          // leaves whose internal nodes get their boxes inside one workgroup (see bvh_leaves_kernel)
 constexpr int kFrontier = 64;           // internal nodes a descent starts from (see tree_frontier)
 constexpr int kErrStack = 1;            // a traversal's node stack was full and a push was dropped (results incomplete)
 constexpr int kErrSort = 2;             // a radix pass computed an output slot outside its segment
@@ -154,7 +157,7 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     l.parent = take(BL * nodes * 4);
     l.node_range = take(BL * (M > 0 ? M - 1 : 0) * 8);
     l.leaf_comp = take(BL * M * 4);
-    l.enc_box = take(BL * (M > 0 ? M - 1 : 0) * 2 * D * 8);
+    l.run_box = take((BL * M + kBoxBlock - 1) / kBoxBlock * kBoxBlock * 4 * D * e);
     l.parts_g = take(BL * ((M + kBlock - 1) / kBlock) * 2 * D * e);
     l.parts_p = take(XL * ((N + kBoundsChunk - 1) / kBoundsChunk) * 2 * D * e);
     l.keys_a = take(BL * M * 4);
@@ -611,6 +614,13 @@ __device__ __forceinline__ int ordered_bits(float v) {
     return b ^ ((b >> 31) & 0x7fffffff);
 }
 __device__ __forceinline__ float from_ordered_bits(int k) { return __builtin_bit_cast(float, k ^ ((k >> 31) & 0x7fffffff)); }
+// the integer type of T's width, and the empty box in it: lower = +inf, upper = -inf
+template <typename T> struct OrderedInt;
+template <> struct OrderedInt<float> { using type = int; static constexpr int kEmptyLo = 0x7fffffff, kEmptyHi = -0x7fffffff - 1; };
+template <> struct OrderedInt<double> {
+    using type = long long;
+    static constexpr long long kEmptyLo = 0x7fffffffffffffffll, kEmptyHi = -0x7fffffffffffffffll - 1;
+};
 
 // Internal node i of the radix tree over the M sorted keys (Karras 2012; lbvh/building.h:11-103); key_at(j) returns the
 // j-th sorted Morton code, the unique keys are (code << 32 | j).  first / last: the range of leaves below the node;
@@ -651,20 +661,21 @@ __device__ __forceinline__ void radix_tree_node(KeyAt key_at, int M, int i, int&
     right = (split + 1 == last) ? ~(split + 1) : split + 1;
 }
 
-// internal node i of the radix tree of mixture bl, keys in memory
-__device__ __forceinline__ void build_internal_node(const uint32_t* __restrict__ keys, int2* __restrict__ children,
+// internal node i of the radix tree of mixture bl (key_at(j): the j-th sorted key of the mixture); returns its range
+template <typename KeyAt>
+__device__ __forceinline__ int2 build_internal_node(KeyAt key_at, int2* __restrict__ children,
                                                     int* __restrict__ parent, int2* __restrict__ node_range, int M,
                                                     size_t bl, int i) {
     const size_t t = bl * (M - 1) + i;
-    const uint32_t* k = keys + bl * M;
     int first, last, left, right;
-    radix_tree_node([&](int j) { return k[j]; }, M, i, first, last, left, right);
+    radix_tree_node(key_at, M, i, first, last, left, right);
     children[t] = make_int2(left, right);
     node_range[t] = make_int2(first, last);
     int* par = parent + bl * (2 * size_t(M) - 1);
     par[left >= 0 ? left : (M - 1) + ~left] = i;
     par[right >= 0 ? right : (M - 1) + ~right] = i;
     if (i == 0) par[0] = -1;
+    return make_int2(first, last);
 }
 
 // Leaf `leaf` (Morton order) of mixture bl, which holds component `comp`: the cutoff box of the Gaussian
@@ -722,40 +733,117 @@ __device__ __forceinline__ void write_leaf(const T* __restrict__ mixture, T* __r
     }
 }
 
+// Boxes of the internal nodes without a walk through the tree.  Internal node i covers the leaves first ... last of the
+// Morton order (its range), so its box is a range union over the leaf boxes, and min / max are idempotent: the union
+// over any range is the union of two overlapping runs of 2^k leaves (a sparse table).  The leaves of all mixtures are
+// numbered through and cut into blocks of kBoxBlock; the workgroup of a block
+//   * writes the records and boxes of its leaves (lanes 0 ... kBoxBlock-1) while the other half of its lanes builds
+//     the internal nodes with the same numbers (node i lies inside its own range; both are short chains of dependent
+//     memory reads that do not depend on each other),
+//   * builds the table of its leaf boxes in LDS (order-preserving integers: the same unions, bit for bit, as integer
+//     atomic min / max would give) and looks up the box of every node whose range lies inside the block,
+//   * leaves, for every leaf, the unions from the start of the block up to the leaf and from the leaf up to the end of
+//     the block in run_box (the latter of the first leaf is the union of the whole block).
+// The few nodes whose range crosses a block border get their box in the next launch (bvh_child_boxes_kernel): the run
+// from the first leaf of the range to the end of its block, the whole blocks in between, the run from the start of the
+// last block to the last leaf.  No step waits for another node: the bottom-up walk this replaces was a chain of one
+// atomic round trip per tree level.
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
                                                            T* __restrict__ box_hi, double threshold, int mode,
                                                            const uint32_t* __restrict__ order,
                                                            const uint32_t* __restrict__ keys, T* __restrict__ node_box,
-                                                           T* __restrict__ leaf_rec, long long* __restrict__ enc_box,
+                                                           T* __restrict__ leaf_rec,
+                                                           typename OrderedInt<T>::type* __restrict__ run_box,
                                                            int2* __restrict__ children, int* __restrict__ parent,
                                                            int2* __restrict__ node_range, int M, size_t total,
                                                            bool covariance_form, T* __restrict__ sums,
                                                            unsigned own_blocks, SortJob rider) {
+    using Enc = typename OrderedInt<T>::type;
+    constexpr int kLevels = 8;                              // runs of 1, 2, ... 128 leaves
+    static_assert(kBoxBlock == 128 && kBlock == 2 * kBoxBlock, "one half of the lanes per leaf, the other per node");
+    __shared__ Enc table[kLevels][2 * D][kBoxBlock];
     // The sort of the query points does not depend on the trees: a pass of it rides behind this kernel's own
     // workgroups, on compute units that would idle otherwise, instead of lengthening a pass of the leaves' sort.
     if (blockIdx.x >= own_blocks) { radix_scatter_pass(rider, blockIdx.x - own_blocks); return; }
-    // The records of the leaves and the internal nodes of the tree do not depend on each other, and both are
-    // short chains of dependent memory reads: the first half of the grid writes the records, the second half
-    // builds the nodes, side by side on different compute units.
-    const unsigned half = own_blocks / 2;
-    const bool tree_job = blockIdx.x >= half;
-    const size_t i = size_t(tree_job ? blockIdx.x - half : blockIdx.x) * kBlock + threadIdx.x;
-    if (i >= total) return;
-    const size_t bl = i / M;
-    const int leaf = int(i - bl * M);
-    if (tree_job) {
-        // lane <-> internal node `leaf` of its mixture (there are M-1 of them)
-        if (leaf < M - 1) build_internal_node(keys, children, parent, node_range, M, bl, leaf);
-        return;
+    const size_t first_leaf = size_t(blockIdx.x) * kBoxBlock;
+    const int idx = threadIdx.x & (kBoxBlock - 1);
+    const bool node_lane = threadIdx.x >= kBoxBlock;
+    const size_t t = first_leaf + idx;
+    const size_t bl = t < total ? t / M : 0;
+    const int leaf = int(t - bl * M);
+    // The searches of a node (its range, its split) read keys at distances 1, 2, 4 ... from the node, each read after
+    // the one before: the keys around the block wait in LDS, only the long steps of the few nodes with long ranges go
+    // to memory.
+    constexpr int kBefore = 192, kWindow = 2 * kBlock;
+    __shared__ uint32_t window[kWindow];
+    const long long window_first = (long long)first_leaf - kBefore;
+    for (int k = threadIdx.x; k < kWindow; k += kBlock) {
+        const long long g = window_first + k;
+        window[k] = g >= 0 && g < (long long)total ? keys[g] : 0u;
     }
-    T blo[D], bhi[D];
-    write_leaf<T, D>(mixture, box_lo, box_hi, threshold, mode, covariance_form, node_box, leaf_rec, parent, sums, M, bl, leaf,
-                     int(order[i]), blo, bhi);
-    if (leaf < M - 1) {
-        // empty box of internal node `leaf`: lower = +inf, upper = -inf in the ordered-integer encoding
-        long long* e = enc_box + (bl * (M - 1) + leaf) * 2 * D;
-        for (int d = 0; d < D; ++d) { e[d] = ordered_bits(double(INFINITY)); e[D + d] = ordered_bits(double(-INFINITY)); }
+    const int comp = !node_lane && t < total ? int(order[t]) : 0;
+    __syncthreads();
+    bool inside = false;                                    // node lanes: the node's range lies inside this block
+    int range_lo = 0, range_hi = 0;                         // ... as slots of the block
+    if (!node_lane) {
+        Enc lo[D], hi[D];
+        for (int d = 0; d < D; ++d) { lo[d] = OrderedInt<T>::kEmptyLo; hi[d] = OrderedInt<T>::kEmptyHi; }
+        if (t < total) {
+            T blo[D], bhi[D];
+            write_leaf<T, D>(mixture, box_lo, box_hi, threshold, mode, covariance_form, node_box, leaf_rec, parent, sums, M, bl,
+                             leaf, comp, blo, bhi);
+            for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(blo[d]); hi[d] = ordered_bits(bhi[d]); }
+        }
+        for (int d = 0; d < D; ++d) { table[0][d][idx] = lo[d]; table[0][D + d][idx] = hi[d]; }
+    } else if (t < total && leaf < M - 1) {
+        // lane <-> internal node `leaf` of its mixture (there are M-1 of them)
+        const long long shift = (long long)(bl * M) - window_first;       // key j of the mixture waits in slot j + shift
+        const uint32_t* k = keys + bl * M;
+        const int2 r = build_internal_node([&](int j) {
+            const long long slot = j + shift;
+            return slot >= 0 && slot < kWindow ? window[slot] : k[j];
+        }, children, parent, node_range, M, bl, leaf);
+        const size_t lo = bl * M + r.x, hi = bl * M + r.y;
+        inside = lo >= first_leaf && hi < first_leaf + kBoxBlock;
+        range_lo = int(lo - first_leaf);
+        range_hi = int(hi - first_leaf);
+    }
+    __syncthreads();
+    for (int k = 1; k < kLevels; ++k) {
+        const int half = 1 << (k - 1);
+        for (int e = threadIdx.x; e < 2 * D * kBoxBlock; e += kBlock) {
+            const int c = e / kBoxBlock, i = e - c * kBoxBlock;
+            const Enc a = table[k - 1][c][i];
+            const Enc b = i + half < kBoxBlock ? table[k - 1][c][i + half] : a;    // (runs that leave the block are never read)
+            table[k][c][i] = c < D ? (b < a ? b : a) : (b > a ? b : a);
+        }
+        __syncthreads();
+    }
+    // union of the leaf boxes in slots a ... b of the block
+    auto range_union = [&](int a, int b, Enc (&out)[2 * D]) {
+        const int k = 31 - __clz(b - a + 1);
+        const int second = b + 1 - (1 << k);
+        for (int c = 0; c < 2 * D; ++c) {
+            const Enc u = table[k][c][a], v = table[k][c][second];
+            out[c] = c < D ? (v < u ? v : u) : (v > u ? v : u);
+        }
+    };
+    if (inside) {
+        Enc u[2 * D];
+        range_union(range_lo, range_hi, u);
+        T* dst = node_box + (bl * (2 * size_t(M) - 1) + leaf) * 2 * D;
+        for (int c = 0; c < 2 * D; ++c) dst[c] = from_ordered_bits(u[c]);
+    }
+    if (!node_lane) {
+        // for the ranges that cross a block border: the unions from the first leaf of the block up to this one and from this
+        // one up to the last leaf of the block
+        Enc u[2 * D];
+        range_union(0, idx, u);
+        Enc* dst = run_box + t * 4 * D;
+        for (int c = 0; c < 2 * D; ++c) dst[c] = u[c];
+        range_union(idx, kBoxBlock - 1, u);
+        for (int c = 0; c < 2 * D; ++c) dst[2 * D + c] = u[c];
     }
 }
 
@@ -806,140 +894,121 @@ __device__ __forceinline__ void tree_frontier(const int2* __restrict__ kids, int
     if (lane < n) out[1 + lane] = cur[lane];
 }
 
-// Bottom-up boxes without inter-lane ordering: a walker goes towards the root and merges ITS OWN box into every
-// ancestor with atomic min/max, as long as it still enlarges the ancestor; it stops at the first ancestor that
-// already contains it.  Every extreme of that ancestor was set by some walker that enlarged it and therefore walks
-// on itself, so all higher ancestors end up containing the stopped box as well: the final boxes are the exact unions
-// of the leaves below each node.  Nothing is read back except the atomics' own return values, so no fences are
-// needed; the decoded boxes are produced by the next kernel.
-// A walk is a chain of atomic round trips, one per tree level.  The lower levels stay inside the workgroup: an
-// internal node whose leaves all belong to the kMergeBlock leaves of this workgroup is touched by these lanes only, so its
-// box lives in LDS while the leaves walk (internal node i lies inside its own leaf range, hence slot i - first leaf
-// of the workgroup is free for it) and is stored once at the end.  The ancestors that reach beyond the workgroup's
-// leaves are merged with global atomics by the roots of the local subtrees alone, with their finished boxes.
-// leaves per workgroup of the box merge (1024 keep two more tree levels in LDS but occupy too few compute units: slower)
-constexpr int kMergeBlock = 256;
+// Second half of the boxes, lane <-> node (internal nodes and leaves): the node takes its own box -- a leaf's and that
+// of an internal node whose range lies inside one block of kBoxBlock leaves from bvh_leaves_kernel, otherwise the union
+// of the runs at both ends of the range and of the whole blocks in between (run_box; up to kNearBlocks whole blocks by
+// the lane itself in one batch of loads, more -- a handful of nodes next to the root -- by the whole wavefront) -- and
+// stores it with its parent (child_box; traversals test both children of a node with one fetch) and, where it was not
+// known before, as its node box.  Which child it is, an internal node reads off its own range (the left child of a
+// node that splits behind leaf s is internal node s, the last leaf of its own range; the right child is s + 1, the
+// first of its own range); a leaf looks at its parent's children.  No lane waits for another node.
+// Behind these workgroups: a pass of the points' sort (see bvh_leaves_kernel), then one wavefront per tree that finds
+// where descents start.
+constexpr int kNearBlocks = 8;
 
 template <typename T, int D>
-__global__ __launch_bounds__(kMergeBlock) void bvh_merge_kernel(const int* __restrict__ parent, const int2* __restrict__ node_range,
-                                                          const T* __restrict__ node_box, long long* enc_box, int M,
-                                                          size_t total, unsigned own_blocks, SortJob rider,
-                                                          const int2* __restrict__ children, int* __restrict__ frontier,
-                                                          size_t mixtures) {
-    __shared__ long long local_box[kMergeBlock][2 * D];
-    __shared__ int local_parent[kMergeBlock];
-    __shared__ int is_local[kMergeBlock];
-    static_assert(kMergeBlock == kBlock, "the riding sort pass works with kBlock lanes");
-    if (blockIdx.x >= own_blocks + rider.blocks) {          // behind both: one wavefront per tree finds where descents start
-        const size_t bl = size_t(blockIdx.x - own_blocks - rider.blocks) * (kMergeBlock / kWave) + (threadIdx.x >> 6);
+__global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __restrict__ children, const int* __restrict__ parent,
+                                                                const int2* __restrict__ node_range,
+                                                                const typename OrderedInt<T>::type* __restrict__ run_box,
+                                                                T* node_box, T* __restrict__ child_box, int M, size_t total,
+                                                                CandidateCache cache, size_t point_groups,
+                                                                unsigned own_blocks, SortJob rider, int* __restrict__ frontier,
+                                                                size_t mixtures) {
+    using Enc = typename OrderedInt<T>::type;
+    if (blockIdx.x >= own_blocks + rider.blocks) {
+        const size_t bl = size_t(blockIdx.x - own_blocks - rider.blocks) * (kBlock / kWave) + (threadIdx.x >> 6);
         if (bl < mixtures) tree_frontier(children + bl * (M - 1), M, frontier + bl * (1 + kFrontier), threadIdx.x & 63);
         return;
     }
-    if (blockIdx.x >= own_blocks) { radix_scatter_pass(rider, blockIdx.x - own_blocks); return; }   // (see bvh_leaves_kernel)
-    const size_t first_leaf = size_t(blockIdx.x) * kMergeBlock;          // leaves of all mixtures, numbered through
-    const size_t t = first_leaf + threadIdx.x;
-    const size_t bl = t < total ? t / M : 0;
-    const int leaf = int(t - bl * M);
-    const size_t nbase = bl * (2 * size_t(M) - 1);
-    // lane <-> internal node `leaf` of its mixture (there are M-1 of them)
-    bool mine = false;
-    if (t < total && leaf < M - 1) {
-        const int2 r = node_range[bl * (M - 1) + leaf];
-        const size_t lo = bl * M + r.x, hi = bl * M + r.y;
-        mine = lo >= first_leaf && hi < first_leaf + kMergeBlock && hi < total;
-        local_parent[threadIdx.x] = parent[nbase + leaf];
-    }
-    is_local[threadIdx.x] = mine ? 1 : 0;
-    for (int d = 0; d < D; ++d) {
-        local_box[threadIdx.x][d] = 0x7fffffffffffffffll;           // empty: lower = +inf, upper = -inf
-        local_box[threadIdx.x][D + d] = -0x7fffffffffffffffll - 1;
-    }
-    __syncthreads();
-    // Two phases.  First every leaf walks through its local ancestors only (LDS atomics).  Then the roots of the local
-    // subtrees -- local internal nodes and leaves whose parent reaches beyond the workgroup, a dozen or two per
-    // workgroup -- walk on through the global ancestors with the finished box of their subtree: a few global atomics
-    // per workgroup and tree level instead of one per leaf on the same few addresses.
-    auto is_local_node = [&](int node) -> bool {
-        const long long slot = (long long)(bl * M + node) - (long long)first_leaf;
-        return slot >= 0 && slot < kMergeBlock && is_local[slot];
-    };
-    long long* enc = enc_box + bl * (M - 1) * 2 * D;
-    // walk from `node` upwards through global ancestors with the box (lo, hi)
-    auto global_walk = [&](int node, const long long (&lo)[D], const long long (&hi)[D]) {
-        // the radix tree over 64-bit keys is at most 64 levels deep; the bound also ends a walk on a malformed chain
-        for (int level = 0; node >= 0 && node < M - 1 && level < 128; ++level) {
-            const int up = parent[nbase + node];            // fetched alongside the atomics: one round trip per level
-            long long* e = enc + size_t(node) * 2 * D;
-            bool grew = false;
-            for (int d = 0; d < D; ++d) {
-                grew |= lo[d] < atomicMin(&e[d], lo[d]);
-                grew |= hi[d] > atomicMax(&e[D + d], hi[d]);
-            }
-            if (!grew) break;
-            node = up;
-        }
-    };
-    long long leaf_lo[D], leaf_hi[D];
-    int leaf_exit = -1;                                     // the first ancestor of this leaf that is not local
-    if (t < total) {
-        const T* box = node_box + (nbase + (M - 1) + leaf) * 2 * D;
-        for (int d = 0; d < D; ++d) { leaf_lo[d] = ordered_bits(double(box[d])); leaf_hi[d] = ordered_bits(double(box[D + d])); }
-        int node = parent[nbase + (M - 1) + leaf];
-        if (node >= 0 && node < M - 1 && !is_local_node(node)) leaf_exit = node;
-        for (int level = 0; node >= 0 && node < M - 1 && level < 128 && is_local_node(node); ++level) {
-            const int slot = int((long long)(bl * M + node) - (long long)first_leaf);
-            bool grew = false;
-            for (int d = 0; d < D; ++d) {
-                grew |= leaf_lo[d] < atomicMin(&local_box[slot][d], leaf_lo[d]);
-                grew |= leaf_hi[d] > atomicMax(&local_box[slot][D + d], leaf_hi[d]);
-            }
-            if (!grew) break;
-            node = local_parent[slot];
-        }
-    }
-    __syncthreads();
-    if (leaf_exit >= 0) global_walk(leaf_exit, leaf_lo, leaf_hi);
-    if (mine) {
-        const int up = local_parent[threadIdx.x];
-        if (up >= 0 && up < M - 1 && !is_local_node(up)) {
-            long long lo[D], hi[D];
-            for (int d = 0; d < D; ++d) { lo[d] = local_box[threadIdx.x][d]; hi[d] = local_box[threadIdx.x][D + d]; }
-            global_walk(up, lo, hi);
-        }
-    }
-    __syncthreads();
-    if (mine) {
-        long long* e = enc_box + (bl * (M - 1) + leaf) * 2 * D;
-        for (int d = 0; d < 2 * D; ++d) e[d] = local_box[threadIdx.x][d];
-    }
-}
-
-// decodes the internal boxes and stores, with every internal node, the boxes of its two children
-template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __restrict__ children,
-                                                                const long long* __restrict__ enc_box, T* node_box,
-                                                                T* __restrict__ child_box, int M, size_t total,
-                                                                CandidateCache cache, size_t point_groups) {
-    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (blockIdx.x >= own_blocks) { radix_scatter_pass(rider, blockIdx.x - own_blocks); return; }
+    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;          // nodes of all trees, numbered through
+    const int lane = threadIdx.x & 63;
     if (cache.count) {                               // a new tree: no candidate list is known yet
-        for (size_t j = t; j < point_groups; j += size_t(gridDim.x) * kBlock) cache.count[j] = -1;
+        for (size_t j = t; j < point_groups; j += size_t(own_blocks) * kBlock) cache.count[j] = -1;
     }
-    if (t >= total) return;
-    const size_t bl = t / (M - 1);
-    const int node = int(t - bl * (M - 1));
-    const size_t nbase = bl * (2 * size_t(M) - 1);
-    const int2 ch = children[t];
-    for (int d = 0; d < 2 * D; ++d) node_box[(nbase + node) * 2 * D + d] = T(from_ordered_bits(enc_box[t * 2 * D + d]));
-    for (int side = 0; side < 2; ++side) {
-        const int c = side == 0 ? ch.x : ch.y;
-        T* dst = child_box + (t * 2 + side) * 2 * D;
-        if (c < 0) {
-            const T* src = node_box + (nbase + (M - 1) + ~c) * 2 * D;       // leaf boxes were written by an earlier kernel
-            for (int d = 0; d < 2 * D; ++d) dst[d] = src[d];
-        } else {
-            const long long* src = enc_box + (bl * (M - 1) + c) * 2 * D;
-            for (int d = 0; d < 2 * D; ++d) dst[d] = T(from_ordered_bits(src[d]));
+    const size_t n_nodes = 2 * size_t(M) - 1;
+    const bool active = t < total;
+    const size_t bl = active ? t / n_nodes : 0;
+    const int node = active ? int(t - bl * n_nodes) : 0;
+    const bool internal = active && node < M - 1;
+    // union of the whole block b
+    auto block_union = [&](size_t b) { return run_box + b * kBoxBlock * 4 * D + 2 * D; };
+    const int up = active ? parent[bl * n_nodes + node] : -1;
+    const int2 range = internal ? node_range[bl * (M - 1) + node] : make_int2(0, 0);
+    const size_t lo = bl * M + range.x, hi = bl * M + range.y;
+    const size_t b_lo = lo / kBoxBlock, b_hi = hi / kBoxBlock;
+    const bool far = b_lo != b_hi;
+    Enc box[2 * D];
+    {
+        const T* src = node_box + (bl * n_nodes + node) * 2 * D;      // written by the launch before, unless `far`
+        for (int d = 0; d < 2 * D; ++d) box[d] = ordered_bits(src[d]);
+    }
+    // a leaf: which child of its parent?
+    int side = node == range.y ? 0 : 1;
+    if (active && !internal && up >= 0 && up < M - 1) side = children[bl * (M - 1) + up].x == ~(node - (M - 1)) ? 0 : 1;
+    bool wide = false;
+    if (far) {
+        const Enc* head = run_box + lo * 4 * D + 2 * D;     // from the first leaf of the range to the end of its block
+        const Enc* tail = run_box + hi * 4 * D;             // from the start of the last block to the last leaf of the range
+        const size_t whole = b_hi - b_lo - 1;
+        Enc v[2 + kNearBlocks][2 * D];
+        for (int d = 0; d < 2 * D; ++d) { v[0][d] = head[d]; v[1][d] = tail[d]; }
+        const bool near = whole <= size_t(kNearBlocks);
+#pragma unroll
+        for (int q = 0; q < kNearBlocks; ++q) {              // all loads in flight together
+            const Enc* src = block_union(near && size_t(q) < whole ? b_lo + 1 + q : b_lo);
+            for (int d = 0; d < 2 * D; ++d) v[2 + q][d] = src[d];
         }
+        for (int d = 0; d < 2 * D; ++d) box[d] = v[0][d];
+#pragma unroll
+        for (int q = 1; q < 2 + kNearBlocks; ++q) {
+            const bool use = q < 2 || (near && size_t(q - 2) < whole);
+            for (int d = 0; d < D; ++d) {
+                box[d] = use && v[q][d] < box[d] ? v[q][d] : box[d];
+                box[D + d] = use && v[q][D + d] > box[D + d] ? v[q][D + d] : box[D + d];
+            }
+        }
+        wide = !near;
+    }
+    unsigned long long todo = __ballot(wide);
+    while (todo) {
+        const int src = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const size_t first = __shfl(b_lo, src, kWave) + 1, last = __shfl(b_hi, src, kWave) - 1;
+        Enc acc[2 * D];
+        for (int d = 0; d < D; ++d) { acc[d] = OrderedInt<T>::kEmptyLo; acc[D + d] = OrderedInt<T>::kEmptyHi; }
+        for (size_t b0 = first; b0 <= last; b0 += 4 * kWave) {
+            Enc v[4][2 * D];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const size_t b = b0 + q * kWave + lane;
+                const Enc* from = block_union(b <= last ? b : first);
+                for (int d = 0; d < 2 * D; ++d) v[q][d] = from[d];
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                for (int d = 0; d < D; ++d) {
+                    acc[d] = v[q][d] < acc[d] ? v[q][d] : acc[d];
+                    acc[D + d] = v[q][D + d] > acc[D + d] ? v[q][D + d] : acc[D + d];
+                }
+        }
+        for (int d = 0; d < D; ++d) { acc[d] = wave_min(acc[d]); acc[D + d] = wave_max(acc[D + d]); }
+        if (lane == src)
+            for (int d = 0; d < D; ++d) {
+                box[d] = acc[d] < box[d] ? acc[d] : box[d];
+                box[D + d] = acc[D + d] > box[D + d] ? acc[D + d] : box[D + d];
+            }
+    }
+    if (!active) return;
+    T out[2 * D];
+    for (int d = 0; d < 2 * D; ++d) out[d] = from_ordered_bits(box[d]);
+    if (far) {
+        T* own = node_box + (bl * n_nodes + node) * 2 * D;
+        for (int d = 0; d < 2 * D; ++d) own[d] = out[d];
+    }
+    if (up >= 0 && up < M - 1) {
+        T* dst = child_box + ((bl * (M - 1) + up) * 2 + side) * 2 * D;
+        for (int d = 0; d < 2 * D; ++d) dst[d] = out[d];
     }
 }
 
@@ -965,13 +1034,6 @@ template <typename T> struct SmallBuild {
     double threshold;
     int mode, covariance_form, M, N, per_mixture /* 64-point groups per mixture */, sort_points;
     unsigned tree_blocks;
-};
-
-template <typename T> struct OrderedInt;
-template <> struct OrderedInt<float> { using type = int; static constexpr int kEmptyLo = 0x7fffffff, kEmptyHi = -0x7fffffff - 1; };
-template <> struct OrderedInt<double> {
-    using type = long long;
-    static constexpr long long kEmptyLo = 0x7fffffffffffffffll, kEmptyHi = -0x7fffffffffffffffll - 1;
 };
 
 // Morton order of one segment of at most kCoarseOrderMax query points by the top 8 bits of their keys, stable.  Wavefront
@@ -1188,7 +1250,11 @@ __device__ __forceinline__ void build_small_tree(const T* __restrict__ mixture, 
         }
     }
     tree_sync<THREADS>();
-    // bottom-up unions: every leaf merges its own box into its ancestors until one already contains it (see bvh_merge_kernel)
+    // Bottom-up unions without inter-lane ordering: every leaf walks towards the root and merges ITS OWN box into every
+    // ancestor with atomic min/max, as long as it still enlarges the ancestor; it stops at the first ancestor that
+    // already contains it.  Every extreme of that ancestor was set by some walker that enlarged it and therefore walks
+    // on itself, so all higher ancestors end up containing the stopped box as well: the final boxes are the exact
+    // unions of the leaves below each node.  Nothing is read back before the barrier except the atomics' own results.
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const int i = tid + k * THREADS;
@@ -2274,7 +2340,9 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     T* node_box = (T*)(bvh + lay.node_box); T* leaf_rec = (T*)(bvh + lay.leaf_rec);
     int2* children = (int2*)(bvh + lay.children); int* parent = (int*)(bvh + lay.parent);
     int2* node_range = (int2*)(bvh + lay.node_range);
-    int* leaf_comp = (int*)(bvh + lay.leaf_comp); long long* enc_box = (long long*)(bvh + lay.enc_box);
+    int* leaf_comp = (int*)(bvh + lay.leaf_comp);
+    using Enc = typename OrderedInt<T>::type;
+    Enc* run_box = (Enc*)(bvh + lay.run_box);
     uint32_t* ka = (uint32_t*)(bvh + lay.keys_a); uint32_t* kb = (uint32_t*)(bvh + lay.keys_b);
     uint32_t* va = (uint32_t*)(bvh + lay.vals_a); uint32_t* vb = (uint32_t*)(bvh + lay.vals_b);
     uint32_t* pka = (uint32_t*)(bvh + lay.pkeys_a); uint32_t* pkb = (uint32_t*)(bvh + lay.pkeys_b);
@@ -2356,20 +2424,16 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     }
     if (have_g) {
         const size_t n = BL * M;
-        const unsigned leaf_blocks = 2 * grid_for(n);
-        bvh_leaves_kernel<T, D><<<dim3(leaf_blocks + jp_first.blocks), dim3(kBlock), 0, st>>>(mixture, box_lo, box_hi,
-                                                                                  double(cfg.aabb_threshold), cfg.aabb_mode, g_order, g_keys,
-                                                                           node_box, leaf_rec, enc_box, children, parent, node_range, M, n,
-                                                                           cfg.covariance_form != 0, (T*)(bvh + lay.sums), leaf_blocks, jp_first);
+        const unsigned leaf_blocks = unsigned((n + kBoxBlock - 1) / kBoxBlock);
+        bvh_leaves_kernel<T, D><<<dim3(leaf_blocks + jp_first.blocks), dim3(kBlock), 0, st>>>(
+            mixture, box_lo, box_hi, double(cfg.aabb_threshold), cfg.aabb_mode, g_order, g_keys, node_box, leaf_rec, run_box,
+            children, parent, node_range, M, n, cfg.covariance_form != 0, (T*)(bvh + lay.sums), leaf_blocks, jp_first);
         if (M > 1) {
-            const size_t ni = BL * (M - 1);
-            const unsigned merge_blocks = unsigned((n + kMergeBlock - 1) / kMergeBlock);
-            const unsigned frontier_blocks = unsigned((BL + kMergeBlock / kWave - 1) / (kMergeBlock / kWave));
-            bvh_merge_kernel<T, D><<<dim3(merge_blocks + jp_second.blocks + frontier_blocks), dim3(kMergeBlock), 0, st>>>(
-                parent, node_range, node_box, enc_box, M, n, merge_blocks, jp_second, children,
-                (int*)(bvh + lay.frontier), BL);
-            bvh_child_boxes_kernel<T, D><<<dim3(grid_for(ni)), dim3(kBlock), 0, st>>>(
-                children, enc_box, node_box, child_box, M, ni, candidate_cache(bvh, lay), lay.point_groups);
+            const size_t nn = BL * (2 * size_t(M) - 1);
+            const unsigned frontier_blocks = unsigned((BL + kBlock / kWave - 1) / (kBlock / kWave));
+            bvh_child_boxes_kernel<T, D><<<dim3(grid_for(nn) + jp_second.blocks + frontier_blocks), dim3(kBlock), 0, st>>>(
+                children, parent, node_range, run_box, node_box, child_box, M, nn, candidate_cache(bvh, lay), lay.point_groups,
+                grid_for(nn), jp_second, (int*)(bvh + lay.frontier), BL);
         } else if (jp_second.blocks > 0) {           // single leaves have no boxes to merge
             radix_scatter_kernel<<<dim3(jp_second.blocks), dim3(kBlock), 0, st>>>(jp_second, none);
         }
