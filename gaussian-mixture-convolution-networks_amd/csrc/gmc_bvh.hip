@@ -597,8 +597,15 @@ __global__ __launch_bounds__(kBlock) void radix_scatter_kernel(SortJob a, SortJo
     else radix_scatter_pass(b, blockIdx.x - a.blocks);
 }
 
+// orders the LDS traffic of one wavefront: stores of some lanes before loads of other lanes
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // ---------------------------------------------------------------------------------------------------------------
-// leaves, radix tree, bottom-up boxes
+// leaves, radix tree, boxes
 // ---------------------------------------------------------------------------------------------------------------
 // Order-preserving map from a floating-point value to a signed 64-bit integer (a < b <=> ordered(a) < ordered(b)),
 // so that box unions can be formed with integer atomic min/max.
@@ -773,8 +780,8 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
     const size_t bl = t < total ? t / M : 0;
     const int leaf = int(t - bl * M);
     // The searches of a node (its range, its split) read keys at distances 1, 2, 4 ... from the node, each read after
-    // the one before: the keys around the block wait in LDS, only the long steps of the few nodes with long ranges go
-    // to memory.
+    // the one before: the keys around the block wait in LDS, only the long steps of the nodes with long ranges go to
+    // memory.  (Measured with all 16384 keys of a tree in LDS: the fetch costs more than the remaining memory reads.)
     constexpr int kBefore = 192, kWindow = 2 * kBlock;
     __shared__ uint32_t window[kWindow];
     const long long window_first = (long long)first_leaf - kBefore;
@@ -810,15 +817,22 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         range_hi = int(hi - first_leaf);
     }
     __syncthreads();
-    for (int k = 1; k < kLevels; ++k) {
-        const int half = 1 << (k - 1);
-        for (int e = threadIdx.x; e < 2 * D * kBoxBlock; e += kBlock) {
-            const int c = e / kBoxBlock, i = e - c * kBoxBlock;
-            const Enc a = table[k - 1][c][i];
-            const Enc b = i + half < kBoxBlock ? table[k - 1][c][i + half] : a;    // (runs that leave the block are never read)
-            table[k][c][i] = c < D ? (b < a ? b : a) : (b > a ? b : a);
+    {
+        // lane (i, h): entry i of every level, the lower bounds (h = 0: minima) or the upper bounds (h = 1: maxima); the
+        // entry of the level before stays in registers
+        const int h = threadIdx.x >> 7;
+        Enc run[D];
+        for (int d = 0; d < D; ++d) run[d] = table[0][h * D + d][idx];
+        for (int k = 1; k < kLevels; ++k) {
+            const int other = idx + (1 << (k - 1));
+            if (other < kBoxBlock)                           // (runs that leave the block are never read)
+                for (int d = 0; d < D; ++d) {
+                    const Enc b = table[k - 1][h * D + d][other];
+                    run[d] = h == 0 ? (b < run[d] ? b : run[d]) : (b > run[d] ? b : run[d]);
+                }
+            for (int d = 0; d < D; ++d) table[k][h * D + d][idx] = run[d];
+            __syncthreads();
         }
-        __syncthreads();
     }
     // union of the leaf boxes in slots a ... b of the block
     auto range_union = [&](int a, int b, Enc (&out)[2 * D]) {
@@ -845,13 +859,6 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         range_union(idx, kBoxBlock - 1, u);
         for (int c = 0; c < 2 * D; ++c) dst[2 * D + c] = u[c];
     }
-}
-
-// orders the LDS traffic of one wavefront: stores of some lanes before loads of other lanes
-__device__ __forceinline__ void wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 template <typename T>
@@ -2354,7 +2361,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     int* p_order = (int*)(bvh + lay.p_order);
     const bool have_g = BL > 0 && M > 0, have_p = XL > 0 && N > 0;
     const bool sort_p = have_p && xes != nullptr;
-    if (g_build_path != 1 && have_g && M <= kSmallTreeMax && (!sort_p || N <= kCoarseOrderMax) && BL + XL < (size_t(1) << 31)) {
+    if (g_build_path == 0 && have_g && M <= kSmallTreeMax && (!sort_p || N <= kCoarseOrderMax) && BL + XL < (size_t(1) << 31)) {
         const CandidateCache cache = candidate_cache(bvh, lay);
         SmallBuild<T> a{box_lo, box_hi, node_box, child_box, leaf_rec, (T*)(bvh + lay.sums), children, parent, node_range,
                         leaf_comp, g_keys, (int*)(bvh + lay.frontier), p_order, cache.count, (int*)(bvh + lay.cand_ctl),
@@ -2388,10 +2395,10 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
             (uint32_t*)(bvh + lay.hist_g), lay.hist_words);
     const int p_passes = N > kCoarseOrderMax ? 2 : 1;
     auto jobs_of_pass = [&](int pass, SortJob& jg, SortJob& jp) {
-        jg = sort_job(ka, va, kb, vb, g_keys, g_order, (uint32_t*)(bvh + lay.hist_g), have_g ? BL : 0, M, 0, 4, pass, (int*)(bvh + lay.cand_ctl));
+        jg = sort_job(ka, va, kb, vb, g_keys, g_order, (uint32_t*)(bvh + lay.hist_g), have_g ? BL : 0, M, 0, 4, pass, (int*)(bvh + lay.cand_ctl) + 2);
         jp = sort_job(pka, pva, pkb, pvb, p_passes == 1 ? pkb : pka, (uint32_t*)p_order,
                       (uint32_t*)(bvh + lay.hist_p), sort_p ? XL : 0, N, 30 - 8 * p_passes, p_passes, pass,
-                      (int*)(bvh + lay.cand_ctl));
+                      (int*)(bvh + lay.cand_ctl) + 2);
     };
     SortJob jg0, jp0;
     jobs_of_pass(0, jg0, jp0);

@@ -526,32 +526,37 @@ def test_one_launch_build_gives_the_trees_of_the_chain_of_launches(dtype, D):
     larger ones by a chain of launches; with the chain forced for the same inputs every integer and every box of the
     object must be identical: leaf order and Morton codes, children and parents, node boxes, per-Gaussian boxes.  The
     culled sums agree to rounding (the Morton order of the query points, hence the order of additions, may differ)."""
-    lib = _native.lib()
     for k, (B, L, M, N) in enumerate(((3, 2, 1, 50), (2, 2, 2, 10), (2, 3, 3, 70), (5, 4, 64, 700), (3, 3, 65, 1100), (4, 2, 128, 784),
                                       (2, 2, 129, 4096), (2, 2, 257, 300), (1, 2, 700, 5000), (1, 1, 1024, 8192))):
         mix, xes, gout = _case(B, L, M, N, D, seed=7300 + k)
         if k == 3:
             mix[:, :, 5:30] = mix[:, :, 5:6]               # identical Gaussians: equal keys, ties broken by the component index
         m, x = mix.to(dtype).to(DEV).contiguous(), xes.to(dtype).to(DEV).contiguous()
-        got = []
-        for path in (0, 1):
-            lib.gmc_bvh_set_build_path(path)
-            try:
-                bvh = _native.Bvh(m, x, 0.001, "reference")
-                lo, up = bvh.boxes()
-                nodes, nb = bvh.nodes()
-                keys, comps = bvh.leaf_order()
-                out = _native.eval_bvh_fwd(m, x, bvh)
-                gmix, gxes = _native.eval_bvh_bwd(gout.to(dtype).to(DEV), m, x, bvh, True, True)
-                torch.cuda.synchronize()
-                assert n_errors(bvh) == 0
-                got.append([t.cpu().numpy() for t in (lo, up, nodes, nb, keys, comps, out, gmix, gxes)])
-            finally:
-                lib.gmc_bvh_set_build_path(0)
-        for a, b, what in zip(got[0][:6], got[1][:6], ("lower", "upper", "nodes", "node boxes", "keys", "components")):
-            assert np.array_equal(a, b), f"{what} differ between the two build paths, B{B} L{L} M{M} N{N} D{D}"
-        for a, b, what in zip(got[0][6:], got[1][6:], ("out", "grad mixture", "grad xes")):
-            assert rel_l2(a, b, FLOOR[dtype]) <= TOL[dtype], what
+        _same_object_by_both_paths(m, x, gout.to(dtype).to(DEV), dtype, (0, 1), f"B{B} L{L} M{M} N{N} D{D}")
+
+
+def _same_object_by_both_paths(m, x, g, dtype, paths, tag):
+    """builds, evaluates and differentiates with each of the two build paths; integers and boxes must be identical"""
+    lib = _native.lib()
+    got = []
+    for path in paths:
+        lib.gmc_bvh_set_build_path(path)
+        try:
+            bvh = _native.Bvh(m, x, 0.001, "reference")
+            lo, up = bvh.boxes()
+            nodes, nb = bvh.nodes()
+            keys, comps = bvh.leaf_order()
+            out = _native.eval_bvh_fwd(m, x, bvh)
+            gmix, gxes = _native.eval_bvh_bwd(g, m, x, bvh, True, True)
+            torch.cuda.synchronize()
+            assert n_errors(bvh) == 0
+            got.append([t.cpu().numpy() for t in (lo, up, nodes, nb, keys, comps, out, gmix, gxes)])
+        finally:
+            lib.gmc_bvh_set_build_path(0)
+    for a, b, what in zip(got[0][:6], got[1][:6], ("lower", "upper", "nodes", "node boxes", "keys", "components")):
+        assert np.array_equal(a, b), f"{what} differ between the build paths {paths}, {tag}"
+    for a, b, what in zip(got[0][6:], got[1][6:], ("out", "grad mixture", "grad xes")):
+        assert rel_l2(a, b, FLOOR[dtype]) <= TOL[dtype], what
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
@@ -563,7 +568,8 @@ def test_leaf_order_is_bit_exact(dtype, D):
     the codes.  Compared bit for bit with the oracle, duplicate codes (identical and nearly identical centres),
     clustered centres and several mixtures included."""
     npdt = np.float32 if dtype == torch.float32 else np.float64
-    for M, seed, spread in ((1, 1, 4.0), (2, 2, 4.0), (37, 3, 4.0), (300, 4, 0.01), (1000, 5, 4.0), (5000, 6, 50.0)):
+    for M, seed, spread in ((1, 1, 4.0), (2, 2, 4.0), (37, 3, 4.0), (300, 4, 0.01), (1000, 5, 4.0), (1500, 7, 4.0), (3000, 8, 0.5),
+                            (5000, 6, 50.0), (9000, 9, 4.0), (16384, 10, 4.0), (16385, 11, 4.0)):
         mix, xes, _ = _case(2, 3, M, 70, D, seed=1200 + seed, spread=spread)
         if M >= 37:
             mix[:, :, 5:25] = mix[:, :, 5:6]                       # identical centres: identical codes, tie order matters
