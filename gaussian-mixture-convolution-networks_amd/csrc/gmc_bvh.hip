@@ -487,6 +487,7 @@ struct SortJob {
     int count, items, blocks_per_seg, shift, chunk_shift;
     unsigned blocks;                     // workgroups of this job in the launch
     int* err;                            // error flags of the BVH object
+    uint32_t* digit_start;               // [segments][256] first output slot of every digit, written if not null
 };
 
 // One pass of the sort by workgroup `id` of job j (all kBlock lanes of the workgroup call it).  The block histograms of
@@ -548,6 +549,7 @@ __device__ __forceinline__ void radix_scatter_pass(const SortJob& j, unsigned id
     __syncthreads();
     for (int w = 0; w < wave; ++w) scan += wave_total[w];
     running[threadIdx.x] = scan - mine + earlier;
+    if (j.digit_start && blk == 0) j.digit_start[size_t(seg) * 256 + threadIdx.x] = scan - mine;
     __syncthreads();
     for (int round = 0; round < j.items; ++round) {
         const int i = begin + round * kBlock + threadIdx.x;
@@ -602,6 +604,55 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Second half of the leaves' sort for one or two large trees (kBucketSortMin < M <= kBucketSortMax): after ONE radix
+// pass over the top 8 key bits the keys of a digit lie together (their first slots in digit_start), and a workgroup per
+// digit sorts them in LDS by the unique key (Morton code << 32 | component), which is the stable order of the codes --
+// a bitonic network on the next power of two.  Two launches instead of four, each at its latency floor; a digit that
+// holds most keys (all centres in one cell) is one long sort by a single workgroup: slower than the four passes, same
+// result.
+constexpr int kBucketSortLanes = 1024;
+constexpr int kBucketSortMax = 16384;
+constexpr int kBucketSortSegments = 2;     // more trees than this: the grid of 256 workgroups per tree would queue up
+
+template <int CAP>
+__global__ __launch_bounds__(kBucketSortLanes) void bucket_sort_kernel(const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
+                                                                      uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
+                                                                      const uint32_t* __restrict__ digit_start, int count, int* __restrict__ err) {
+    __shared__ unsigned long long k[CAP];
+    const int seg = blockIdx.x >> 8, digit = blockIdx.x & 255;
+    const uint32_t begin = digit_start[size_t(seg) * 256 + digit];
+    const uint32_t end = digit < 255 ? digit_start[size_t(seg) * 256 + digit + 1] : uint32_t(count);
+    if (end <= begin) return;                                // (the same for every lane of the workgroup)
+    const int n = int(end - begin);
+    if (end > uint32_t(count) || n > CAP) {                 // never, for a consistent histogram
+        if (threadIdx.x == 0) atomicOr(err, kErrSort);
+        return;
+    }
+    const size_t at = size_t(seg) * count + begin;
+    int np = 2;
+    while (np < n) np <<= 1;
+    // up to 128 keys: one wavefront, no workgroup barriers
+    const bool single = np <= 2 * kWave;
+    if (single && threadIdx.x >= kWave) return;
+    const int lanes = single ? kWave : kBucketSortLanes;
+    for (int i = threadIdx.x; i < np; i += lanes)
+        k[i] = i < n ? ((unsigned long long)keys_in[at + i] << 32) | vals_in[at + i] : ~0ull;
+    if (single) wave_lds_fence(); else __syncthreads();
+    for (int size = 2; size <= np; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int q = threadIdx.x; q < np / 2; q += lanes) {
+                const int i0 = ((q & ~(stride - 1)) << 1) | (q & (stride - 1)), i1 = i0 | stride;
+                const unsigned long long k0 = k[i0], k1 = k[i1];
+                if ((k0 > k1) == ((i0 & size) == 0)) { k[i0] = k1; k[i1] = k0; }
+            }
+            if (single) wave_lds_fence(); else __syncthreads();
+        }
+    for (int i = threadIdx.x; i < n; i += lanes) {
+        keys_out[at + i] = uint32_t(k[i] >> 32);
+        vals_out[at + i] = uint32_t(k[i]);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1032,7 +1083,8 @@ __global__ __launch_bounds__(kBlock) void bvh_child_boxes_kernel(const int2* __r
 // the top 8 key bits).  Same trees and boxes as the chain of launches, bit for bit; the order of the points may differ
 // where a point lies on the border of a Morton cell (any order of the points gives the same sums).
 constexpr int kSmallTreeMax = 1024;
-static int g_build_path = 0;            // test knob (gmc_bvh_set_build_path): 1 = always the chain of launches
+static int g_build_path = 0;            // test knob (gmc_bvh_set_build_path): 1 = always the chain of launches, 2 = and the
+                                        // leaves' sort always as four radix passes
 
 template <typename T> struct SmallBuild {
     T* box_lo; T* box_hi; T* node_box; T* child_box; T* leaf_rec; T* sums;
@@ -2403,6 +2455,14 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     SortJob jg0, jp0;
     jobs_of_pass(0, jg0, jp0);
     MortonJob<T> mg = {}, mp = {};
+    // one or two large trees: one radix pass over the top 8 key bits, then every digit sorted in LDS (bucket_sort_kernel)
+    const bool bucket_sort = have_g && g_build_path != 2 && M > kSmallTreeMax && M <= kBucketSortMax && BL <= size_t(kBucketSortSegments);
+    if (bucket_sort) {
+        jg0.shift = 22;
+        jg0.keys_out = kb; jg0.vals_out = vb;
+        jg0.hist_next = nullptr;
+        jg0.digit_start = (uint32_t*)(bvh + lay.hist_g) + BL * size_t(jg0.blocks_per_seg) * 256;     // (the second pass's histograms)
+    }
     if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm),
                                   (uint32_t*)jg0.hist, jg0.blocks_per_seg, jg0.chunk_shift, jg0.shift};
     if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx),
@@ -2422,8 +2482,17 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         jobs_of_pass(pass, jg, jp);
         if (pass == 0) jp_first = jp;
         if (pass == 1) jp_second = jp;
-        if (jg.blocks == 0) continue;
+        if (jg.blocks == 0 || bucket_sort) continue;
         radix_scatter_kernel<<<dim3(jg.blocks), dim3(kBlock), 0, st>>>(jg, none);
+    }
+    if (bucket_sort) {
+        radix_scatter_kernel<<<dim3(jg0.blocks), dim3(kBlock), 0, st>>>(jg0, none);
+        const dim3 grid{unsigned(BL * 256)}, block{unsigned(kBucketSortLanes)};
+        int* err = (int*)(bvh + lay.cand_ctl) + 2;
+        if (M <= 2048) bucket_sort_kernel<2048><<<grid, block, 0, st>>>(kb, vb, g_keys, g_order, jg0.digit_start, M, err);
+        else if (M <= 4096) bucket_sort_kernel<4096><<<grid, block, 0, st>>>(kb, vb, g_keys, g_order, jg0.digit_start, M, err);
+        else if (M <= 8192) bucket_sort_kernel<8192><<<grid, block, 0, st>>>(kb, vb, g_keys, g_order, jg0.digit_start, M, err);
+        else bucket_sort_kernel<16384><<<grid, block, 0, st>>>(kb, vb, g_keys, g_order, jg0.digit_start, M, err);
     }
     if (!have_g) {                                   // no trees to build: the points' passes are launches of their own
         if (jp_first.blocks > 0) radix_scatter_kernel<<<dim3(jp_first.blocks), dim3(kBlock), 0, st>>>(jp_first, none);
@@ -2590,7 +2659,7 @@ static int bvh_export_t(const char* bvh, T* lower, T* upper, int32_t* nodes, T* 
 
 extern "C" {
 
-void gmc_bvh_set_build_path(int path) { gmc::g_build_path = path == 1 ? 1 : 0; }
+void gmc_bvh_set_build_path(int path) { gmc::g_build_path = path == 1 || path == 2 ? path : 0; }
 void gmc_bvh_set_eval_path(int path) { gmc::g_eval_path = path == 1 ? 1 : 0; }
 
 size_t gmc_bvh_bytes(const gmc_shape* shape) {

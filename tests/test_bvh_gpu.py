@@ -560,6 +560,23 @@ def _same_object_by_both_paths(m, x, g, dtype, paths, tag):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_sort_by_digits_in_lds_gives_the_order_of_the_four_radix_passes(dtype):
+    """The leaves of one or two trees of 1025 ... 16384 components are sorted by one radix pass over the top 8 key bits
+    and a sort of every digit in LDS, all others by four radix passes; with the latter forced for the same inputs the
+    objects must be identical.  Sizes at both ends of every LDS capacity, duplicate keys, and centres crowded into a
+    few cells (one digit holds most keys) included."""
+    for k, (B, L, M, N, D) in enumerate(((2, 1, 1025, 300, 2), (1, 2, 2048, 100, 3), (1, 2, 2049, 100, 2), (2, 1, 4096, 200, 3),
+                                         (1, 1, 4100, 100, 3), (1, 1, 8192, 9000, 2), (1, 2, 12000, 100, 3), (1, 1, 16384, 500, 3))):
+        mix, xes, gout = _case(B, L, M, N, D, seed=7500 + k)
+        mix[:, :, 40:300] = mix[:, :, 40:41]                # identical Gaussians: equal keys, ties broken by the component index
+        mix[-1, -1, 1::2, 1:1 + D] *= 1e-3                  # half the centres of one mixture crowd into a few cells
+        if k == 4:
+            mix[..., 1:1 + D] = mix[:, :, :1, 1:1 + D]      # all centres in one point: one digit, one key
+        m, x = mix.to(dtype).to(DEV).contiguous(), xes.to(dtype).to(DEV).contiguous()
+        _same_object_by_both_paths(m, x, gout.to(dtype).to(DEV), dtype, (0, 2), f"B{B} L{L} M{M} N{N} D{D}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("D", [2, 3])
 def test_leaf_order_is_bit_exact(dtype, D):
     """Integer part of the build: the 30-bit Morton codes of the centres (lbvh/morton_code.h:77-85,145-168, positions
@@ -570,12 +587,13 @@ def test_leaf_order_is_bit_exact(dtype, D):
     npdt = np.float32 if dtype == torch.float32 else np.float64
     for M, seed, spread in ((1, 1, 4.0), (2, 2, 4.0), (37, 3, 4.0), (300, 4, 0.01), (1000, 5, 4.0), (1500, 7, 4.0), (3000, 8, 0.5),
                             (5000, 6, 50.0), (9000, 9, 4.0), (16384, 10, 4.0), (16385, 11, 4.0)):
-        mix, xes, _ = _case(2, 3, M, 70, D, seed=1200 + seed, spread=spread)
+        B, L = (2, 3) if M < 1500 or M == 5000 else (1, 2)          # (one or two large trees take a sort path of their own)
+        mix, xes, _ = _case(B, L, M, 70, D, seed=1200 + seed, spread=spread)
         if M >= 37:
             mix[:, :, 5:25] = mix[:, :, 5:6]                       # identical centres: identical codes, tie order matters
             mix[:, :, 25:30, 1:1 + D] = mix[:, :, 25:26, 1:1 + D] * (1 + 1e-7)
         if M >= 300:
-            mix[:, 1, ::2, 1:1 + D] *= 1e-3                        # half the centres crowd into a few cells
+            mix[:, -1, ::2, 1:1 + D] *= 1e-3                       # half the centres crowd into a few cells
         m = mix.to(dtype).to(DEV).contiguous()
         bvh = _native.Bvh(m, xes.to(dtype).to(DEV).contiguous(), 0.001, "tight")
         keys, comps = bvh.leaf_order()
