@@ -442,7 +442,7 @@ template <typename T> struct MortonJob {
     const T* parts; int n_parts;                                   // partial bounds of every segment
     uint32_t* keys; uint32_t* vals;
     unsigned blocks;                                               // workgroups of this job in the launch
-    uint32_t* hist; int sort_blocks_per_seg, sort_chunk_shift, shift;   // block histograms of the first radix pass
+    uint32_t* hist; int sort_blocks_per_seg, sort_chunk_shift, shift;   // block histograms of the first radix pass (null: none wanted)
 };
 
 // Morton keys and index payload for two jobs in one launch (job b behind job a); every workgroup first combines
@@ -473,7 +473,7 @@ __global__ __launch_bounds__(kBlock) void morton_kernel(MortonJob<T> a, MortonJo
     const uint32_t key = morton30<T, D>(j.pts + at * j.stride + j.offset, bounds);
     j.keys[at] = key;
     j.vals[at] = uint32_t(i);
-    atomicAdd(&j.hist[(size_t(seg) * j.sort_blocks_per_seg + (i >> j.sort_chunk_shift)) * 256 + ((key >> j.shift) & 255u)], 1u);
+    if (j.hist) atomicAdd(&j.hist[(size_t(seg) * j.sort_blocks_per_seg + (i >> j.sort_chunk_shift)) * 256 + ((key >> j.shift) & 255u)], 1u);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -487,7 +487,6 @@ struct SortJob {
     int count, items, blocks_per_seg, shift, chunk_shift;
     unsigned blocks;                     // workgroups of this job in the launch
     int* err;                            // error flags of the BVH object
-    uint32_t* digit_start;               // [segments][256] first output slot of every digit, written if not null
 };
 
 // One pass of the sort by workgroup `id` of job j (all kBlock lanes of the workgroup call it).  The block histograms of
@@ -549,7 +548,6 @@ __device__ __forceinline__ void radix_scatter_pass(const SortJob& j, unsigned id
     __syncthreads();
     for (int w = 0; w < wave; ++w) scan += wave_total[w];
     running[threadIdx.x] = scan - mine + earlier;
-    if (j.digit_start && blk == 0) j.digit_start[size_t(seg) * 256 + threadIdx.x] = scan - mine;
     __syncthreads();
     for (int round = 0; round < j.items; ++round) {
         const int i = begin + round * kBlock + threadIdx.x;
@@ -606,40 +604,95 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Second half of the leaves' sort for one or two large trees (kBucketSortMin < M <= kBucketSortMax): after ONE radix
-// pass over the top 8 key bits the keys of a digit lie together (their first slots in digit_start), and a workgroup per
-// digit sorts them in LDS by the unique key (Morton code << 32 | component), which is the stable order of the codes --
-// a bitonic network on the next power of two.  Two launches instead of four, each at its latency floor; a digit that
+// The leaves' sort for one or two large trees (kSmallTreeMax < M <= kBucketSortMax) in ONE launch instead of four radix
+// passes at their latency floor: 256 workgroups per tree, one per value of the top 8 key bits.  Workgroup d reads all
+// keys of the tree (in component order, as the Morton kernel wrote them; 64 KB at most, from L2), keeps those whose top
+// bits are d as unique keys (Morton code << 32 | component) in LDS, counts those with smaller top bits -- the first
+// slot of its own --, sorts its keys (by counting ranks; more than kBucketRankMax: a bitonic network) and writes them out: ascending
+// unique keys are the stable order of the codes.  No histograms, no passes that wait for each other.  A digit that
 // holds most keys (all centres in one cell) is one long sort by a single workgroup: slower than the four passes, same
 // result.
 constexpr int kBucketSortLanes = 1024;
 constexpr int kBucketSortMax = 16384;
+constexpr int kBucketRankMax = 256;        // keys of one digit up to which counting ranks beats the sorting network
 constexpr int kBucketSortSegments = 2;     // more trees than this: the grid of 256 workgroups per tree would queue up
 
 template <int CAP>
-__global__ __launch_bounds__(kBucketSortLanes) void bucket_sort_kernel(const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
-                                                                      uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
-                                                                      const uint32_t* __restrict__ digit_start, int count, int* __restrict__ err) {
+__global__ __launch_bounds__(kBucketSortLanes) void bucket_sort_kernel(const uint32_t* __restrict__ keys_in, uint32_t* __restrict__ keys_out,
+                                                                      uint32_t* __restrict__ vals_out, int count, int* __restrict__ err) {
+    constexpr int kPerLane = CAP / kBucketSortLanes;         // keys of the tree per lane, at most
     __shared__ unsigned long long k[CAP];
-    const int seg = blockIdx.x >> 8, digit = blockIdx.x & 255;
-    const uint32_t begin = digit_start[size_t(seg) * 256 + digit];
-    const uint32_t end = digit < 255 ? digit_start[size_t(seg) * 256 + digit + 1] : uint32_t(count);
-    if (end <= begin) return;                                // (the same for every lane of the workgroup)
-    const int n = int(end - begin);
-    if (end > uint32_t(count) || n > CAP) {                 // never, for a consistent histogram
+    __shared__ int n_mine, n_before;
+    const int seg = blockIdx.x >> 8, lane = threadIdx.x & 63;
+    const uint32_t digit = blockIdx.x & 255;
+    const uint32_t* in = keys_in + size_t(seg) * count;
+    if (threadIdx.x == 0) { n_mine = 0; n_before = 0; }
+    static_assert(kPerLane % 4 == 0 || kPerLane == 2, "keys are fetched four (two) at a time");
+    constexpr int kVec = kPerLane == 2 ? 2 : 4, kLoads = kPerLane / kVec;
+    uint32_t key[kPerLane];
+    // (a second segment may start off a multiple of the vector width: key by key then)
+    const bool wide = (size_t(seg) * count) % kVec == 0;
+#pragma unroll
+    for (int r = 0; r < kLoads; ++r) {                       // all loads in flight together
+        const int i = (r * kBucketSortLanes + threadIdx.x) * kVec;
+        if (wide && i + kVec <= count) {
+            if constexpr (kVec == 4) {
+                const uint4 v = *reinterpret_cast<const uint4*>(in + i);
+                key[4 * r] = v.x; key[4 * r + 1] = v.y; key[4 * r + 2] = v.z; key[4 * r + 3] = v.w;
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2*>(in + i);
+                key[2 * r] = v.x; key[2 * r + 1] = v.y;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < kVec; ++c) key[kVec * r + c] = i + c < count ? in[i + c] : 0xffffffffu;   // (real keys have 30 bits)
+        }
+    }
+    __syncthreads();
+    int before = 0;
+#pragma unroll
+    for (int r = 0; r < kPerLane; ++r) {
+        const int i = ((r / kVec) * kBucketSortLanes + threadIdx.x) * kVec + r % kVec;      // the component of this key
+        const uint32_t top = key[r] >> 22;
+        before += top < digit ? 1 : 0;
+        const bool mine = top == digit;
+        const unsigned long long m = __ballot(mine);
+        if (m != 0ull) {                                     // (the order inside the digit does not matter: the keys are unique)
+            int base = 0;
+            if (lane == __ffsll((long long)m) - 1) base = atomicAdd(&n_mine, __popcll(m));
+            base = __shfl(base, __ffsll((long long)m) - 1, kWave);
+            if (mine) k[base + __popcll(m & ((1ull << lane) - 1ull))] = ((unsigned long long)key[r] << 32) | uint32_t(i);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, kWave);
+    if (lane == 0 && before != 0) atomicAdd(&n_before, before);
+    __syncthreads();
+    const int n = n_mine, begin = n_before;
+    if (n == 0) return;                                      // (the same for every lane of the workgroup)
+    if (begin + n > count) {                                 // never
         if (threadIdx.x == 0) atomicOr(err, kErrSort);
         return;
     }
     const size_t at = size_t(seg) * count + begin;
+    if (n <= kBucketRankMax) {
+        // a few keys (the usual case: M / 256 on average): lane i counts the keys below key i and puts it there -- every
+        // read is a broadcast, no step waits for another
+        if (int(threadIdx.x) < n) {
+            const unsigned long long mine = k[threadIdx.x];
+            int rank = 0;
+#pragma unroll 8
+            for (int j = 0; j < n; ++j) rank += k[j] < mine ? 1 : 0;
+            keys_out[at + rank] = uint32_t(mine >> 32);
+            vals_out[at + rank] = uint32_t(mine);
+        }
+        return;
+    }
     int np = 2;
     while (np < n) np <<= 1;
-    // up to 128 keys: one wavefront, no workgroup barriers
-    const bool single = np <= 2 * kWave;
-    if (single && threadIdx.x >= kWave) return;
-    const int lanes = single ? kWave : kBucketSortLanes;
-    for (int i = threadIdx.x; i < np; i += lanes)
-        k[i] = i < n ? ((unsigned long long)keys_in[at + i] << 32) | vals_in[at + i] : ~0ull;
-    if (single) wave_lds_fence(); else __syncthreads();
+    constexpr int lanes = kBucketSortLanes;
+    for (int i = n + threadIdx.x; i < np; i += lanes) k[i] = ~0ull;
+    __syncthreads();
     for (int size = 2; size <= np; size <<= 1)
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             for (int q = threadIdx.x; q < np / 2; q += lanes) {
@@ -647,7 +700,7 @@ __global__ __launch_bounds__(kBucketSortLanes) void bucket_sort_kernel(const uin
                 const unsigned long long k0 = k[i0], k1 = k[i1];
                 if ((k0 > k1) == ((i0 & size) == 0)) { k[i0] = k1; k[i1] = k0; }
             }
-            if (single) wave_lds_fence(); else __syncthreads();
+            __syncthreads();
         }
     for (int i = threadIdx.x; i < n; i += lanes) {
         keys_out[at + i] = uint32_t(k[i] >> 32);
@@ -2455,16 +2508,10 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     SortJob jg0, jp0;
     jobs_of_pass(0, jg0, jp0);
     MortonJob<T> mg = {}, mp = {};
-    // one or two large trees: one radix pass over the top 8 key bits, then every digit sorted in LDS (bucket_sort_kernel)
+    // one or two large trees: every value of the top 8 key bits gathered and sorted in LDS (bucket_sort_kernel)
     const bool bucket_sort = have_g && g_build_path != 2 && M > kSmallTreeMax && M <= kBucketSortMax && BL <= size_t(kBucketSortSegments);
-    if (bucket_sort) {
-        jg0.shift = 22;
-        jg0.keys_out = kb; jg0.vals_out = vb;
-        jg0.hist_next = nullptr;
-        jg0.digit_start = (uint32_t*)(bvh + lay.hist_g) + BL * size_t(jg0.blocks_per_seg) * 256;     // (the second pass's histograms)
-    }
     if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm),
-                                  (uint32_t*)jg0.hist, jg0.blocks_per_seg, jg0.chunk_shift, jg0.shift};
+                                  bucket_sort ? nullptr : (uint32_t*)jg0.hist, jg0.blocks_per_seg, jg0.chunk_shift, jg0.shift};
     if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx),
                                   (uint32_t*)jp0.hist, jp0.blocks_per_seg, jp0.chunk_shift, jp0.shift};
     if (mg.blocks + mp.blocks > 0) morton_kernel<T, D><<<dim3(mg.blocks + mp.blocks), dim3(kBlock), 0, st>>>(mg, mp);
@@ -2486,13 +2533,12 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         radix_scatter_kernel<<<dim3(jg.blocks), dim3(kBlock), 0, st>>>(jg, none);
     }
     if (bucket_sort) {
-        radix_scatter_kernel<<<dim3(jg0.blocks), dim3(kBlock), 0, st>>>(jg0, none);
         const dim3 grid{unsigned(BL * 256)}, block{unsigned(kBucketSortLanes)};
         int* err = (int*)(bvh + lay.cand_ctl) + 2;
-        if (M <= 2048) bucket_sort_kernel<2048><<<grid, block, 0, st>>>(kb, vb, g_keys, g_order, jg0.digit_start, M, err);
-        else if (M <= 4096) bucket_sort_kernel<4096><<<grid, block, 0, st>>>(kb, vb, g_keys, g_order, jg0.digit_start, M, err);
-        else if (M <= 8192) bucket_sort_kernel<8192><<<grid, block, 0, st>>>(kb, vb, g_keys, g_order, jg0.digit_start, M, err);
-        else bucket_sort_kernel<16384><<<grid, block, 0, st>>>(kb, vb, g_keys, g_order, jg0.digit_start, M, err);
+        if (M <= 2048) bucket_sort_kernel<2048><<<grid, block, 0, st>>>(ka, g_keys, g_order, M, err);
+        else if (M <= 4096) bucket_sort_kernel<4096><<<grid, block, 0, st>>>(ka, g_keys, g_order, M, err);
+        else if (M <= 8192) bucket_sort_kernel<8192><<<grid, block, 0, st>>>(ka, g_keys, g_order, M, err);
+        else bucket_sort_kernel<16384><<<grid, block, 0, st>>>(ka, g_keys, g_order, M, err);
     }
     if (!have_g) {                                   // no trees to build: the points' passes are launches of their own
         if (jp_first.blocks > 0) radix_scatter_kernel<<<dim3(jp_first.blocks), dim3(kBlock), 0, st>>>(jp_first, none);
