@@ -7,12 +7,13 @@
 //   (lbvh/bvh.cu:460-510), so the result does not depend on tree shape, Morton resolution or sort order.
 //
 // Build, one tree per (b,l) mixture, all on device and without host synchronisation:
-//   boxes + centre bounds -> 30-bit Morton codes of the centres (lbvh/morton_code.h:77-85,145-168) -> segmented LSD
-//   radix sort (8 bits per pass, stable, keys uint32 + index payload) -> leaves in Morton order with their
-//   evaluation records -> Karras radix tree over the unique keys (morton << 32 | rank), as lbvh/building.h:11-103
-//   -> bottom-up union of boxes with integer atomic min/max on order-preserving encodings.
+//   centre bounds -> 30-bit Morton codes of the centres (lbvh/morton_code.h:77-85,145-168) -> stable sort of the codes
+//   (segmented LSD radix sort, 8 bits per pass; one or two large trees: one launch that sorts every value of the top 8
+//   key bits in LDS) -> leaves in Morton order with their boxes and evaluation records, Karras radix tree over the
+//   unique keys (morton << 32 | rank) as lbvh/building.h:11-103 -> boxes of the internal nodes as unions of the leaf
+//   boxes of their ranges (order-preserving integers: exactly the unions a bottom-up merge gives, lbvh/bvh.cu:460-510).
 // Query points are Morton-sorted the same way (on their top 16 or 8 key bits) so that a wavefront owns 64
-// neighbouring points; their two sort passes ride as extra workgroups in the two longest launches of the tree
+// neighbouring points; their two sort passes ride as extra workgroups in the two last launches of the tree
 // construction, and one wavefront per tree leaves a cut through the tree a few levels below the root (tree_frontier).
 //
 // Small trees take short cuts: mixtures of at most 1024 components (query points in segments of at most 8192) are built
@@ -2521,7 +2522,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     // land in a spare buffer, which must not be the input of the last pass.
     // The launches of the leaves' four passes are bound by their latency and would take twice as long with the six
     // times more numerous points in them; the points' passes ride in the two longest launches of the tree
-    // construction instead (leaf records + radix tree, box merge), which use a quarter of the compute units.
+    // construction instead (leaf records + radix tree, boxes), which use a quarter of the compute units.
     const SortJob none = {};
     SortJob jp_first = none, jp_second = none;
     for (int pass = 0; pass < 4; ++pass) {

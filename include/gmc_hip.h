@@ -175,8 +175,8 @@ int gmc_convolution_bwd(const void* grad_out, const void* data, const void* kern
 
 /* ---- LBVH-culled evaluation ------------------------------------------------------------------------
  * Replaces lbvh::Bvh<D,T> (src/gmc/cpp/extensions/lbvh/bvh.h:97-148, bvh.cu:24-144: per-Gaussian boxes from
- * the contribution cutoff, Morton codes, sort, Karras node build, bottom-up box merge) and the point query
- * lbvh::query_device_with_fun (lbvh/query.h:13-66) composed with the evaluation, i.e. the (absent)
+ * the contribution cutoff, Morton codes, sort, Karras node build, box unions of the internal nodes) and the point
+ * query lbvh::query_device_with_fun (lbvh/query.h:13-66) composed with the evaluation, i.e. the (absent)
  * cuda_bvh_forward / cuda_bvh_backward named at evaluate_inversed/test_evaluate_inversed.cpp:22-23:
  *   out[b,l,n] = sum over Gaussians m whose own box contains x_n (closed interval, lbvh/aabb.h:39-47).
  */
