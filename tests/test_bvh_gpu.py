@@ -210,6 +210,86 @@ def test_small_trees_many_mixtures(dtype):
         _check_culled(mix, xes, gout, dtype, "tight" if k % 2 else "reference", tag=f"B{B} L{L} M{M} N{N} D{D} bc{bc}")
 
 
+def _check_tree_on_the_host(nd, bx, ky, cp, lo, up, M, D, tag):
+    """One exported tree: nd [2M-1, 4] = parent, left, right, component-or--1 (internal nodes first, leaves in Morton
+    order), bx their boxes, ky / cp the sorted codes and the component of every leaf, lo / up the components' boxes."""
+    assert np.array_equal(np.sort(cp), np.arange(M)), tag + ": every component is exactly one leaf"
+    assert np.all(np.diff(ky) >= 0), tag + ": codes ascend"
+    assert np.all(np.diff(cp)[np.diff(ky) == 0] > 0), tag + ": equal codes in component order"
+    assert np.array_equal(nd[M - 1:, 3], cp), tag
+    assert np.array_equal(bx[M - 1:, :D], lo[cp]) and np.array_equal(bx[M - 1:, D:], up[cp]), tag + ": leaf boxes"
+    if M == 1:
+        return
+    par, left, right = nd[:, 0], nd[:M - 1, 1], nd[:M - 1, 2]
+    assert left.min() > 0 and right.min() > 0 and max(left.max(), right.max()) < 2 * M - 1, tag
+    assert np.array_equal(np.sort(np.concatenate([left, right])), np.arange(1, 2 * M - 1)), tag + ": one parent per node"
+    assert np.array_equal(par[left], np.arange(M - 1)) and np.array_equal(par[right], np.arange(M - 1)) and par[0] == -1, tag
+    assert np.array_equal(bx[:M - 1, :D], np.minimum(bx[left, :D], bx[right, :D])), tag + ": parent box = union (lower)"
+    assert np.array_equal(bx[:M - 1, D:], np.maximum(bx[left, D:], bx[right, D:])), tag + ": parent box = union (upper)"
+    # leaf ranges, accumulated level by level from the deepest nodes: the two children of a node cover adjacent ranges
+    depth = np.zeros(2 * M - 1, dtype=np.int64)
+    level, d = np.array([0]), 0
+    while level.size:
+        depth[level] = d
+        d += 1
+        assert d < 200, tag + ": depth"
+        inner = level[level < M - 1]
+        level = np.concatenate([left[inner], right[inner]])
+    size = np.zeros(2 * M - 1, dtype=np.int64); size[M - 1:] = 1
+    first = np.full(2 * M - 1, 1 << 40, dtype=np.int64); first[M - 1:] = np.arange(M)
+    for dd in range(int(depth.max()), 0, -1):
+        idx = np.nonzero(depth == dd)[0]
+        np.add.at(size, par[idx], size[idx])
+        np.minimum.at(first, par[idx], first[idx])
+    assert size[0] == M and first[0] == 0, tag + ": the root covers all leaves"
+    assert np.array_equal(first[left] + size[left], first[right]), tag + ": children cover adjacent ranges"
+
+
+def test_large_trees_checked_on_the_host():
+    """Trees of the chain of launches (boxes of the internal nodes as range unions over blocks of 128 leaves; leaves
+    sorted by one launch or by four radix passes), sizes around the block length and the capacities of the sort, several
+    trees per call, degenerate geometry: every exported tree is checked on the host -- structure, leaf order, leaf boxes,
+    every parent box the exact union of its children's -- and the culled sums against the masked sum."""
+    lib = _native.lib()
+    cases = ((1, 1, 1025, 2, 0, "none"), (2, 1, 1279, 3, 0, "identical"), (1, 2, 2049, 3, 2, "cells"), (1, 1, 4097, 2, 0, "point"),
+             (3, 1, 1281, 3, 1, "line"), (1, 1, 8193, 3, 0, "cells"), (1, 2, 16384, 3, 0, "identical"), (1, 1, 16385, 2, 0, "none"),
+             (5, 1, 3000, 3, 0, "cells"), (1, 1, 129, 3, 1, "none"), (1, 3, 257, 2, 1, "point"))
+    for k, (B, L, M, D, path, kind) in enumerate(cases):
+        dtype = torch.float32 if k % 2 else torch.float64
+        mix, xes, gout = _case(B, L, M, 300, D, seed=8100 + k, cov_radius=0.05 if k % 3 else 0.3)
+        if kind == "identical": mix[:, :, 1:M // 2] = mix[:, :, :1]
+        elif kind == "cells": mix[:, :, ::2, 1:1 + D] *= 1e-3
+        elif kind == "point": mix[..., 1:1 + D] = mix[:, :, :1, 1:1 + D]
+        elif kind == "line": mix[..., 2:1 + D] = 0.0
+        m, x = mix.to(dtype).to(DEV).contiguous(), xes.to(dtype).to(DEV).contiguous()
+        lib.gmc_bvh_set_build_path(path)
+        try:
+            bvh = _native.Bvh(m, x, 0.001, "reference" if k % 4 == 0 else "tight")
+            lo, up = bvh.boxes()
+            nodes, nb = bvh.nodes()
+            keys, comps = bvh.leaf_order()
+            out = _native.eval_bvh_fwd(m, x, bvh)
+            torch.cuda.synchronize()
+        finally:
+            lib.gmc_bvh_set_build_path(0)
+        assert n_errors(bvh) == 0
+        lo, up, nodes, nb, keys, comps, out = (t.cpu().numpy() for t in (lo, up, nodes, nb, keys, comps, out))
+        for b in range(B):
+            for l in range(L):
+                _check_tree_on_the_host(nodes[b, l], nb[b, l], keys[b, l].astype(np.int64), comps[b, l], lo[b, l], up[b, l], M, D,
+                                        f"case {k}: B{B} L{L} M{M} D{D} path {path} {kind}, tree ({b}, {l})")
+        # the culled forward sum against the masked sum on these boxes; thousands of terms of both signs at one place
+        # cancel, so the error is measured against the sum of the terms' magnitudes
+        npdt = np.float32 if dtype == torch.float32 else np.float64
+        m64, x64 = (t.numpy().astype(npdt).astype(np.float64) for t in (mix, xes))
+        lo64, up64 = lo.astype(np.float64), up.astype(np.float64)
+        ref = cpu_ref.forward(m64, x64, lo64, up64, n_threads=16)
+        m64[..., 0] = np.abs(m64[..., 0])
+        scale = cpu_ref.forward(m64, x64, lo64, up64, n_threads=16)
+        err = np.abs(out - ref).max() / max(scale.max(), FLOOR[dtype])
+        assert err <= 3 * TOL[dtype], f"case {k}: culled forward sum off by {err:.3g} of the terms' magnitudes"
+
+
 def test_mixture_beyond_the_reference_node_index_range():
     """The reference stores node indices in 16 bits (lbvh/bvh.h:16-24: at most 32768 components per mixture); here
     they are 32-bit.  One mixture of 70000 components: every component is exactly one leaf, every parent box is the
