@@ -439,23 +439,41 @@ __device__ __forceinline__ uint32_t morton30(const T* __restrict__ p, const T* _
 
 // a set of points to be Morton-coded: the centres of the mixtures or the query points
 template <typename T> struct MortonJob {
-    const T* pts; int stride, offset, count, blocks_per_seg;      // workgroup (blk, seg) codes 256 points
+    const T* pts; int stride, offset, count;
+    int items, blocks_per_seg;                                     // workgroup (blk, seg) codes kBlock * items points
     const T* parts; int n_parts;                                   // partial bounds of every segment
     uint32_t* keys; uint32_t* vals;
     unsigned blocks;                                               // workgroups of this job in the launch
-    uint32_t* hist; int sort_blocks_per_seg, sort_chunk_shift, shift;   // block histograms of the first radix pass (null: none wanted)
+    uint32_t* hist; int shift;       // block histograms of the first radix pass, one per workgroup (null: none wanted)
 };
 
 // Morton keys and index payload for two jobs in one launch (job b behind job a); every workgroup first combines
-// its segment's partial bounds
+// its segment's partial bounds.  A workgroup codes the keys of exactly one block of the first radix pass, so that the
+// block's digit histogram is counted in LDS and stored (global atomics would leave the launch waiting for their round
+// trip to the memory side).
 template <typename T, int D>
 __global__ __launch_bounds__(kBlock) void morton_kernel(MortonJob<T> a, MortonJob<T> b) {
     __shared__ T red[2 * D][kBlock];
     __shared__ T bounds[2 * D];
+    __shared__ uint32_t digits[256];
     const bool first = blockIdx.x < a.blocks;
     const MortonJob<T>& j = first ? a : b;
     const unsigned id = first ? blockIdx.x : blockIdx.x - a.blocks;
     const int seg = id / j.blocks_per_seg, blk = id - seg * j.blocks_per_seg;
+    // eight points per lane at a time, all loads in flight; the first ones are fetched while the bounds are combined
+    constexpr int kBatch = 8;
+    T p[kBatch][D];
+    auto fetch = [&](int r0) {
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            const int i = (blk * j.items + r0 + r) * kBlock + threadIdx.x;
+            if (r0 + r < j.items && i < j.count) {
+                const T* src = j.pts + (size_t(seg) * j.count + i) * j.stride + j.offset;
+                for (int d = 0; d < D; ++d) p[r][d] = src[d];
+            }
+        }
+    };
+    fetch(0);
     T lo[D], hi[D];
     for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
     for (int i = threadIdx.x; i < j.n_parts; i += kBlock) {
@@ -467,14 +485,25 @@ __global__ __launch_bounds__(kBlock) void morton_kernel(MortonJob<T> a, MortonJo
     }
     const T v = block_bounds<T, D>(lo, hi, red);
     if (threadIdx.x < 2 * D) bounds[threadIdx.x] = v;
+    digits[threadIdx.x] = 0u;
     __syncthreads();
-    const int i = blk * kBlock + threadIdx.x;
-    if (i >= j.count) return;
-    const size_t at = size_t(seg) * j.count + i;
-    const uint32_t key = morton30<T, D>(j.pts + at * j.stride + j.offset, bounds);
-    j.keys[at] = key;
-    j.vals[at] = uint32_t(i);
-    if (j.hist) atomicAdd(&j.hist[(size_t(seg) * j.sort_blocks_per_seg + (i >> j.sort_chunk_shift)) * 256 + ((key >> j.shift) & 255u)], 1u);
+    for (int r0 = 0; r0 < j.items; r0 += kBatch) {
+        if (r0 > 0) fetch(r0);
+#pragma unroll
+        for (int r = 0; r < kBatch; ++r) {
+            const int i = (blk * j.items + r0 + r) * kBlock + threadIdx.x;
+            if (r0 + r < j.items && i < j.count) {
+                const size_t at = size_t(seg) * j.count + i;
+                const uint32_t key = morton30<T, D>(p[r], bounds);
+                j.keys[at] = key;
+                j.vals[at] = uint32_t(i);
+                if (j.hist) atomicAdd(&digits[(key >> j.shift) & 255u], 1u);
+            }
+        }
+    }
+    if (!j.hist) return;
+    __syncthreads();
+    j.hist[(size_t(seg) * j.blocks_per_seg + blk) * 256 + threadIdx.x] = digits[threadIdx.x];
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -2493,7 +2522,6 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     }
     const int bpm = (M + kBlock - 1) / kBlock;               // workgroups per mixture (boxes, keys)
     const int nbp = (N + kBoundsChunk - 1) / kBoundsChunk;   // partial bounds per point segment
-    const int bpx = (N + kBlock - 1) / kBlock;               // workgroups per point segment (keys)
     const unsigned box_blocks = have_g ? unsigned(BL * bpm) : 0u, bound_blocks = sort_p ? unsigned(XL * nbp) : 0u;
     if (box_blocks + bound_blocks > 0)
         bvh_bounds_kernel<T, D><<<dim3(box_blocks + bound_blocks), dim3(kBlock), 0, st>>>(
@@ -2511,10 +2539,11 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     MortonJob<T> mg = {}, mp = {};
     // one or two large trees: every value of the top 8 key bits gathered and sorted in LDS (bucket_sort_kernel)
     const bool bucket_sort = have_g && g_build_path != 2 && M > kSmallTreeMax && M <= kBucketSortMax && BL <= size_t(kBucketSortSegments);
-    if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bpm, parts_g, bpm, ka, va, unsigned(BL * bpm),
-                                  bucket_sort ? nullptr : (uint32_t*)jg0.hist, jg0.blocks_per_seg, jg0.chunk_shift, jg0.shift};
-    if (sort_p) mp = MortonJob<T>{xes, D, 0, N, bpx, parts_p, nbp, pka, pva, unsigned(XL * bpx),
-                                  (uint32_t*)jp0.hist, jp0.blocks_per_seg, jp0.chunk_shift, jp0.shift};
+    // (a Morton workgroup per block of the first radix pass; without a radix sort behind it: 256 keys each)
+    if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bucket_sort ? 1 : jg0.items, bucket_sort ? bpm : jg0.blocks_per_seg, parts_g, bpm, ka, va,
+                                  unsigned(BL * (bucket_sort ? bpm : jg0.blocks_per_seg)), bucket_sort ? nullptr : (uint32_t*)jg0.hist, jg0.shift};
+    if (sort_p) mp = MortonJob<T>{xes, D, 0, N, jp0.items, jp0.blocks_per_seg, parts_p, nbp, pka, pva, unsigned(XL * jp0.blocks_per_seg),
+                                  (uint32_t*)jp0.hist, jp0.shift};
     if (mg.blocks + mp.blocks > 0) morton_kernel<T, D><<<dim3(mg.blocks + mp.blocks), dim3(kBlock), 0, st>>>(mg, mp);
     // leaves: all 30 key bits; points: the top 16 Morton bits (65536 cells) are enough to make 64 consecutive
     // points neighbours, the top 8 bits for segments of at most kCoarseOrderMax points (32 points per cell; measured:
