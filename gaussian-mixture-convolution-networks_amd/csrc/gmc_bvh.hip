@@ -41,7 +41,6 @@ constexpr double kSqFloor = 5.991464547107982;   // -2 ln 0.05 (lbvh/bvh.cu:194)
 // layout of the opaque BVH object
 // ---------------------------------------------------------------------------------------------------------------
 struct BvhLayout {
-    size_t box_lo, box_hi;      // T [BL][M][D]            per-Gaussian boxes, component order
     size_t node_box;            // T [BL][2M-1][2D]        lower, upper; internal nodes first, then leaves (Morton order)
     size_t child_box;           // T [BL][M-1][2][2D]      boxes of the left and right child, stored with the parent
     size_t leaf_rec;            // T [BL][M][RS]           evaluation records in leaf order
@@ -149,8 +148,6 @@ static BvhLayout bvh_layout(const gmc_shape& s) {
     BvhLayout l;
     size_t o = 0;
     auto take = [&](size_t bytes) { const size_t at = o; o = align_up(o + bytes); return at; };
-    l.box_lo = take(BL * M * D * e);
-    l.box_hi = take(BL * M * D * e);
     l.node_box = take(BL * nodes * 2 * D * e);
     l.child_box = take(BL * (M > 0 ? M - 1 : 0) * 4 * D * e);
     l.leaf_rec = take(BL * M * rs * e);
@@ -820,11 +817,10 @@ __device__ __forceinline__ int2 build_internal_node(KeyAt key_at, int2* __restri
 }
 
 // Leaf `leaf` (Morton order) of mixture bl, which holds component `comp`: the cutoff box of the Gaussian
-// (lbvh/bvh.cu:164-231; kept in component order too for gmc_bvh_export_boxes, and as the leaf's node box), its
-// evaluation record behind its own box, zeroed sums of the backward pass.  blo / bhi receive the box.
+// (lbvh/bvh.cu:164-231; stored as the leaf's node box), its evaluation record behind its own box, zeroed sums of the
+// backward pass.  blo / bhi receive the box.
 template <typename T, int D>
-__device__ __forceinline__ void write_leaf(const T* __restrict__ mixture, T* __restrict__ box_lo, T* __restrict__ box_hi,
-                                           double threshold, int mode, bool covariance_form, T* __restrict__ node_box,
+__device__ __forceinline__ void write_leaf(const T* __restrict__ mixture, double threshold, int mode, bool covariance_form, T* __restrict__ node_box,
                                            T* __restrict__ leaf_rec, int* __restrict__ parent, T* __restrict__ sums, int M,
                                            size_t bl, int leaf, int comp, T (&blo)[D], T (&bhi)[D]) {
     constexpr int G = 1 + D + D * D;
@@ -843,8 +839,6 @@ __device__ __forceinline__ void write_leaf(const T* __restrict__ mixture, T* __r
         for (int d = 0; d < D; ++d) {
             blo[d] = T(double(g[1 + d]) - delta[d]);
             bhi[d] = T(double(g[1 + d]) + delta[d]);
-            box_lo[gi * D + d] = blo[d];
-            box_hi[gi * D + d] = bhi[d];
         }
     }
     for (int d = 0; d < D; ++d) {
@@ -890,8 +884,7 @@ __device__ __forceinline__ void write_leaf(const T* __restrict__ mixture, T* __r
 // last block to the last leaf.  No step waits for another node: the bottom-up walk this replaces was a chain of one
 // atomic round trip per tree level.
 template <typename T, int D>
-__global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, T* __restrict__ box_lo,
-                                                           T* __restrict__ box_hi, double threshold, int mode,
+__global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict__ mixture, double threshold, int mode,
                                                            const uint32_t* __restrict__ order,
                                                            const uint32_t* __restrict__ keys, T* __restrict__ node_box,
                                                            T* __restrict__ leaf_rec,
@@ -932,7 +925,7 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         for (int d = 0; d < D; ++d) { lo[d] = OrderedInt<T>::kEmptyLo; hi[d] = OrderedInt<T>::kEmptyHi; }
         if (t < total) {
             T blo[D], bhi[D];
-            write_leaf<T, D>(mixture, box_lo, box_hi, threshold, mode, covariance_form, node_box, leaf_rec, parent, sums, M, bl,
+            write_leaf<T, D>(mixture, threshold, mode, covariance_form, node_box, leaf_rec, parent, sums, M, bl,
                              leaf, comp, blo, bhi);
             for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(blo[d]); hi[d] = ordered_bits(bhi[d]); }
         }
@@ -1170,7 +1163,7 @@ static int g_build_path = 0;            // test knob (gmc_bvh_set_build_path): 1
                                         // leaves' sort always as four radix passes
 
 template <typename T> struct SmallBuild {
-    T* box_lo; T* box_hi; T* node_box; T* child_box; T* leaf_rec; T* sums;
+    T* node_box; T* child_box; T* leaf_rec; T* sums;
     int2* children; int* parent; int2* node_range; int* leaf_comp; uint32_t* g_keys; int* frontier;
     int* p_order; int* cand_count; int* ctl;
     double threshold;
@@ -1369,7 +1362,7 @@ __device__ __forceinline__ void build_small_tree(const T* __restrict__ mixture, 
             const int comp = int(unsigned(key));
             a.g_keys[bl * M + i] = uint32_t(key >> 32);
             a.leaf_comp[bl * M + i] = comp;
-            write_leaf<T, D>(mixture, a.box_lo, a.box_hi, a.threshold, a.mode, a.covariance_form != 0, a.node_box, a.leaf_rec,
+            write_leaf<T, D>(mixture, a.threshold, a.mode, a.covariance_form != 0, a.node_box, a.leaf_rec,
                              a.parent, a.sums, M, bl, i, comp, blo[k], bhi[k]);
         }
     }
@@ -2428,6 +2421,23 @@ __global__ __launch_bounds__(kBlock) void export_nodes_kernel(const int2* __rest
     }
 }
 
+// the boxes of the Gaussians in component order, from the boxes of the leaves (Morton order)
+template <typename T, int D>
+__global__ __launch_bounds__(kBlock) void export_boxes_kernel(const T* __restrict__ node_box, const int* __restrict__ leaf_comp,
+                                                             T* __restrict__ lower, T* __restrict__ upper, int M, size_t total) {
+    const size_t t = size_t(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= total) return;
+    const size_t bl = t / M;
+    const int leaf = int(t - bl * M);
+    int comp = leaf_comp[t];
+    comp = (comp >= 0 && comp < M) ? comp : 0;
+    const T* box = node_box + (bl * (2 * size_t(M) - 1) + (M - 1) + leaf) * 2 * D;
+    for (int d = 0; d < D; ++d) {
+        if (lower) lower[(bl * M + comp) * D + d] = box[d];
+        if (upper) upper[(bl * M + comp) * D + d] = box[D + d];
+    }
+}
+
 template <typename T>
 __global__ void copy_kernel(const T* __restrict__ src, T* __restrict__ dst, size_t n) {
     const size_t stride = size_t(gridDim.x) * blockDim.x;
@@ -2478,7 +2488,6 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     const BvhLayout lay = bvh_layout(s);
     const size_t BL = size_t(s.B) * s.L, XL = size_t(s.Bx) * s.Lx;
     const int M = s.M, N = s.N;
-    T* box_lo = (T*)(bvh + lay.box_lo); T* box_hi = (T*)(bvh + lay.box_hi);
     T* node_box = (T*)(bvh + lay.node_box); T* leaf_rec = (T*)(bvh + lay.leaf_rec);
     int2* children = (int2*)(bvh + lay.children); int* parent = (int*)(bvh + lay.parent);
     int2* node_range = (int2*)(bvh + lay.node_range);
@@ -2498,7 +2507,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     const bool sort_p = have_p && xes != nullptr;
     if (g_build_path == 0 && have_g && M <= kSmallTreeMax && (!sort_p || N <= kCoarseOrderMax) && BL + XL < (size_t(1) << 31)) {
         const CandidateCache cache = candidate_cache(bvh, lay);
-        SmallBuild<T> a{box_lo, box_hi, node_box, child_box, leaf_rec, (T*)(bvh + lay.sums), children, parent, node_range,
+        SmallBuild<T> a{node_box, child_box, leaf_rec, (T*)(bvh + lay.sums), children, parent, node_range,
                         leaf_comp, g_keys, (int*)(bvh + lay.frontier), p_order, cache.count, (int*)(bvh + lay.cand_ctl),
                         double(cfg.aabb_threshold), cfg.aabb_mode, cfg.covariance_form != 0 ? 1 : 0, M, N,
                         (N + kWave - 1) / kWave, sort_p ? 1 : 0, 0u};
@@ -2578,7 +2587,7 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
         const size_t n = BL * M;
         const unsigned leaf_blocks = unsigned((n + kBoxBlock - 1) / kBoxBlock);
         bvh_leaves_kernel<T, D><<<dim3(leaf_blocks + jp_first.blocks), dim3(kBlock), 0, st>>>(
-            mixture, box_lo, box_hi, double(cfg.aabb_threshold), cfg.aabb_mode, g_order, g_keys, node_box, leaf_rec, run_box,
+            mixture, double(cfg.aabb_threshold), cfg.aabb_mode, g_order, g_keys, node_box, leaf_rec, run_box,
             children, parent, node_range, M, n, cfg.covariance_form != 0, (T*)(bvh + lay.sums), leaf_blocks, jp_first);
         if (M > 1) {
             const size_t nn = BL * (2 * size_t(M) - 1);
@@ -2718,8 +2727,9 @@ static int bvh_export_t(const char* bvh, T* lower, T* upper, int32_t* nodes, T* 
     auto copy = [&](const T* src, T* dst, size_t cnt) {
         if (cnt) copy_kernel<T><<<dim3(grid_for(cnt) < 4096 ? grid_for(cnt) : 4096), dim3(kBlock), 0, st>>>(src, dst, cnt);
     };
-    if (lower) copy((const T*)(bvh + lay.box_lo), lower, n);
-    if (upper) copy((const T*)(bvh + lay.box_hi), upper, n);
+    if ((lower || upper) && n)
+        export_boxes_kernel<T, D><<<dim3(grid_for(BL * s.M)), dim3(kBlock), 0, st>>>(
+            (const T*)(bvh + lay.node_box), (const int*)(bvh + lay.leaf_comp), lower, upper, s.M, BL * s.M);
     if (s.M > 0) {
         const size_t nn = BL * (2 * size_t(s.M) - 1);
         if (nodes && nn)
