@@ -816,23 +816,19 @@ __device__ __forceinline__ int2 build_internal_node(KeyAt key_at, int2* __restri
     return make_int2(first, last);
 }
 
-// Leaf `leaf` (Morton order) of mixture bl, which holds component `comp`: the cutoff box of the Gaussian
+// Leaf `leaf` (Morton order) of mixture bl, which holds component `comp` with the record g: the cutoff box of the Gaussian
 // (lbvh/bvh.cu:164-231; stored as the leaf's node box), its evaluation record behind its own box, zeroed sums of the
 // backward pass.  blo / bhi receive the box.
 template <typename T, int D>
-__device__ __forceinline__ void write_leaf(const T* __restrict__ mixture, double threshold, int mode, bool covariance_form, T* __restrict__ node_box,
+__device__ __forceinline__ void write_leaf(const T* __restrict__ g, double threshold, int mode, bool covariance_form, T* __restrict__ node_box,
                                            T* __restrict__ leaf_rec, int* __restrict__ parent, T* __restrict__ sums, int M,
                                            size_t bl, int leaf, int comp, T (&blo)[D], T (&bhi)[D]) {
-    constexpr int G = 1 + D + D * D;
     constexpr int RS = LeafRec<D>::kStride;
     constexpr int NS = 1 + D + D * (D + 1) / 2;
     const size_t i = bl * M + leaf;
     // the per-Gaussian sums of the backward pass start from zero (and return to zero after every backward pass)
     for (int k = 0; k < NS; ++k) sums[i * NS + k] = T(0);
-    comp = (comp >= 0 && comp < M) ? comp : 0;      // a permutation by construction; never index out of bounds
-    const size_t gi = bl * M + comp;
     const size_t node = bl * (2 * size_t(M) - 1) + (M - 1) + leaf;
-    const T* g = mixture + gi * G;
     {
         double delta[D];
         box_half_extent<T, D>(g, threshold, mode, covariance_form, delta);
@@ -925,8 +921,9 @@ __global__ __launch_bounds__(kBlock) void bvh_leaves_kernel(const T* __restrict_
         for (int d = 0; d < D; ++d) { lo[d] = OrderedInt<T>::kEmptyLo; hi[d] = OrderedInt<T>::kEmptyHi; }
         if (t < total) {
             T blo[D], bhi[D];
-            write_leaf<T, D>(mixture, threshold, mode, covariance_form, node_box, leaf_rec, parent, sums, M, bl,
-                             leaf, comp, blo, bhi);
+            const int c = (comp >= 0 && comp < M) ? comp : 0;      // a permutation by construction; never index out of bounds
+            write_leaf<T, D>(mixture + (bl * M + c) * (1 + D + D * D), threshold, mode, covariance_form, node_box, leaf_rec, parent,
+                             sums, M, bl, leaf, c, blo, bhi);
             for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(blo[d]); hi[d] = ordered_bits(bhi[d]); }
         }
         for (int d = 0; d < D; ++d) { table[0][d][idx] = lo[d]; table[0][D + d][idx] = hi[d]; }
@@ -1304,14 +1301,22 @@ __device__ __forceinline__ void build_small_tree(const T* __restrict__ mixture, 
         for (int g = tid; g < a.per_mixture; g += THREADS) a.cand_count[bl * a.per_mixture + g] = -1;
     // bounds of the centres and keys
     T c[K][D], bounds[2 * D];
+    // one leaf per lane: the lane keeps ITS component (the whole record is fetched with the centre, one round trip) and
+    // learns the leaf it becomes from the sort
+    T rec[K == 1 ? G : 1];
     {
         T lo[D], hi[D];
         for (int d = 0; d < D; ++d) { lo[d] = T(INFINITY); hi[d] = T(-INFINITY); }
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             const int i = tid + k * THREADS;
+            if constexpr (K == 1) {
+#pragma unroll
+                for (int q = 0; q < G; ++q) rec[q] = i < M ? mixture[(bl * M + i) * G + q] : T(0);
+            }
             for (int d = 0; d < D; ++d) {
-                c[k][d] = i < M ? mixture[(bl * M + i) * G + 1 + d] : T(0);
+                if constexpr (K == 1) c[k][d] = rec[1 + d];
+                else c[k][d] = i < M ? mixture[(bl * M + i) * G + 1 + d] : T(0);
                 if (i < M) {
                     lo[d] = c[k][d] < lo[d] ? c[k][d] : lo[d];       // a NaN coordinate is skipped
                     hi[d] = c[k][d] > hi[d] ? c[k][d] : hi[d];
@@ -1334,38 +1339,63 @@ __device__ __forceinline__ void build_small_tree(const T* __restrict__ mixture, 
                 }
         }
     }
-    int Mp = 1;
-    while (Mp < M) Mp <<= 1;
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int i = tid + k * THREADS;
-        if (i < Mp) s.keys[i] = i < M ? ((unsigned long long)morton30<T, D>(c[k], bounds) << 32) | (unsigned)i : ~0ull;
-    }
-    tree_sync<THREADS>();
-    // bitonic sort of the unique keys
-    for (int size = 2; size <= Mp; size <<= 1)
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            for (int q = tid; q < Mp / 2; q += THREADS) {
-                const int i0 = ((q & ~(stride - 1)) << 1) | (q & (stride - 1)), i1 = i0 | stride;
-                const unsigned long long k0 = s.keys[i0], k1 = s.keys[i1];
-                if ((k0 > k1) == ((i0 & size) == 0)) { s.keys[i0] = k1; s.keys[i1] = k0; }
-            }
-            tree_sync<THREADS>();
-        }
-    // leaves: lane <-> leaf i (Morton order) and, below, internal node i
+    int leaf_of[K];                                         // the leaf (Morton order) whose box and record lane slot k writes
     T blo[K][D], bhi[K][D];
+    if constexpr (K == 1) {
+        // Sort by counting: the leaf of component i is the number of unique keys below its own (every read a broadcast,
+        // no step waits for another); the keys then move to their places for the tree build.
+        const unsigned long long mine = tid < M ? ((unsigned long long)morton30<T, D>(c[0], bounds) << 32) | (unsigned)tid : ~0ull;
+        if (tid < M) s.keys[tid] = mine;
+        tree_sync<THREADS>();
+        int rank = 0;
+#pragma unroll 8
+        for (int j = 0; j < M; ++j) rank += s.keys[j] < mine ? 1 : 0;
+        tree_sync<THREADS>();                               // every lane has counted before the keys move
+        if (tid < M) s.keys[rank] = mine;
+        leaf_of[0] = rank;
+        if (tid < M) {
+            a.g_keys[bl * M + rank] = uint32_t(mine >> 32);
+            a.leaf_comp[bl * M + rank] = tid;
+            write_leaf<T, D>(rec, a.threshold, a.mode, a.covariance_form != 0, a.node_box, a.leaf_rec, a.parent, a.sums, M, bl,
+                             rank, tid, blo[0], bhi[0]);
+        }
+        tree_sync<THREADS>();                               // the sorted keys are in place
+    } else {
+        int Mp = 1;
+        while (Mp < M) Mp <<= 1;
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int i = tid + k * THREADS;
-        if (i < M) {
-            const unsigned long long key = s.keys[i];
-            const int comp = int(unsigned(key));
-            a.g_keys[bl * M + i] = uint32_t(key >> 32);
-            a.leaf_comp[bl * M + i] = comp;
-            write_leaf<T, D>(mixture, a.threshold, a.mode, a.covariance_form != 0, a.node_box, a.leaf_rec,
-                             a.parent, a.sums, M, bl, i, comp, blo[k], bhi[k]);
+        for (int k = 0; k < K; ++k) {
+            const int i = tid + k * THREADS;
+            if (i < Mp) s.keys[i] = i < M ? ((unsigned long long)morton30<T, D>(c[k], bounds) << 32) | (unsigned)i : ~0ull;
+        }
+        tree_sync<THREADS>();
+        // bitonic sort of the unique keys
+        for (int size = 2; size <= Mp; size <<= 1)
+            for (int stride = size >> 1; stride > 0; stride >>= 1) {
+                for (int q = tid; q < Mp / 2; q += THREADS) {
+                    const int i0 = ((q & ~(stride - 1)) << 1) | (q & (stride - 1)), i1 = i0 | stride;
+                    const unsigned long long k0 = s.keys[i0], k1 = s.keys[i1];
+                    if ((k0 > k1) == ((i0 & size) == 0)) { s.keys[i0] = k1; s.keys[i1] = k0; }
+                }
+                tree_sync<THREADS>();
+            }
+        // leaves: lane <-> leaf i (Morton order)
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const int i = tid + k * THREADS;
+            leaf_of[k] = i;
+            if (i < M) {
+                const unsigned long long key = s.keys[i];
+                int comp = int(unsigned(key));
+                comp = (comp >= 0 && comp < M) ? comp : 0;  // a permutation by construction; never index out of bounds
+                a.g_keys[bl * M + i] = uint32_t(key >> 32);
+                a.leaf_comp[bl * M + i] = comp;
+                write_leaf<T, D>(mixture + (bl * M + comp) * G, a.threshold, a.mode, a.covariance_form != 0, a.node_box, a.leaf_rec,
+                                 a.parent, a.sums, M, bl, i, comp, blo[k], bhi[k]);
+            }
         }
     }
+    // below: lane <-> internal node i
     if (M < 2) return;
     int* par = a.parent + bl * (2 * size_t(M) - 1);
 #pragma unroll
@@ -1396,7 +1426,7 @@ __device__ __forceinline__ void build_small_tree(const T* __restrict__ mixture, 
         if (i < M) {
             Enc lo[D], hi[D];
             for (int d = 0; d < D; ++d) { lo[d] = ordered_bits(blo[k][d]); hi[d] = ordered_bits(bhi[k][d]); }
-            int node = s.parent[(M - 1) + i];
+            int node = s.parent[(M - 1) + leaf_of[k]];
             for (int level = 0; node >= 0 && node < M - 1 && level < 128; ++level) {
                 bool grew = false;
                 for (int d = 0; d < D; ++d) {
@@ -1426,9 +1456,9 @@ __device__ __forceinline__ void build_small_tree(const T* __restrict__ mixture, 
             }
         }
         if (i < M) {
-            const int up = s.parent[(M - 1) + i];
+            const int up = s.parent[(M - 1) + leaf_of[k]];
             if (up >= 0 && up < M - 1) {
-                const int side = s.kids[up].x == ~i ? 0 : 1;
+                const int side = s.kids[up].x == ~leaf_of[k] ? 0 : 1;
                 for (int d = 0; d < D; ++d) {
                     cb[(size_t(up) * 2 + side) * 2 * D + d] = blo[k][d];
                     cb[(size_t(up) * 2 + side) * 2 * D + D + d] = bhi[k][d];
