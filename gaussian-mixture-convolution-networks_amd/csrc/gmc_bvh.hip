@@ -631,7 +631,8 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// The leaves' sort for one or two large trees (kSmallTreeMax < M <= kBucketSortMax) in ONE launch instead of four radix
+// The leaves' sort for one large tree (kSmallTreeMax < M <= kBucketSortMax; two trees of up to half that size, whose
+// workgroups fit a compute unit in pairs: more would queue up) in ONE launch instead of four radix
 // passes at their latency floor: 256 workgroups per tree, one per value of the top 8 key bits.  Workgroup d reads all
 // keys of the tree (in component order, as the Morton kernel wrote them; 64 KB at most, from L2), keeps those whose top
 // bits are d as unique keys (Morton code << 32 | component) in LDS, counts those with smaller top bits -- the first
@@ -642,7 +643,7 @@ __device__ __forceinline__ void wave_lds_fence() {
 constexpr int kBucketSortLanes = 1024;
 constexpr int kBucketSortMax = 16384;
 constexpr int kBucketRankMax = 256;        // keys of one digit up to which counting ranks beats the sorting network
-constexpr int kBucketSortSegments = 2;     // more trees than this: the grid of 256 workgroups per tree would queue up
+constexpr int kBucketCrowded = 1024;       // expected keys of one value of the top bits from which splitters are taken instead
 
 template <int CAP>
 __global__ __launch_bounds__(kBucketSortLanes) void bucket_sort_kernel(const uint32_t* __restrict__ keys_in, uint32_t* __restrict__ keys_out,
@@ -675,20 +676,74 @@ __global__ __launch_bounds__(kBucketSortLanes) void bucket_sort_kernel(const uin
             for (int c = 0; c < kVec; ++c) key[kVec * r + c] = i + c < count ? in[i + c] : 0xffffffffu;   // (real keys have 30 bits)
         }
     }
+    // the component of key r of this lane
+    auto component = [&](int r) { return ((r / kVec) * kBucketSortLanes + int(threadIdx.x)) * kVec + r % kVec; };
+    // Which workgroup takes a key: the one numbered by its top 8 bits -- unless the centres crowd into a few Morton
+    // cells (a stray Gaussian far from the others is enough to stretch the bounds), when one workgroup would sort most
+    // of the tree alone.  Every workgroup tests the same sample for that (every lane one of its keys: 1024 of the tree's),
+    // and all take splitters instead when a value of the top bits is expected to hold more than kBucketCrowded keys:
+    // 256 sampled unique keys, sorted by counting; workgroup d takes the keys from splitter d up to splitter d + 1, found
+    // by bisection.  Same result either way; the choice is a function of the keys alone.
+    __shared__ uint32_t sample_bins[256];
+    __shared__ unsigned long long sample[256], splitter[256];
+    if (threadIdx.x < 256) sample_bins[threadIdx.x] = 0u;
     __syncthreads();
+    {
+        // (which of its keys a lane samples, and which lane of four gives a splitter candidate, change with the higher bits
+        // of the lane number: components that follow a pattern of period 2, 4, 8 ... are all represented)
+        uint32_t mine = key[0];
+        int r_mine = 0;
+#pragma unroll
+        for (int r = 1; r < kPerLane; ++r)
+            if (int(threadIdx.x >> 3) % kPerLane == r) { mine = key[r]; r_mine = r; }
+        const int i = component(r_mine);
+        if (i < count) atomicAdd(&sample_bins[(mine >> 22) & 255u], 1u);
+        if ((threadIdx.x & 3) == ((threadIdx.x >> 5) & 3))
+            sample[threadIdx.x >> 2] = i < count ? ((unsigned long long)mine << 32) | uint32_t(i) : ~0ull;
+    }
+    __syncthreads();                                         // the sample is counted
+    const bool crowded = __syncthreads_or(threadIdx.x < 256 && sample_bins[threadIdx.x & 255] * kPerLane > uint32_t(kBucketCrowded));
+    if (crowded) {
+        if (threadIdx.x < 256) {
+            const unsigned long long mine = sample[threadIdx.x];
+            int rank = 0;
+#pragma unroll 8
+            for (int j = 0; j < 256; ++j) rank += (sample[j] < mine || (sample[j] == mine && j < int(threadIdx.x))) ? 1 : 0;
+            splitter[rank] = mine;                           // (absent samples, all ones, share the end)
+        }
+        __syncthreads();
+    }
+    // number of the workgroup that takes unique key x: the last splitter not above it (workgroup 0 also takes what lies below splitter 0)
+    auto taker = [&](unsigned long long x) {
+        int lo = 0;                                          // splitter[lo] <= x or lo == 0
+#pragma unroll
+        for (int step = 128; step > 0; step >>= 1)
+            lo = splitter[lo + step] <= x ? lo + step : lo;
+        return uint32_t(lo);
+    };
+    uint32_t top[kPerLane];
+#pragma unroll
+    for (int r = 0; r < kPerLane; ++r) top[r] = key[r] >> 22;
+    if (crowded) {                                           // (the searches of a lane's keys side by side)
+#pragma unroll
+        for (int r = 0; r < kPerLane; ++r) {
+            const int i = component(r);
+            top[r] = i < count ? taker(((unsigned long long)key[r] << 32) | uint32_t(i)) : 1024u;
+        }
+    }
     int before = 0;
 #pragma unroll
     for (int r = 0; r < kPerLane; ++r) {
-        const int i = ((r / kVec) * kBucketSortLanes + threadIdx.x) * kVec + r % kVec;      // the component of this key
-        const uint32_t top = key[r] >> 22;
-        before += top < digit ? 1 : 0;
-        const bool mine = top == digit;
+        const int i = component(r);
+        const unsigned long long unique = ((unsigned long long)key[r] << 32) | uint32_t(i);
+        before += top[r] < digit ? 1 : 0;
+        const bool mine = top[r] == digit;
         const unsigned long long m = __ballot(mine);
         if (m != 0ull) {                                     // (the order inside the digit does not matter: the keys are unique)
             int base = 0;
             if (lane == __ffsll((long long)m) - 1) base = atomicAdd(&n_mine, __popcll(m));
             base = __shfl(base, __ffsll((long long)m) - 1, kWave);
-            if (mine) k[base + __popcll(m & ((1ull << lane) - 1ull))] = ((unsigned long long)key[r] << 32) | uint32_t(i);
+            if (mine) k[base + __popcll(m & ((1ull << lane) - 1ull))] = unique;
         }
     }
 #pragma unroll
@@ -717,7 +772,9 @@ __global__ __launch_bounds__(kBucketSortLanes) void bucket_sort_kernel(const uin
     }
     int np = 2;
     while (np < n) np <<= 1;
-    constexpr int lanes = kBucketSortLanes;
+    // (wavefronts without a pair of keys leave before the barriers)
+    const int lanes = np / 2 < kBucketSortLanes ? np / 2 : kBucketSortLanes;
+    if (int(threadIdx.x) >= lanes) return;
     for (int i = n + threadIdx.x; i < np; i += lanes) k[i] = ~0ull;
     __syncthreads();
     for (int size = 2; size <= np; size <<= 1)
@@ -2577,7 +2634,8 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
     jobs_of_pass(0, jg0, jp0);
     MortonJob<T> mg = {}, mp = {};
     // one or two large trees: every value of the top 8 key bits gathered and sorted in LDS (bucket_sort_kernel)
-    const bool bucket_sort = have_g && g_build_path != 2 && M > kSmallTreeMax && M <= kBucketSortMax && BL <= size_t(kBucketSortSegments);
+    const bool bucket_sort = have_g && g_build_path != 2 && M > kSmallTreeMax && M <= kBucketSortMax &&
+                             (BL == 1 || (BL == 2 && M <= kBucketSortMax / 2));
     // (a Morton workgroup per block of the first radix pass; without a radix sort behind it: 256 keys each)
     if (have_g) mg = MortonJob<T>{mixture, G, 1, M, bucket_sort ? 1 : jg0.items, bucket_sort ? bpm : jg0.blocks_per_seg, parts_g, bpm, ka, va,
                                   unsigned(BL * (bucket_sort ? bpm : jg0.blocks_per_seg)), bucket_sort ? nullptr : (uint32_t*)jg0.hist, jg0.shift};

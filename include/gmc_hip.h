@@ -199,9 +199,9 @@ typedef struct gmc_bvh_config {
 
 /* Test knob (no counterpart in the reference; process-wide): trees of at most 1024 components whose query points come
  * in segments of at most 8192 are built by one launch (every tree inside one workgroup's LDS), all others by a chain
- * of launches (Morton keys, sort, leaf and tree kernel, box kernel), in which the leaves of one or two trees of at
- * most 16384 components are sorted by one launch (a workgroup per value of the top 8 key bits gathers and sorts its
- * keys in LDS), all others by four radix passes.  path == 1 forces the chain for every shape, path == 2 the chain with four radix passes, path == 0 returns
+ * of launches (Morton keys, sort, leaf and tree kernel, box kernel), in which the leaves of one tree of at most 16384
+ * components (or two of at most 8192) are sorted by one launch (256 workgroups per tree, each gathers and sorts its
+ * share of the keys in LDS), all others by four radix passes.  path == 1 forces the chain for every shape, path == 2 the chain with four radix passes, path == 0 returns
  * to the automatic choice.  All give the same trees, boxes and leaf order bit for bit; the Morton order of the query
  * points may differ for points on the border of a Morton cell. */
 void gmc_bvh_set_build_path(int path);

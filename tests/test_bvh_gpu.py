@@ -641,9 +641,10 @@ def _same_object_by_both_paths(m, x, g, dtype, paths, tag):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 def test_sort_by_digits_in_lds_gives_the_order_of_the_four_radix_passes(dtype):
-    """The leaves of one or two trees of 1025 ... 16384 components are sorted by one launch (a workgroup per value of the
-    top 8 key bits gathers and sorts its keys in LDS), all others by four radix passes; with the latter forced for the
-    same inputs the objects must be identical.  Sizes at both ends of every LDS capacity, duplicate keys, and centres crowded into a
+    """The leaves of one tree of 1025 ... 16384 components (two of at most 8192) are sorted by one launch (256 workgroups
+    per tree, each gathers and sorts its share of the keys in LDS: by the top 8 key bits, or between sampled splitters
+    when the centres crowd into a few cells), all others by four radix passes; with the latter forced for the same
+    inputs the objects must be identical.  Sizes at both ends of every LDS capacity, duplicate keys, and centres crowded into a
     few cells (one digit holds most keys) included."""
     for k, (B, L, M, N, D) in enumerate(((2, 1, 1025, 300, 2), (1, 2, 2048, 100, 3), (1, 2, 2049, 100, 2), (2, 1, 4096, 200, 3),
                                          (1, 1, 4100, 100, 3), (1, 1, 8192, 9000, 2), (1, 2, 12000, 100, 3), (1, 1, 16384, 500, 3))):
