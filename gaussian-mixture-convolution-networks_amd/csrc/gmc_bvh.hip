@@ -8,10 +8,11 @@
 //
 // Build, one tree per (b,l) mixture, all on device and without host synchronisation:
 //   centre bounds -> 30-bit Morton codes of the centres (lbvh/morton_code.h:77-85,145-168) -> stable sort of the codes
-//   (segmented LSD radix sort, 8 bits per pass; one or two large trees: one launch that sorts every value of the top 8
-//   key bits in LDS) -> leaves in Morton order with their boxes and evaluation records, Karras radix tree over the
-//   unique keys (morton << 32 | rank) as lbvh/building.h:11-103 -> boxes of the internal nodes as unions of the leaf
-//   boxes of their ranges (order-preserving integers: exactly the unions a bottom-up merge gives, lbvh/bvh.cu:460-510).
+//   (segmented LSD radix sort, 8 bits per pass; a single large tree: one launch whose 256 workgroups each gather and
+//   sort their share of the keys in LDS) -> leaves in Morton order with their boxes and evaluation records, Karras
+//   radix tree over the unique keys (morton << 32 | rank) as lbvh/building.h:11-103 -> boxes of the internal nodes as
+//   unions of the leaf boxes of their ranges (order-preserving integers: exactly the unions a bottom-up merge gives,
+//   lbvh/bvh.cu:460-510).
 // Query points are Morton-sorted the same way (on their top 16 or 8 key bits) so that a wavefront owns 64
 // neighbouring points; their two sort passes ride as extra workgroups in the two last launches of the tree
 // construction, and one wavefront per tree leaves a cut through the tree a few levels below the root (tree_frontier).
