@@ -2697,12 +2697,17 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
 // the resident workgroups in one go (measured on one mixture of 16384 Gaussians, groups -> best choice and time:
 // 391 -> 1, 43 us; 782 -> 2, 39 us; 1563 -> 4, 46 us against 63 us with 2; 3125 ... 25000 -> 4).  A backward pass
 // reads the candidate lists: small workgroups balance better over the compute units until the launch has many times
-// more groups than resident workgroups (1563 -> 1, 77 us against 85 us with 4; 3125 -> 2; 6250 -> 3; 25000 -> 4).
-static int traversal_groups(size_t BL, int N, bool backward) {
+// more groups than resident workgroups (1563 -> 1, 77 us against 85 us with 4; 3125 -> 2; 6250 -> 3; 25000 -> 4).  The
+// lists of many small trees are short and the fixed work of a workgroup weighs more: their backward launches take the
+// forward rule (64 trees of 512 leaves, 4096 groups: 72 us with 4 against 79 with 3 and 98 with 1; 256 trees of 200
+// leaves, 3328 groups: 44 us with 4, 46 with 2, 52 with 1).
+static int g_traversal_groups[2] = {0, 0};      // test knob (gmc_bvh_set_traversal_groups): forward, backward; 0 = automatic
+static int traversal_groups(size_t BL, int M, int N, bool backward) {
     const size_t per_mixture = (size_t(N) + kWave - 1) / kWave;
     const size_t total = BL * per_mixture, slots = size_t(kTravSlots);
     size_t g;
-    if (backward) g = total < 4 * slots ? 1 : total < 8 * slots ? 2 : total < 16 * slots ? 3 : kGroupsMax;
+    if (g_traversal_groups[backward ? 1 : 0] > 0) g = size_t(g_traversal_groups[backward ? 1 : 0]);
+    else if (backward && M > kSmallTreeMax) g = total < 4 * slots ? 1 : total < 8 * slots ? 2 : total < 16 * slots ? 3 : kGroupsMax;
     else g = total <= slots ? 1 : total <= 2 * slots ? 2 : kGroupsMax;
     if (g > per_mixture) g = per_mixture;
     return g < 1 ? 1 : int(g);
@@ -2728,7 +2733,7 @@ static int bvh_fwd_t(const T* xes, char* bvh, T* out, const gmc_shape& s, hipStr
 #undef GMC_ALL
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    const int groups = traversal_groups(BL, s.N, false);
+    const int groups = traversal_groups(BL, s.M, s.N, false);
     int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
     // A launch that would leave resident slots empty is spread over all of them: workgroups whose last wavefront
     // finds no group left serve one group fewer (1563 groups: 512 workgroups of 3 or 4 instead of 391 of 4, 50.6 -> 46.5 us).
@@ -2781,8 +2786,12 @@ static int bvh_bwd_t(const T* grad_out, const T* mixture, const T* xes, char* bv
         }
         return hipGetLastError() == hipSuccess ? GMC_OK : GMC_E_LAUNCH;
     }
-    const int groups = traversal_groups(BL, s.N, true);
-    const int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
+    const int groups = traversal_groups(BL, s.M, s.N, true);
+    int chunks = (s.N + kWave * groups - 1) / (kWave * groups);
+    if (groups > 1 && BL * size_t(chunks) < size_t(kTravSlots)) {       // (as in the forward pass: no resident slot left empty)
+        const size_t per_mixture = (size_t(s.N) + kWave - 1) / kWave, fill = size_t(kTravSlots) / BL;
+        chunks = int(fill < per_mixture ? fill : per_mixture);
+    }
     // one helper workgroup per piece that a forward pass may have published, behind the owners
     const int helpers = lay.pieces_max;
     const dim3 grid(unsigned(BL * chunks + helpers));
@@ -2834,6 +2843,10 @@ static int bvh_export_t(const char* bvh, T* lower, T* upper, int32_t* nodes, T* 
 
 extern "C" {
 
+void gmc_bvh_set_traversal_groups(int forward, int backward) {
+    gmc::g_traversal_groups[0] = forward >= 1 && forward <= gmc::kGroupsMax ? forward : 0;
+    gmc::g_traversal_groups[1] = backward >= 1 && backward <= gmc::kGroupsMax ? backward : 0;
+}
 void gmc_bvh_set_build_path(int path) { gmc::g_build_path = path == 1 || path == 2 ? path : 0; }
 void gmc_bvh_set_eval_path(int path) { gmc::g_eval_path = path == 1 ? 1 : 0; }
 

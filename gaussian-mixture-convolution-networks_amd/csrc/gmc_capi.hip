@@ -37,7 +37,7 @@ int check_shape(const gmc_shape* s) {
 
 extern "C" {
 
-int gmc_abi_version(void) { return 10; }
+int gmc_abi_version(void) { return 11; }
 
 const char* gmc_error_string(int code) {
     switch (code) {

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(CSRC_DIR, "libgmc_hip.so")
 
 GMC_F32, GMC_F64 = 0, 1
 GMC_AABB_REFERENCE, GMC_AABB_TIGHT = 0, 1
-ABI_VERSION = 10
+ABI_VERSION = 11
 STATIC_SCRATCH_BYTES = 64 << 20
 
 
@@ -87,6 +87,8 @@ def lib() -> ctypes.CDLL:
         l.gmc_bvh_set_build_path.argtypes = [ci]
         l.gmc_bvh_set_eval_path.restype = None
         l.gmc_bvh_set_eval_path.argtypes = [ci]
+        l.gmc_bvh_set_traversal_groups.restype = None
+        l.gmc_bvh_set_traversal_groups.argtypes = [ci, ci]
         l.gmc_bvh_bytes.restype = sz
         l.gmc_bvh_bytes.argtypes = [shp]
         l.gmc_bvh_build.argtypes = [vp, vp, vp, sz, shp, cfg, vp]

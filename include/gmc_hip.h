@@ -209,6 +209,10 @@ void gmc_bvh_set_build_path(int path);
  * all points with the box test in front of every evaluation: same rule, same sums); path == 1 forces the traversal for
  * every shape, path == 0 returns to the automatic choice. */
 void gmc_bvh_set_eval_path(int path);
+/* Test knob like the ones above: the number of 64-point groups that a workgroup of the traversal serves (1 ... 4) in
+ * forward and in backward launches; 0 returns to the automatic choice by the size of the launch.  Same sums for every
+ * value; for parameter sweeps. */
+void gmc_bvh_set_traversal_groups(int forward, int backward);
 
 /* Bytes of the opaque BVH object for `shape` (nodes, boxes, sorted orders, build scratch). */
 size_t gmc_bvh_bytes(const gmc_shape* shape);

@@ -66,6 +66,8 @@ def test_scratch_sizes_and_knobs_without_a_device():
     for knob in (lib.gmc_bvh_set_build_path, lib.gmc_bvh_set_eval_path):
         knob(1)
         knob(0)
+    lib.gmc_bvh_set_traversal_groups(2, 3)
+    lib.gmc_bvh_set_traversal_groups(0, 0)
 
 
 def test_python_boundary_errors():
