@@ -2697,7 +2697,9 @@ static int bvh_build_t(const T* mixture, const T* xes, char* bvh, const gmc_shap
 // the resident workgroups in one go (measured on one mixture of 16384 Gaussians, groups -> best choice and time:
 // 391 -> 1, 43 us; 782 -> 2, 39 us; 1563 -> 4, 46 us against 63 us with 2; 3125 ... 25000 -> 4).  A backward pass
 // reads the candidate lists: small workgroups balance better over the compute units until the launch has many times
-// more groups than resident workgroups (1563 -> 1, 77 us against 85 us with 4; 3125 -> 2; 6250 -> 3; 25000 -> 4).  The
+// more groups than resident workgroups (1563 -> 1, 77 us against 85 us with 4; 3125 -> 2; 6250 -> 3; 25000 -> 4).  (Four
+// groups spread over exactly one round of resident workgroups are 3-6 % ahead at 1563 groups when the same backward
+// pass is repeated on one tree, and not ahead in a step that builds, traverses forward and backward: not taken.)  The
 // lists of many small trees are short and the fixed work of a workgroup weighs more: their backward launches take the
 // forward rule (64 trees of 512 leaves, 4096 groups: 72 us with 4 against 79 with 3 and 98 with 1; 256 trees of 200
 // leaves, 3328 groups: 44 us with 4, 46 with 2, 52 with 1).
