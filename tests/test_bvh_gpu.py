@@ -290,6 +290,22 @@ def test_large_trees_checked_on_the_host():
         assert err <= 3 * TOL[dtype], f"case {k}: culled forward sum off by {err:.3g} of the terms' magnitudes"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_groups_per_traversal_workgroup_do_not_change_the_sums(dtype):
+    """A workgroup of the traversal serves one to four 64-point groups (chosen by the size of the launch; a launch that
+    would leave resident workgroup slots empty is spread over all of them): every choice, forced through the test knob,
+    gives the masked sums -- forward with a descent, backward on the kept lists, ragged last groups included."""
+    lib = _native.lib()
+    for k, (B, L, M, N, D) in enumerate(((3, 2, 300, 1000, 3), (1, 1, 2000, 9000, 2), (5, 1, 150, 70, 3))):
+        mix, xes, gout = _case(B, L, M, N, D, seed=9100 + k, cov_radius=0.2)
+        for fwd_groups, bwd_groups in ((1, 4), (2, 3), (3, 2), (4, 1)):
+            lib.gmc_bvh_set_traversal_groups(fwd_groups, bwd_groups)
+            try:
+                _check_culled(mix, xes, gout, dtype, "tight", tag=f"case {k}, {fwd_groups} / {bwd_groups} groups per workgroup")
+            finally:
+                lib.gmc_bvh_set_traversal_groups(0, 0)
+
+
 def test_mixture_beyond_the_reference_node_index_range():
     """The reference stores node indices in 16 bits (lbvh/bvh.h:16-24: at most 32768 components per mixture); here
     they are 32-bit.  One mixture of 70000 components: every component is exactly one leaf, every parent box is the
